@@ -1,0 +1,93 @@
+/* paperkiln_amd -- C ABI of the MI355X (gfx950) attention hot path.
+ *
+ * Plain pointers and sizes only; every pointer is DEVICE memory unless it is
+ * named host_*. A call enqueues work on `stream` (a hipStream_t passed as
+ * void*; NULL = the default stream) and returns without synchronising; work
+ * on one stream is ordered. Every entry returns PK_OK or an error code and
+ * leaves a message for pk_last_error() (thread-local).
+ *
+ * The reference (paperkiln, C++ namespace microtorch) has no FFI registry:
+ * its seam is a set of C++ free functions that return "handled?" plus the tape
+ * ops themselves. Each entry below names the reference function it stands
+ * behind (paths relative to the paperkiln tree).
+ */
+#ifndef PAPERKILN_AMD_H
+#define PAPERKILN_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+    PK_OK = 0,
+    PK_ERR_SHAPE = 1,       /* the reference's "shape mismatch" throws, src/ops.cpp:866-870 */
+    PK_ERR_ARGUMENT = 2,    /* bad flag / null pointer / unsupported dtype */
+    PK_ERR_WORKSPACE = 3,   /* workspace too small */
+    PK_ERR_HIP = 4,         /* a HIP runtime call failed (cuda_check's role, src/cuda_ops.cu:34-38) */
+    PK_ERR_OOM = 5
+};
+
+enum { PK_F32 = 0, PK_BF16 = 1 };
+
+/* A [B, T, H, dk] tensor view: element strides for batch, token and head; the
+ * head_dim axis is contiguous. The reference's activation layout, a row-major
+ * [B*T, H*dk] Matrix whose heads are column slices (src/llama.cpp:48-50,
+ * src/nn.cpp:146-148), is {stride_b = T*H*dk, stride_t = H*dk, stride_h = dk};
+ * a fused [N, 3d] qkv projection is read in place with stride_t = 3*H*dk. */
+typedef struct pk_tensor4 {
+    void* ptr;
+    int64_t stride_b, stride_t, stride_h;
+} pk_tensor4;
+
+typedef struct pk_attn_shape {
+    int32_t B;          /* sequences; the reference's rows / seq_len blocks (src/ops.cpp:869-879) */
+    int32_t T;          /* tokens per sequence (seq_len) */
+    int32_t Hq, Hkv;    /* query heads, KV heads; Hq % Hkv == 0; query head h reads KV head h/(Hq/Hkv) */
+    int32_t dk;         /* head_dim */
+    int32_t causal;     /* fused_attention's `causal` flag */
+    int32_t window;     /* 0 = no band (fused_attention); >=1 = swa_attention's window (causal only) */
+    int32_t sinks;      /* swa_attention's always-visible leading keys */
+    float scale;        /* the op's `scale` argument (1/sqrt(dk) at every reference call site) */
+    int32_t dtype;      /* PK_F32 | PK_BF16: element type of q, k, v, o, dO */
+    int32_t grad_dtype; /* PK_F32 | PK_BF16: element type of dq, dk, dv */
+} pk_attn_shape;
+
+const char* pk_last_error(void);
+
+/* Library / device bring-up. Returns the gfx architecture name through
+ * arch[0..arch_len) when non-NULL. Fails loudly when no gfx950 device is
+ * visible: there is no CPU path behind this ABI.
+ * Stands where device::set(Device::CUDA) / cuda_compiled() do (src/device.cpp:32-46). */
+int pk_init(int device, char* arch, size_t arch_len);
+
+/* Forward of ops::fused_attention (src/ops.cpp:863-902) and, with window>=1,
+ * ops::swa_attention (src/ops.cpp:948-995), for all B*Hq heads in one launch.
+ * Writes O and the per-row logsumexp lse[B,Hq,T] (fp32, natural log of the
+ * sum of exp(scale*s_ij) over the visible set) and nothing else: the [T,T]
+ * weight matrix the reference keeps for its closure (src/ops.cpp:876,902) is
+ * never materialised. */
+int pk_attn_fwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k,
+                const pk_tensor4* v, const pk_tensor4* o, float* lse, void* stream);
+
+/* Bytes of scratch pk_attn_bwd needs for this shape (row sums D_i and, for
+ * GQA / bf16 gradients, nothing more). */
+size_t pk_attn_bwd_workspace_bytes(const pk_attn_shape* s);
+
+/* Backward closure of the same node (src/ops.cpp:902-933, 997-1026),
+ * recomputed from Q, K and LSE: dV = P^T dO, dP = dO V^T,
+ * dS = scale * P .* (dP - rowsum(dO .* O)), dQ = dS K, dK = dS^T Q.
+ * dK/dV are summed over the Hq/Hkv query heads of each KV head, which is what
+ * Variable::accumulate does when one K/V Variable parents several head nodes
+ * (src/autograd.cpp:16-24). Outputs are overwritten (not accumulated). */
+int pk_attn_bwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k,
+                const pk_tensor4* v, const pk_tensor4* o, const float* lse,
+                const pk_tensor4* d_o, const pk_tensor4* dq, const pk_tensor4* dk,
+                const pk_tensor4* dv, void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PAPERKILN_AMD_H */

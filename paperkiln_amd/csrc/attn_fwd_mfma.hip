@@ -1,0 +1,269 @@
+// bf16 flash-attention forward for gfx950: O and per-row logsumexp only.
+// Replaces the forward half of the reference's per-head
+// ops::fused_attention / ops::swa_attention (paperkiln src/ops.cpp:863-902,
+// 948-995), which materialise a [T,T] fp32 weight matrix per head.
+//
+// One workgroup = 4 wavefronts = one (batch, head, 128*NQ-query block). Each
+// wavefront owns NQ blocks of 32 queries and walks the visible key tiles
+// (64 keys per step). The work is phrased TRANSPOSED so that every softmax
+// row lives in one lane pair:
+//   S^T[key, query] = K . Q^T      A = K tile from LDS (ds_read_b128),
+//                                  B = Q, held in registers for the whole loop
+//   C layout => lane c holds query c: row max / row sum are in-lane loops plus
+//   one v_permlane32_swap with lane c^32.
+//   O^T[d, query]  += V^T . P^T    B = exp2(S^T) straight from the C registers
+//                                  (no LDS round trip), A = V^T fetched from
+//                                  the row-major V tile with transposing LDS
+//                                  reads (ds_read_b64_tr_b16).
+// Softmax runs in base 2 with the scale folded into one FMA per element:
+// p = exp2(s*c - m*c), c = scale*log2(e). Fully masked 32x64 blocks are
+// skipped per wavefront, fully masked key tiles are never loaded.
+#include "mfma_common.h"
+#include "pk_internal.h"
+
+namespace pk {
+namespace {
+
+constexpr int BN = 64;  // keys per step
+
+template <int D>
+struct FwdCfg {
+    static constexpr int KS = D + 8;    // K tile row pitch: 4 banks past a multiple of 64 -> b128 row reads conflict-free
+    static constexpr int VS = D + 32;   // V tile row pitch: 16 banks past -> the 4-row transposing reads conflict-free
+    static constexpr int NCH = D / 8;   // 16-byte chunks per row
+    static constexpr int CPT = BN * NCH / 256;  // chunks per thread per tile
+};
+
+template <int D>
+__device__ inline void load_kv_regs(const AttnArgs& a, int64_t kb, int64_t vb, int n0, u32x4* kr,
+                                    u32x4* vr) {
+    using C = FwdCfg<D>;
+#pragma unroll
+    for (int i = 0; i < C::CPT; ++i) {
+        const int c = threadIdx.x + 256 * i;
+        const int row = c / C::NCH, ch = c % C::NCH;
+        const int t = n0 + row;
+        u32x4 z = {0, 0, 0, 0};
+        kr[i] = z;
+        vr[i] = z;
+        if (t < a.T) {
+            kr[i] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.k) + kb + t * a.k_st + ch * 8);
+            vr[i] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.v) + vb + t * a.v_st + ch * 8);
+        }
+    }
+}
+
+template <int D>
+__device__ inline void store_kv_lds(uint16_t* Ks, uint16_t* Vs, const u32x4* kr, const u32x4* vr) {
+    using C = FwdCfg<D>;
+#pragma unroll
+    for (int i = 0; i < C::CPT; ++i) {
+        const int c = threadIdx.x + 256 * i;
+        const int row = c / C::NCH, ch = c % C::NCH;
+        *reinterpret_cast<u32x4*>(Ks + row * C::KS + ch * 8) = kr[i];
+        *reinterpret_cast<u32x4*>(Vs + row * C::VS + ch * 8) = vr[i];
+    }
+}
+
+template <int D, int NQ>
+__global__ __launch_bounds__(256) void mfma_fwd(AttnArgs a) {
+    using C = FwdCfg<D>;
+    constexpr int BM = 128 * NQ;
+    constexpr int KK = D / 16;  // k-chunks of the QK^T contraction
+    constexpr int DB = D / 32;  // 32-row blocks of O^T
+    __shared__ __attribute__((aligned(16))) uint16_t Ks[BN * C::KS];
+    __shared__ __attribute__((aligned(16))) uint16_t Vs[BN * C::VS];
+
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int g = lane >> 5, c32 = lane & 31;
+    // Heaviest query blocks (most visible keys) are dispatched first.
+    const int qblk = gridDim.x - 1 - blockIdx.x;
+    const int q0 = qblk * BM, h = blockIdx.y, b = blockIdx.z;
+    const int hk = h / (a.Hq / a.Hkv);
+    const int64_t qb_off = b * a.q_sb + h * a.q_sh;
+    const int64_t kb = b * a.k_sb + hk * a.k_sh, vb = b * a.v_sb + hk * a.v_sh;
+    const float cexp = a.scale * 1.4426950408889634f;
+
+    // Q as the B operand: lane c holds query c, d = 16kk + 8g .. +7.
+    bf16x8 qreg[NQ][KK];
+#pragma unroll
+    for (int qb = 0; qb < NQ; ++qb) {
+        const int row = q0 + (w * NQ + qb) * 32 + c32;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            u32x4 z = {0, 0, 0, 0};
+            if (row < a.T)
+                z = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.q) + qb_off +
+                                                    row * a.q_st + kk * 16 + g * 8);
+            qreg[qb][kk] = *reinterpret_cast<bf16x8*>(&z);
+        }
+    }
+
+    f32x16 acc_o[NQ][DB];
+    float m[NQ], l[NQ];
+#pragma unroll
+    for (int qb = 0; qb < NQ; ++qb) {
+        m[qb] = -1e30f;  // the reference's running-max seed, src/ops.cpp:881
+        l[qb] = 0.0f;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc_o[qb][db][r] = 0.0f;
+    }
+
+    // Key tiles this query block can see: the sink tiles [0, ns) and the
+    // band / causal tiles [lo, hi] (src/ops.cpp:960-965 in tile units).
+    const int qmax = min(q0 + BM, a.T) - 1;
+    const int hi = (a.causal ? qmax : a.T - 1) / BN;
+    const int lo = a.window > 0 ? max(0, q0 + 1 - a.window) / BN : 0;
+    const int ns = a.window > 0 ? min((a.sinks + BN - 1) / BN, lo) : 0;
+    int t = ns > 0 ? 0 : lo;
+
+    u32x4 kr[C::CPT], vr[C::CPT];
+    load_kv_regs<D>(a, kb, vb, t * BN, kr, vr);
+    store_kv_lds<D>(Ks, Vs, kr, vr);
+    __syncthreads();
+
+    while (t <= hi) {
+        const int n0 = t * BN;
+        const int tn = (t + 1 == ns) ? lo : t + 1;
+        if (tn <= hi) load_kv_regs<D>(a, kb, vb, tn * BN, kr, vr);  // in flight during the math
+
+#pragma unroll
+        for (int qb = 0; qb < NQ; ++qb) {
+            const int qlo = q0 + (w * NQ + qb) * 32, qhi = qlo + 31;
+            // wavefront-uniform: nothing of this 32x64 block is visible
+            if (qlo >= a.T) continue;
+            if (a.causal && n0 > qhi) continue;
+            if (a.window > 0 && n0 + BN - 1 + a.window <= qlo && n0 >= a.sinks) continue;
+
+            f32x16 s[2];
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[nb][r] = 0.0f;
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) {
+                    bf16x8 kf = lds_read8(Ks + (nb * 32 + c32) * C::KS + kk * 16 + g * 8);
+                    s[nb] = mfma32(kf, qreg[qb][kk], s[nb]);
+                }
+            }
+            const bool full = (n0 + BN - 1 < a.T) && (!a.causal || n0 + BN - 1 <= qlo) &&
+                              (a.window == 0 || n0 + a.window > qhi || n0 + BN - 1 < a.sinks);
+            if (!full) {
+                const int qi = qlo + c32;
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int kj = n0 + nb * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
+                        if (!pk_visible(qi, kj, a.T, a.causal, a.window, a.sinks)) s[nb][r] = -INFINITY;
+                    }
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[nb][r]);
+            mx = xhalf_max(mx);
+            const float mn = fmaxf(m[qb], mx);
+            const float alpha = __builtin_amdgcn_exp2f((m[qb] - mn) * cexp);
+            const float mc = mn * cexp;
+            float psum = 0.0f;
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float p = __builtin_amdgcn_exp2f(fmaf(s[nb][r], cexp, -mc));
+                    s[nb][r] = p;
+                    psum += p;
+                }
+            l[qb] = l[qb] * alpha + psum;  // per-lane partial; the two halves meet in the epilogue
+            m[qb] = mn;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc_o[qb][db][r] *= alpha;
+
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) {
+                const bf16x8 p0 = c_to_operand<0>(s[nb]);
+                const bf16x8 p1 = c_to_operand<1>(s[nb]);
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    bf16x8 v0 = lds_read_tr_operand(Vs, C::VS, nb * 32, db * 32, lane);
+                    acc_o[qb][db] = mfma32(v0, p0, acc_o[qb][db]);
+                    bf16x8 v1 = lds_read_tr_operand(Vs, C::VS, nb * 32 + 16, db * 32, lane);
+                    acc_o[qb][db] = mfma32(v1, p1, acc_o[qb][db]);
+                }
+            }
+        }
+
+        __syncthreads();  // every wavefront is done reading this tile
+        if (tn <= hi) store_kv_lds<D>(Ks, Vs, kr, vr);
+        __syncthreads();
+        t = tn;
+    }
+
+    // Epilogue: O = acc / l, LSE = m*scale + ln(l) (natural log, scaled units).
+#pragma unroll
+    for (int qb = 0; qb < NQ; ++qb) {
+        const int qi = q0 + (w * NQ + qb) * 32 + c32;
+        const float lt = xhalf_sum(l[qb]);
+        if (qi >= a.T) continue;
+        const float inv = 1.0f / lt;
+        uint16_t* orow = static_cast<uint16_t*>(a.o) + b * a.o_sb + h * a.o_sh + qi * a.o_st;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                u32x2 pk2 = {pack_bf16(acc_o[qb][db][qd * 4 + 0] * inv, acc_o[qb][db][qd * 4 + 1] * inv),
+                             pack_bf16(acc_o[qb][db][qd * 4 + 2] * inv, acc_o[qb][db][qd * 4 + 3] * inv)};
+                *reinterpret_cast<u32x2*>(orow + db * 32 + qd * 8 + g * 4) = pk2;
+            }
+        if (g == 0)
+            a.lse[(static_cast<int64_t>(b) * a.Hq + h) * a.T + qi] = m[qb] * a.scale + logf(lt);
+    }
+}
+
+template <int D, int NQ>
+int launch(const AttnArgs& a, hipStream_t st) {
+    constexpr int BM = 128 * NQ;
+    dim3 grid((a.T + BM - 1) / BM, a.Hq, a.B);
+    hipLaunchKernelGGL((mfma_fwd<D, NQ>), grid, dim3(256), 0, st, a);
+    PK_HIP(hipGetLastError());
+    return PK_OK;
+}
+
+bool aligned16(const void* p, int64_t sb, int64_t st, int64_t sh) {
+    return (reinterpret_cast<uintptr_t>(p) % 16 == 0) && sb % 8 == 0 && st % 8 == 0 && sh % 8 == 0;
+}
+
+}  // namespace
+
+// The MFMA kernels take bf16 storage, head_dim 64 or 128, a positive scale
+// (the running max is tracked on raw scores) and 16-byte-aligned rows.
+bool mfma_supported(const AttnArgs& a) {
+    if (a.dk_dim != 64 && a.dk_dim != 128) return false;
+    if (!(a.scale > 0.0f)) return false;
+    if (!aligned16(a.q, a.q_sb, a.q_st, a.q_sh) || !aligned16(a.k, a.k_sb, a.k_st, a.k_sh) ||
+        !aligned16(a.v, a.v_sb, a.v_st, a.v_sh) || !aligned16(a.o, a.o_sb, a.o_st, a.o_sh))
+        return false;
+    if (a.d_o) {
+        if (!aligned16(a.d_o, a.do_sb, a.do_st, a.do_sh)) return false;
+        if (!aligned16(a.dq, a.dq_sb, a.dq_st, a.dq_sh) || !aligned16(a.dk, a.dk_sb, a.dk_st, a.dk_sh) ||
+            !aligned16(a.dv, a.dv_sb, a.dv_st, a.dv_sh))
+            return false;
+    }
+    return true;
+}
+
+int launch_mfma_fwd(const AttnArgs& a, hipStream_t st) {
+    // Two 32-query blocks per wavefront halve the LDS traffic per MFMA; short
+    // sequences keep one so that the grid still covers the chip.
+    const bool big = static_cast<int64_t>(a.T) * a.Hq * a.B >= 256 * 256 * 2;
+    if (a.dk_dim == 128) return big ? launch<128, 2>(a, st) : launch<128, 1>(a, st);
+    return big ? launch<64, 2>(a, st) : launch<64, 1>(a, st);
+}
+
+}  // namespace pk

@@ -1,0 +1,128 @@
+// The C ABI of libpaperkiln_amd.so: argument checking, dispatch between the
+// MFMA and the generic kernels, and the thread-local error string. There is
+// no CPU path behind any entry: without a gfx950 device every call fails.
+#include <cstdio>
+#include <cstring>
+
+#include "pk_internal.h"
+
+namespace pk {
+
+namespace {
+thread_local std::string g_err;
+}
+
+void set_error(const std::string& msg) { g_err = msg; }
+
+int fail(int code, const std::string& msg) {
+    g_err = msg;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    g_err = std::string("HIP error: ") + hipGetErrorString(e) + " in " + what;
+    return PK_ERR_HIP;
+}
+
+namespace {
+
+int check_shape(const pk_attn_shape* s, const char* who) {
+    if (!s) return fail(PK_ERR_ARGUMENT, std::string(who) + ": null shape");
+    if (s->B <= 0 || s->T <= 0 || s->Hq <= 0 || s->Hkv <= 0 || s->dk <= 0)
+        return fail(PK_ERR_SHAPE, std::string(who) + ": shape mismatch (non-positive dimension)");
+    if (s->Hq % s->Hkv != 0)
+        return fail(PK_ERR_SHAPE, std::string(who) + ": shape mismatch (Hq not a multiple of Hkv)");
+    if (s->dk > 256) return fail(PK_ERR_SHAPE, std::string(who) + ": head_dim > 256 not supported");
+    if (s->window < 0 || s->sinks < 0)
+        return fail(PK_ERR_ARGUMENT, std::string(who) + ": window and sinks must be >= 0");
+    if (s->window > 0 && !s->causal)
+        return fail(PK_ERR_ARGUMENT, std::string(who) + ": a window requires causal (swa_attention is causal)");
+    if ((s->dtype != PK_F32 && s->dtype != PK_BF16) || (s->grad_dtype != PK_F32 && s->grad_dtype != PK_BF16))
+        return fail(PK_ERR_ARGUMENT, std::string(who) + ": dtype must be PK_F32 or PK_BF16");
+    return PK_OK;
+}
+
+bool bad(const pk_tensor4* t) { return !t || !t->ptr; }
+
+void fill_common(AttnArgs& a, const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k,
+                 const pk_tensor4* v, const pk_tensor4* o) {
+    std::memset(&a, 0, sizeof a);
+    a.q = q->ptr; a.q_sb = q->stride_b; a.q_st = q->stride_t; a.q_sh = q->stride_h;
+    a.k = k->ptr; a.k_sb = k->stride_b; a.k_st = k->stride_t; a.k_sh = k->stride_h;
+    a.v = v->ptr; a.v_sb = v->stride_b; a.v_st = v->stride_t; a.v_sh = v->stride_h;
+    a.o = o->ptr; a.o_sb = o->stride_b; a.o_st = o->stride_t; a.o_sh = o->stride_h;
+    a.B = s->B; a.T = s->T; a.Hq = s->Hq; a.Hkv = s->Hkv; a.dk_dim = s->dk;
+    a.causal = s->causal != 0; a.window = s->window; a.sinks = s->sinks;
+    a.scale = s->scale;
+    a.grad_f32 = s->grad_dtype == PK_F32;
+}
+
+}  // namespace
+}  // namespace pk
+
+using namespace pk;
+
+extern "C" {
+
+const char* pk_last_error(void) { return g_err.c_str(); }
+
+int pk_init(int device, char* arch, size_t arch_len) {
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0)
+        return fail(PK_ERR_HIP, "pk_init: no HIP device visible (this library has no CPU path)");
+    if (device < 0 || device >= n) return fail(PK_ERR_ARGUMENT, "pk_init: device index out of range");
+    PK_HIP(hipSetDevice(device));
+    hipDeviceProp_t p;
+    PK_HIP(hipGetDeviceProperties(&p, device));
+    if (arch && arch_len) {
+        std::snprintf(arch, arch_len, "%s", p.gcnArchName);
+    }
+    if (std::strncmp(p.gcnArchName, "gfx950", 6) != 0)
+        return fail(PK_ERR_HIP, std::string("pk_init: kernels are built for gfx950 only, found ") + p.gcnArchName);
+    return PK_OK;
+}
+
+int pk_attn_fwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k, const pk_tensor4* v,
+                const pk_tensor4* o, float* lse, void* stream) {
+    if (int rc = check_shape(s, "pk_attn_fwd")) return rc;
+    if (bad(q) || bad(k) || bad(v) || bad(o) || !lse)
+        return fail(PK_ERR_ARGUMENT, "pk_attn_fwd: null tensor");
+    AttnArgs a;
+    fill_common(a, s, q, k, v, o);
+    a.lse = lse;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (s->dtype == PK_BF16 && mfma_supported(a)) return launch_mfma_fwd(a, st);
+    return launch_generic_fwd(a, s->dtype == PK_BF16, st);
+}
+
+size_t pk_attn_bwd_workspace_bytes(const pk_attn_shape* s) {
+    if (check_shape(s, "pk_attn_bwd_workspace_bytes")) return 0;
+    return sizeof(float) * static_cast<size_t>(s->B) * s->Hq * s->T;
+}
+
+int pk_attn_bwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k, const pk_tensor4* v,
+                const pk_tensor4* o, const float* lse, const pk_tensor4* d_o, const pk_tensor4* dq,
+                const pk_tensor4* dk, const pk_tensor4* dv, void* workspace, size_t workspace_bytes,
+                void* stream) {
+    if (int rc = check_shape(s, "pk_attn_bwd")) return rc;
+    if (bad(q) || bad(k) || bad(v) || bad(o) || !lse || bad(d_o) || bad(dq) || bad(dk) || bad(dv))
+        return fail(PK_ERR_ARGUMENT, "pk_attn_bwd: null tensor");
+    if (!workspace || workspace_bytes < pk_attn_bwd_workspace_bytes(s))
+        return fail(PK_ERR_WORKSPACE, "pk_attn_bwd: workspace smaller than pk_attn_bwd_workspace_bytes()");
+    if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+        return fail(PK_ERR_ARGUMENT, "pk_attn_bwd: workspace must be 16-byte aligned");
+    AttnArgs a;
+    fill_common(a, s, q, k, v, o);
+    a.lse = const_cast<float*>(lse);
+    a.d_o = d_o->ptr; a.do_sb = d_o->stride_b; a.do_st = d_o->stride_t; a.do_sh = d_o->stride_h;
+    a.dq = dq->ptr; a.dq_sb = dq->stride_b; a.dq_st = dq->stride_t; a.dq_sh = dq->stride_h;
+    a.dk = dk->ptr; a.dk_sb = dk->stride_b; a.dk_st = dk->stride_t; a.dk_sh = dk->stride_h;
+    a.dv = dv->ptr; a.dv_sb = dv->stride_b; a.dv_st = dv->stride_t; a.dv_sh = dv->stride_h;
+    a.delta = static_cast<float*>(workspace);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (s->dtype == PK_BF16 && mfma_supported(a)) return launch_mfma_bwd(a, st);
+    return launch_generic_bwd(a, s->dtype == PK_BF16, st);
+}
+
+}  // extern "C"

@@ -1,0 +1,89 @@
+// gfx950 (CDNA4) building blocks shared by the bf16 MFMA attention kernels.
+//
+// v_mfma_f32_32x32x16_bf16 operand layout (64-lane wavefront, g = lane / 32,
+// c = lane % 32), verified on hardware:
+//   A (32 x 16): lane holds row c,    k = 8g .. 8g+7   (8 bf16, 4 VGPRs)
+//   B (16 x 32): lane holds column c, k = 8g .. 8g+7
+//   C (32 x 32): lane holds column c, element r (0..15) is row (r/4)*8 + 4g + r%4
+// The k index is a summation index, so A and B may use ANY common permutation
+// of it. The kernels exploit that: a C tile whose rows are the contraction
+// index of the next GEMM is fed back as a B operand directly from registers,
+// elements 8h..8h+7 (h = 0, 1) forming one k-chunk, and the other operand is
+// fetched with the matching row permutation {4g..4g+3} u {8+4g..8+4g+3}.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace pk {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define PK_LDS __attribute__((address_space(3)))
+
+__device__ inline f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// Exchange a value with lane ^ 32 and combine (v_permlane32_swap: lanes 0..31
+// of the second operand trade places with lanes 32..63 of the first).
+__device__ inline float xhalf_max(float x) {
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ inline float xhalf_sum(float x) {
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// Two fp32 -> packed bf16 (v_cvt_pk_bf16_f32, round to nearest even).
+__device__ inline uint32_t pack_bf16(float lo, float hi) {
+    f32x2 f = {lo, hi};
+    bf16x2 h = __builtin_convertvector(f, bf16x2);
+    return *reinterpret_cast<uint32_t*>(&h);
+}
+
+// Elements 8h .. 8h+7 of a C tile as one bf16 k-chunk (a B or A operand).
+template <int H>
+__device__ inline bf16x8 c_to_operand(const f32x16& c) {
+    u32x4 u = {pack_bf16(c[8 * H + 0], c[8 * H + 1]), pack_bf16(c[8 * H + 2], c[8 * H + 3]),
+               pack_bf16(c[8 * H + 4], c[8 * H + 5]), pack_bf16(c[8 * H + 6], c[8 * H + 7])};
+    return *reinterpret_cast<bf16x8*>(&u);
+}
+
+// 16-byte LDS read of 8 consecutive bf16 (ds_read_b128).
+__device__ inline bf16x8 lds_read8(const uint16_t* p) {
+    return *reinterpret_cast<const bf16x8*>(p);
+}
+
+// Transposing LDS read (ds_read_b64_tr_b16). Within each group of 16 lanes,
+// lane 4a+c receives element c of the four 8-byte rows addressed by lanes
+// a, a+4, a+8, a+12 (verified on hardware). With lane j of a group pointing
+// at  tile[row0 + j/4][col0 + 4*(j%4)]  lane i of the group ends up holding
+// tile[row0 .. row0+3][col0 + i]: four consecutive ROWS of its own column.
+__device__ inline s16x4 lds_read_tr4(const uint16_t* p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((PK_LDS s16x4*)(p));
+}
+
+// Operand whose k-chunk is rows {row0+4g..+3} u {row0+8+4g..+3} of a row-major
+// LDS tile, for the 32 columns col0 .. col0+31 (one per lane c). `stride` is
+// the tile's row pitch in elements. Matches c_to_operand's row permutation.
+__device__ inline bf16x8 lds_read_tr_operand(const uint16_t* tile, int stride, int row0, int col0,
+                                             int lane) {
+    const int g = lane >> 5, u = (lane >> 4) & 1, j = lane & 15;
+    const uint16_t* p = tile + (row0 + 4 * g + (j >> 2)) * stride + col0 + 16 * u + 4 * (j & 3);
+    s16x4 lo = lds_read_tr4(p);
+    s16x4 hi = lds_read_tr4(p + 8 * stride);
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return *reinterpret_cast<bf16x8*>(&v);
+}
+
+}  // namespace pk

@@ -1,0 +1,195 @@
+"""GPU parity tests proper: the HIP path (through the C ABI) against the CPU
+oracle and the committed reference vectors. Run with -m gpu on an MI355X.
+
+Bars (BASELINE.json): fp32 path max-abs 1e-5 on O/LSE/dQ/dK/dV; bf16 path
+max-abs 2e-2 on O/dQ/dK/dV and 1e-3 on LSE, against the fp32 CPU arithmetic run
+on the same bf16-rounded inputs.
+"""
+import numpy as np
+import pytest
+import torch
+
+from paperkiln_amd import ops, synth
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-5
+BF16_TOL, BF16_LSE_TOL = 2e-2, 1e-3
+
+
+def maxabs(a, b):
+    return float(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64)).max())
+
+
+def dev(x, dtype):
+    return torch.from_numpy(np.ascontiguousarray(x)).to("cuda").to(dtype)
+
+
+def host(x):
+    return x.detach().float().cpu().numpy()
+
+
+def run_gpu(q, k, v, d_o, scale, causal, window, sinks, dtype, grad_dtype=None):
+    tq, tk, tv, tg = (dev(x, dtype) for x in (q, k, v, d_o))
+    o, lse = ops.attn_fwd(tq, tk, tv, scale, causal, window, sinks)
+    dq, dk, dv = ops.attn_bwd(tq, tk, tv, o, lse, tg, scale, causal, window, sinks, grad_dtype=grad_dtype)
+    torch.cuda.synchronize()
+    return host(o), host(lse), host(dq), host(dk), host(dv)
+
+
+def report(tag, got, want):
+    errs = [maxabs(a, b) for a, b in zip(got, want)]
+    print(f"\n  {tag}: O {errs[0]:.2e} LSE {errs[1]:.2e} dQ {errs[2]:.2e} dK {errs[3]:.2e} dV {errs[4]:.2e}", flush=True)
+    return errs
+
+
+def test_fp32_against_reference_vectors(golden):
+    """Every committed vector from the compiled reference, fp32 path, 1e-5."""
+    g = golden
+    got = run_gpu(g.q, g.k, g.v, g.d_o, g.scale, g.causal, g.window, g.sinks, torch.float32)
+    errs = report(g.name, got, (g.o, g.lse, g.dq, g.dk, g.dv))
+    assert max(errs) < FP32_TOL
+
+
+def test_bf16_against_reference_vectors(golden):
+    """Vectors whose inputs are bf16-exact, bf16 path (MFMA kernels at d=64/128), fp32 gradients out."""
+    g = golden
+    if not g.bf16:
+        pytest.skip("inputs of this vector are not bf16-representable")
+    got = run_gpu(g.q, g.k, g.v, g.d_o, g.scale, g.causal, g.window, g.sinks, torch.bfloat16, torch.float32)
+    errs = report(g.name, got, (g.o, g.lse, g.dq, g.dk, g.dv))
+    assert max(errs[0], errs[2], errs[3], errs[4]) < BF16_TOL and errs[1] < BF16_LSE_TOL
+
+
+def make(B, T, Hq, Hkv, dk, std, seed, rope_theta=None):
+    q = synth.randn(seed, (B, T, Hq, dk), std)
+    k = synth.randn(seed + 1, (B, T, Hkv, dk), std)
+    v = synth.randn(seed + 2, (B, T, Hkv, dk), std)
+    d_o = synth.randn(seed + 3, (B, T, Hq, dk), 1.0)
+    if rope_theta:
+        q, k = synth.rope_interleaved(q, rope_theta), synth.rope_interleaved(k, rope_theta)
+    return tuple(synth.bf16_round(x) for x in (q, k, v, d_o))
+
+
+# (name, B, T, Hq, Hkv, dk, std, causal, window, sinks, rope theta): the BASELINE workloads at sizes the
+# single-threaded oracle finishes in seconds, plus ragged / edge shapes.
+BF16_CASES = [
+    ("cfg2_tinystories_B2_H2_T512_d64", 2, 512, 2, 2, 64, 1.0, True, 0, 0, 1e4),
+    ("cfg3_qwen_gqa_Hq14_Hkv2_T384_d64", 1, 384, 14, 2, 64, 1.0, True, 0, 0, 1e6),
+    ("cfg4_causal_H2_T1024_d128", 1, 1024, 2, 2, 128, 0.5, True, 0, 0, None),
+    ("cfg4_window256_sinks4_H2_T1024_d128", 1, 1024, 2, 2, 128, 0.5, True, 256, 4, None),
+    ("ragged_T333_d128_causal", 2, 333, 2, 1, 128, 1.0, True, 0, 0, None),
+    ("ragged_T77_d64_bidir", 2, 77, 2, 2, 64, 1.0, False, 0, 0, None),
+    ("window_smaller_than_tile_T500_w17_s70_d64", 1, 500, 2, 2, 64, 1.0, True, 17, 70, None),
+    ("T1_d64", 3, 1, 2, 2, 64, 1.0, True, 0, 0, None),
+    ("generic_bf16_d32_T100", 2, 100, 2, 1, 32, 1.0, True, 9, 2, None),
+]
+
+
+@pytest.mark.parametrize("case", BF16_CASES, ids=[c[0] for c in BF16_CASES])
+def test_bf16_against_oracle(oracle, case):
+    name, B, T, Hq, Hkv, dk, std, causal, window, sinks, theta = case
+    q, k, v, d_o = make(B, T, Hq, Hkv, dk, std, 500, theta)
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
+    want_o, want_lse = oracle.attn_fwd(q, k, v, scale, causal, window, sinks)
+    want = (want_o, want_lse) + oracle.attn_bwd(q, k, v, d_o, scale, causal, window, sinks)
+    got = run_gpu(q, k, v, d_o, scale, causal, window, sinks, torch.bfloat16, torch.float32)
+    errs = report(name + " (fp32 grads out)", got, want)
+    assert max(errs[0], errs[2], errs[3], errs[4]) < BF16_TOL and errs[1] < BF16_LSE_TOL
+    # bf16 gradient outputs: same accumulators, rounded once on the way out. The rounding alone is
+    # |x| * 2^-9, so the bar is checked on values the format can hold to 2e-2 (|x| < 8).
+    got16 = run_gpu(q, k, v, d_o, scale, causal, window, sinks, torch.bfloat16, torch.bfloat16)
+    for a, b, w in zip(got16[2:], got[2:], want[2:]):
+        assert maxabs(a, synth.bf16_round(b)) == 0.0  # exactly the fp32 result rounded to bf16
+        if np.abs(w).max() < 8.0:
+            assert maxabs(a, w) < BF16_TOL
+
+
+def test_fp32_path_on_bf16_shapes_agrees(oracle):
+    """The generic fp32 kernels at an MFMA-eligible shape: 1e-5."""
+    q, k, v, d_o = make(1, 200, 2, 1, 64, 1.0, 900)
+    scale = 0.125
+    want_o, want_lse = oracle.attn_fwd(q, k, v, scale, True, 40, 3)
+    want = (want_o, want_lse) + oracle.attn_bwd(q, k, v, d_o, scale, True, 40, 3)
+    errs = report("fp32 generic", run_gpu(q, k, v, d_o, scale, True, 40, 3, torch.float32), want)
+    assert max(errs) < FP32_TOL
+
+
+def test_strided_qkv_views():
+    """Heads read in place from a fused [N, 3d] projection (no repack)."""
+    B, T, H, dk = 2, 256, 4, 64
+    qkv = torch.from_numpy(synth.randn(7, (B, T, 3, H, dk))).cuda().bfloat16()
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+    o1, l1 = ops.attn_fwd(q, k, v, 0.125)
+    o2, l2 = ops.attn_fwd(q.contiguous(), k.contiguous(), v.contiguous(), 0.125)
+    assert torch.equal(o1, o2) and torch.equal(l1, l2)
+
+
+def test_reference_op_surface(oracle):
+    """ops.fused_attention / ops.swa_attention: per-head [rows, dk] matrices, seq_len stacking,
+    autograd through the O+LSE-only node, and the reference's error behaviour."""
+    T, dk = 96, 32
+    q, k, v = (torch.from_numpy(synth.randn(s, (2 * T, dk))).cuda().requires_grad_() for s in (1, 2, 3))
+    y = ops.fused_attention(q, k, v, 0.2, seq_len=T, causal=True)
+    (y * y).sum().mul(0.5).backward()
+    want_y, _, A = oracle.head_fwd(host(q), host(k), host(v), 0.2, T, True, 0, 0)
+    dq, dk_, dv = oracle.head_bwd(host(q), host(k), host(v), A, want_y, 0.2, T, True, 0, 0)
+    assert maxabs(host(y), want_y) < FP32_TOL
+    assert max(maxabs(host(q.grad), dq), maxabs(host(k.grad), dk_), maxabs(host(v.grad), dv)) < FP32_TOL
+    y2 = ops.swa_attention(q, k, v, 0.2, window=7, sinks=2, seq_len=T)
+    assert maxabs(host(y2), oracle.head_fwd(host(q), host(k), host(v), 0.2, T, True, 7, 2)[0]) < FP32_TOL
+    with pytest.raises(RuntimeError, match="window must be >= 1"):
+        ops.swa_attention(q, k, v, 0.2, window=0, sinks=0)
+    with pytest.raises(RuntimeError, match="rows not a multiple of seq_len"):
+        ops.fused_attention(q, k, v, 0.2, seq_len=7)
+    with pytest.raises(RuntimeError, match="shape mismatch"):
+        ops.fused_attention(q, k[:, :16], v, 0.2)
+
+
+def test_full_size_properties_cfg4(oracle):
+    """B=4, H=16, T=4096, d=128 bf16: properties that do not need the oracle at full size, plus
+    one (batch, head) unit against the oracle itself."""
+    B, T, H, dk = 4, 4096, 16, 128
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q = (torch.randn((B, T, H, dk), generator=g, device="cuda") * 0.5).bfloat16()
+    k = (torch.randn((B, T, H, dk), generator=g, device="cuda") * 0.5).bfloat16()
+    v = (torch.randn((B, T, H, dk), generator=g, device="cuda") * 0.5).bfloat16()
+    d_o = torch.randn((B, T, H, dk), generator=g, device="cuda").bfloat16()
+    o, lse = ops.attn_fwd(q, k, v, scale, True)
+    dq, dk_, dv = ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, grad_dtype=torch.float32)
+    # swa(window >= T, sinks = 0) == causal, bitwise (tests/test_swa.cpp:47-57)
+    o_w, lse_w = ops.attn_fwd(q, k, v, scale, True, window=T, sinks=0)
+    assert torch.equal(o, o_w) and torch.equal(lse, lse_w)
+    # batch / head isolation: a unit computed alone equals the unit inside the batch, bitwise
+    o_1, lse_1 = ops.attn_fwd(q[2:3, :, 5:6], k[2:3, :, 5:6], v[2:3, :, 5:6], scale, True)
+    assert torch.equal(o_1, o[2:3, :, 5:6]) and torch.equal(lse_1, lse[2:3, 5:6])
+    # causality: changing the last 100 tokens leaves every earlier row untouched, bitwise
+    k2, v2 = k.clone(), v.clone()
+    k2[:, -100:] += 1.0
+    v2[:, -100:] -= 1.0
+    o_c, lse_c = ops.attn_fwd(q, k2, v2, scale, True)
+    assert torch.equal(o_c[:, :-100], o[:, :-100]) and torch.equal(lse_c[:, :, :-100], lse[:, :, :-100])
+    # sum_j dS_ij = 0  =>  with every key equal, dQ vanishes and dK sums to scale * sum_i 0 = 0 per column
+    kc = k[:, :1].expand_as(k).contiguous()
+    oc, lsec = ops.attn_fwd(q, kc, v, scale, True)
+    dqc, dkc, _ = ops.attn_bwd(q, kc, v, oc, lsec, d_o, scale, True, grad_dtype=torch.float32)
+    assert float(dqc.abs().max()) < 2e-2
+    # window = 256 + 4 sinks at full size: locality, bitwise (tests/test_swa.cpp:92-122)
+    ow, _ = ops.attn_fwd(q, k, v, scale, True, window=256, sinks=4)
+    v3 = v.clone()
+    v3[:, 1000:1200] += 3.0  # outside window u sinks of rows >= 1455
+    ow3, _ = ops.attn_fwd(q, k, v3, scale, True, window=256, sinks=4)
+    assert torch.equal(ow3[:, 1455:], ow[:, 1455:]) and not torch.equal(ow3[:, 1000:1455], ow[:, 1000:1455])
+    v3 = v.clone()
+    v3[:, 2] += 3.0  # a sink token: every later row moves
+    ow4, _ = ops.attn_fwd(q, k, v3, scale, True, window=256, sinks=4)
+    assert (ow4[:, 3000:] != ow[:, 3000:]).any(dim=-1).all()
+    # one (b, h) unit against the oracle at the full T
+    b, h = 1, 7
+    hq, hk, hv, hg = (host(x[b, :, h]) for x in (q, k, v, d_o))
+    want_y, want_lse, A = oracle.head_fwd(hq, hk, hv, scale, 0, True, 0, 0)
+    want = (want_y, want_lse) + oracle.head_bwd(hq, hk, hv, A, hg, scale, 0, True, 0, 0)
+    got = (host(o[b, :, h]), host(lse[b, h]), host(dq[b, :, h]), host(dk_[b, :, h]), host(dv[b, :, h]))
+    errs = report("cfg4 full size, unit (1,7)", got, want)
+    assert max(errs[0], errs[2], errs[3], errs[4]) < BF16_TOL and errs[1] < BF16_LSE_TOL
