@@ -1,0 +1,174 @@
+#!/usr/bin/env python3
+"""Headline benchmark: bf16 causal attention forward + recompute backward at
+B=4, H=16, T=4096, head_dim=128 on ONE MI355X, through the C ABI.
+
+A "step" is one forward (O + LSE) plus one backward (dQ, dK, dV) over one
+batch of synthetic inputs already resident in HBM. Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+Work model (same for every rate printed here): FLOPs = 14 * dk * pairs * B*Hq
+(forward 2 GEMMs = 4*dk*pairs, backward 5 GEMMs = 10*dk*pairs; masked tiles
+and recomputation earn nothing), pairs = T(T+1)/2 for causal. Bytes = one
+read of Q,K,V + one write of O,LSE (forward) + one read of Q,K,V,O,dO,LSE and
+one write of dQ,dK,dV (backward).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
+
+# HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs
+# (FETCH_SIZE, WRITE_SIZE) scaled by a copy kernel of known size; see
+# profiles/. None until measured for the current kernel.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def cpu_baseline(B, T, H, dk, scale, seconds_budget=30.0):
+    """The reference's CPU attention (ops.cpp path) on ONE (batch, head) unit of
+    the same workload, single thread, timed with a wall clock; the rate is
+    FLOPs-per-unit / time, so it compares with `value` directly."""
+    import numpy as np
+    from oracle.bindings import Oracle, load_reference
+    from paperkiln_amd import synth
+
+    q = synth.bf16_round(synth.randn(11, (T, dk), 0.5))
+    k = synth.bf16_round(synth.randn(12, (T, dk), 0.5))
+    v = synth.bf16_round(synth.randn(13, (T, dk), 0.5))
+    g = synth.bf16_round(synth.randn(14, (T, dk), 1.0))
+    flops_unit = 14.0 * dk * (T * (T + 1) // 2)
+    ref = load_reference()
+    t0 = time.perf_counter()
+    if ref is not None:
+        ref.fused_attention(q, k, v, scale, 0, True, dy=g)
+        kind = "reference"
+    else:
+        orc = Oracle()
+        _, _, A = orc.head_fwd(q, k, v, scale, 0, True, 0, 0)
+        orc.head_bwd(q, k, v, A, g, scale, 0, True, 0, 0)
+        kind = "port"
+    dt = time.perf_counter() - t0
+    cpu = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                cpu = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {"value": flops_unit / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": kind,
+            "sample": f"1 of {B * H} (batch, head) units of the same workload, fwd+bwd, {dt:.2f} s wall; "
+                      f"whole job would take ~{dt * B * H:.0f} s on one core",
+            "host_cpu": cpu, "host_nproc": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (one process, one MI355X); --gpus must be 1. "
+                 "Each (batch, KV-head group) is an independent unit, so N GPUs would each take B*Hkv/N of them.")
+
+    import numpy as np
+    import torch
+    from paperkiln_amd import _lib, ops, synth
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; paperkiln_amd has no CPU path")
+    _lib.check(_lib.lib().pk_init(0, None, 0))
+    dev = torch.device("cuda:0")
+
+    B, H, T, dk = 4, 16, 4096, 128
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
+    gen = torch.Generator(device=dev).manual_seed(4)
+    q = (torch.randn((B, T, H, dk), generator=gen, device=dev) * 0.5).bfloat16()
+    k = (torch.randn((B, T, H, dk), generator=gen, device=dev) * 0.5).bfloat16()
+    v = (torch.randn((B, T, H, dk), generator=gen, device=dev) * 0.5).bfloat16()
+    d_o = torch.randn((B, T, H, dk), generator=gen, device=dev).bfloat16()
+    # outputs and scratch are allocated once; the timed region allocates nothing but O/LSE views
+    dq, dkk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    ws = torch.empty(4 * B * H * T, dtype=torch.uint8, device=dev)
+    out = (dq, dkk, dv, ws)
+
+    pairs = synth.visible_pairs(T, True, 0, 0)
+    unit = dk * pairs * B * H
+    flops_step = 14.0 * unit
+    bytes_step = 12.0 * B * T * H * dk * 2 + 2.0 * B * H * T * 4
+    # algorithmic work per launch: forward = S and PV; dkdv = S, dP, dV, dK; dq = dQ only
+    # (its S and dP are recomputation and earn nothing); delta is a pure HBM pass.
+    alg_flops = {"fwd": 4.0 * unit, "dkdv": 8.0 * unit, "dq": 2.0 * unit}
+
+    def step(events=None):
+        def mark(name):
+            if events is not None:
+                e = torch.cuda.Event(enable_timing=True)
+                e.record()
+                events.append((name, e))
+        mark("start")
+        o, lse = ops.attn_fwd(q, k, v, scale, True)
+        mark("fwd")
+        ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, out=out, stages=ops.BWD_DELTA)
+        mark("delta")
+        ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, out=out, stages=ops.BWD_DKDV)
+        mark("dkdv")
+        ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, out=out, stages=ops.BWD_DQ)
+        mark("dq")
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    all_events = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ev = []
+        step(ev)
+        all_events.append(ev)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+
+    ms_per_step = dt / args.steps * 1e3
+    kern_ms = {}
+    for ev in all_events:
+        for (_, e0), (name, e1) in zip(ev[:-1], ev[1:]):
+            kern_ms[name] = kern_ms.get(name, 0.0) + e0.elapsed_time(e1)
+    kern_ms = {n: t / args.steps for n, t in kern_ms.items()}
+    dominant = max(alg_flops, key=lambda n: kern_ms[n])
+    achieved = alg_flops[dominant] / (kern_ms[dominant] * 1e-3) / 1e12
+    value = flops_step / (ms_per_step * 1e-3) / 1e12
+
+    res = {
+        "metric": "causal attn fwd+bwd TFLOP/s (% bf16 MFMA peak) at T=4096",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "causal attention fwd + recompute bwd, B=4 H=16 T=4096 head_dim=128, bf16 in/out, "
+                               "fp32 accumulate (BASELINE config 4, full causal)", "B": B, "H": H, "T": T,
+                   "head_dim": dk, "causal": True},
+        "pct_of_bf16_mfma_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
+        "tokens_per_s": round(B * T / (ms_per_step * 1e-3), 1),
+        "hbm_gb_per_s_algorithmic": round(bytes_step / (ms_per_step * 1e-3) / 1e9, 1),
+        "kernel_ms": {n: round(t, 4) for n, t in kern_ms.items()},
+        "roofline": {"bound": "mfma", "kernel": dominant, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES},
+    }
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(B, T, H, dk, scale)
+    print(json.dumps(res), flush=True)
+
+
+if __name__ == "__main__":
+    main()

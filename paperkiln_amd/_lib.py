@@ -34,7 +34,7 @@ class PkError(RuntimeError):
 _lib = None
 
 # every symbol include/paperkiln_amd.h declares
-EXPORTS = ["pk_last_error", "pk_init", "pk_attn_fwd", "pk_attn_bwd_workspace_bytes", "pk_attn_bwd"]
+EXPORTS = ["pk_last_error", "pk_init", "pk_attn_fwd", "pk_attn_bwd_workspace_bytes", "pk_attn_bwd", "pk_attn_bwd_stages"]
 
 
 def lib() -> C.CDLL:
@@ -52,6 +52,8 @@ def lib() -> C.CDLL:
         L.pk_attn_bwd_workspace_bytes.argtypes = [SH]
         L.pk_attn_bwd_workspace_bytes.restype = C.c_size_t
         L.pk_attn_bwd.argtypes = [SH, T4, T4, T4, T4, C.c_void_p, T4, T4, T4, T4, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.pk_attn_bwd_stages.argtypes = [SH, T4, T4, T4, T4, C.c_void_p, T4, T4, T4, T4, C.c_void_p, C.c_size_t,
+                                         C.c_int, C.c_void_p]
         _lib = L
     return _lib
 

@@ -368,23 +368,29 @@ __global__ __launch_bounds__(256) void mfma_dq(AttnArgs a) {
 }
 
 template <int D, bool GF32>
-int launch(const AttnArgs& a, hipStream_t st) {
+int launch(const AttnArgs& a, int stages, hipStream_t st) {
     const int64_t rows = static_cast<int64_t>(a.B) * a.Hq * a.T;
     constexpr int RPB = 256 / (D / 8);
-    hipLaunchKernelGGL((mfma_delta<D>), dim3((rows + RPB - 1) / RPB), dim3(256), 0, st, a);
-    PK_HIP(hipGetLastError());
-    hipLaunchKernelGGL((mfma_dkdv<D, GF32>), dim3((a.T + 127) / 128, a.Hkv, a.B), dim3(256), 0, st, a);
-    PK_HIP(hipGetLastError());
-    hipLaunchKernelGGL((mfma_dq<D, GF32>), dim3((a.T + 127) / 128, a.Hq, a.B), dim3(256), 0, st, a);
-    PK_HIP(hipGetLastError());
+    if (stages & PK_BWD_DELTA) {
+        hipLaunchKernelGGL((mfma_delta<D>), dim3((rows + RPB - 1) / RPB), dim3(256), 0, st, a);
+        PK_HIP(hipGetLastError());
+    }
+    if (stages & PK_BWD_DKDV) {
+        hipLaunchKernelGGL((mfma_dkdv<D, GF32>), dim3((a.T + 127) / 128, a.Hkv, a.B), dim3(256), 0, st, a);
+        PK_HIP(hipGetLastError());
+    }
+    if (stages & PK_BWD_DQ) {
+        hipLaunchKernelGGL((mfma_dq<D, GF32>), dim3((a.T + 127) / 128, a.Hq, a.B), dim3(256), 0, st, a);
+        PK_HIP(hipGetLastError());
+    }
     return PK_OK;
 }
 
 }  // namespace
 
-int launch_mfma_bwd(const AttnArgs& a, hipStream_t st) {
-    if (a.dk_dim == 128) return a.grad_f32 ? launch<128, true>(a, st) : launch<128, false>(a, st);
-    return a.grad_f32 ? launch<64, true>(a, st) : launch<64, false>(a, st);
+int launch_mfma_bwd(const AttnArgs& a, int stages, hipStream_t st) {
+    if (a.dk_dim == 128) return a.grad_f32 ? launch<128, true>(a, stages, st) : launch<128, false>(a, stages, st);
+    return a.grad_f32 ? launch<64, true>(a, stages, st) : launch<64, false>(a, stages, st);
 }
 
 }  // namespace pk

@@ -355,20 +355,26 @@ int fwd_impl(const AttnArgs& a, hipStream_t st) {
 }
 
 template <typename IO, typename GO>
-int bwd_impl(const AttnArgs& a, hipStream_t st) {
+int bwd_impl(const AttnArgs& a, int stages, hipStream_t st) {
     const int ld = a.dk_dim + 1;
     const size_t lds = sizeof(float) * (4 * TM * ld + 2 * TM * (TN + 1) + 2 * TM);
     if (int rc = set_lds(generic_bwd_dkdv<IO, GO>, lds)) return rc;
     if (int rc = set_lds(generic_bwd_dq<IO, GO>, lds)) return rc;
     const int64_t rows = static_cast<int64_t>(a.B) * a.Hq * a.T;
-    hipLaunchKernelGGL(generic_delta<IO>, dim3((rows + 3) / 4), dim3(256), 0, st, a);
-    PK_HIP(hipGetLastError());
-    hipLaunchKernelGGL((generic_bwd_dkdv<IO, GO>), dim3((a.T + TN - 1) / TN, a.Hkv, a.B), dim3(256),
-                       lds, st, a);
-    PK_HIP(hipGetLastError());
-    hipLaunchKernelGGL((generic_bwd_dq<IO, GO>), dim3((a.T + TM - 1) / TM, a.Hq, a.B), dim3(256),
-                       lds, st, a);
-    PK_HIP(hipGetLastError());
+    if (stages & PK_BWD_DELTA) {
+        hipLaunchKernelGGL(generic_delta<IO>, dim3((rows + 3) / 4), dim3(256), 0, st, a);
+        PK_HIP(hipGetLastError());
+    }
+    if (stages & PK_BWD_DKDV) {
+        hipLaunchKernelGGL((generic_bwd_dkdv<IO, GO>), dim3((a.T + TN - 1) / TN, a.Hkv, a.B), dim3(256),
+                           lds, st, a);
+        PK_HIP(hipGetLastError());
+    }
+    if (stages & PK_BWD_DQ) {
+        hipLaunchKernelGGL((generic_bwd_dq<IO, GO>), dim3((a.T + TM - 1) / TM, a.Hq, a.B), dim3(256),
+                           lds, st, a);
+        PK_HIP(hipGetLastError());
+    }
     return PK_OK;
 }
 
@@ -378,9 +384,9 @@ int launch_generic_fwd(const AttnArgs& a, bool bf16_in, hipStream_t st) {
     return bf16_in ? fwd_impl<BF16>(a, st) : fwd_impl<F32>(a, st);
 }
 
-int launch_generic_bwd(const AttnArgs& a, bool bf16_in, hipStream_t st) {
-    if (bf16_in) return a.grad_f32 ? bwd_impl<BF16, F32>(a, st) : bwd_impl<BF16, BF16>(a, st);
-    return a.grad_f32 ? bwd_impl<F32, F32>(a, st) : bwd_impl<F32, BF16>(a, st);
+int launch_generic_bwd(const AttnArgs& a, bool bf16_in, int stages, hipStream_t st) {
+    if (bf16_in) return a.grad_f32 ? bwd_impl<BF16, F32>(a, stages, st) : bwd_impl<BF16, BF16>(a, stages, st);
+    return a.grad_f32 ? bwd_impl<F32, F32>(a, stages, st) : bwd_impl<F32, BF16>(a, stages, st);
 }
 
 }  // namespace pk

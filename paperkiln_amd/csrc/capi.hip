@@ -105,7 +105,18 @@ int pk_attn_bwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k
                 const pk_tensor4* o, const float* lse, const pk_tensor4* d_o, const pk_tensor4* dq,
                 const pk_tensor4* dk, const pk_tensor4* dv, void* workspace, size_t workspace_bytes,
                 void* stream) {
+    return pk_attn_bwd_stages(s, q, k, v, o, lse, d_o, dq, dk, dv, workspace, workspace_bytes,
+                              PK_BWD_ALL, stream);
+}
+
+int pk_attn_bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k,
+                       const pk_tensor4* v, const pk_tensor4* o, const float* lse,
+                       const pk_tensor4* d_o, const pk_tensor4* dq, const pk_tensor4* dk,
+                       const pk_tensor4* dv, void* workspace, size_t workspace_bytes, int stages,
+                       void* stream) {
     if (int rc = check_shape(s, "pk_attn_bwd")) return rc;
+    if (stages <= 0 || (stages & ~PK_BWD_ALL))
+        return fail(PK_ERR_ARGUMENT, "pk_attn_bwd_stages: stages must be a non-empty subset of PK_BWD_ALL");
     if (bad(q) || bad(k) || bad(v) || bad(o) || !lse || bad(d_o) || bad(dq) || bad(dk) || bad(dv))
         return fail(PK_ERR_ARGUMENT, "pk_attn_bwd: null tensor");
     if (!workspace || workspace_bytes < pk_attn_bwd_workspace_bytes(s))
@@ -121,8 +132,8 @@ int pk_attn_bwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k
     a.dv = dv->ptr; a.dv_sb = dv->stride_b; a.dv_st = dv->stride_t; a.dv_sh = dv->stride_h;
     a.delta = static_cast<float*>(workspace);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (s->dtype == PK_BF16 && mfma_supported(a)) return launch_mfma_bwd(a, st);
-    return launch_generic_bwd(a, s->dtype == PK_BF16, st);
+    if (s->dtype == PK_BF16 && mfma_supported(a)) return launch_mfma_bwd(a, stages, st);
+    return launch_generic_bwd(a, s->dtype == PK_BF16, stages, st);
 }
 
 }  // extern "C"

@@ -61,11 +61,11 @@ __host__ __device__ inline bool pk_visible(int qi, int kj, int T, int causal, in
 // attn_generic.hip: fp32-math kernels for any head_dim <= 256 and either
 // element type. The fp32 contract (max-abs 1e-5 vs the CPU reference) lives here.
 int launch_generic_fwd(const AttnArgs& a, bool bf16_in, hipStream_t st);
-int launch_generic_bwd(const AttnArgs& a, bool bf16_in, hipStream_t st);
+int launch_generic_bwd(const AttnArgs& a, bool bf16_in, int stages, hipStream_t st);
 
 // attn_fwd_mfma.hip / attn_bwd_mfma.hip: bf16 MFMA kernels, head_dim 64 or 128.
 bool mfma_supported(const AttnArgs& a);
 int launch_mfma_fwd(const AttnArgs& a, hipStream_t st);
-int launch_mfma_bwd(const AttnArgs& a, hipStream_t st);
+int launch_mfma_bwd(const AttnArgs& a, int stages, hipStream_t st);
 
 }  // namespace pk

@@ -55,7 +55,11 @@ def attn_fwd(q, k, v, scale, causal=True, window=0, sinks=0):
     return o, lse
 
 
-def attn_bwd(q, k, v, o, lse, d_o, scale, causal=True, window=0, sinks=0, grad_dtype=None, out=None):
+BWD_DELTA, BWD_DKDV, BWD_DQ, BWD_ALL = 1, 2, 4, 7
+
+
+def attn_bwd(q, k, v, o, lse, d_o, scale, causal=True, window=0, sinks=0, grad_dtype=None, out=None,
+             stages=BWD_ALL):
     """Recompute backward from (Q, K, V, O, LSE, dO). Returns (dq, dk, dv);
     dk/dv are summed over each GQA group. ``out`` may supply preallocated
     (dq, dk, dv, workspace) to keep a timed loop free of allocations."""
@@ -70,9 +74,10 @@ def attn_bwd(q, k, v, o, lse, d_o, scale, causal=True, window=0, sinks=0, grad_d
         ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
     else:
         dq, dk, dv, ws = out
-    _lib.check(L.pk_attn_bwd(C.byref(sh), C.byref(_t4(q)), C.byref(_t4(k)), C.byref(_t4(v)), C.byref(_t4(o)),
-                             C.c_void_p(lse.data_ptr()), C.byref(_t4(d_o)), C.byref(_t4(dq)), C.byref(_t4(dk)),
-                             C.byref(_t4(dv)), C.c_void_p(ws.data_ptr()), ws.numel(), _stream()))
+    _lib.check(L.pk_attn_bwd_stages(C.byref(sh), C.byref(_t4(q)), C.byref(_t4(k)), C.byref(_t4(v)),
+                                    C.byref(_t4(o)), C.c_void_p(lse.data_ptr()), C.byref(_t4(d_o)),
+                                    C.byref(_t4(dq)), C.byref(_t4(dk)), C.byref(_t4(dv)),
+                                    C.c_void_p(ws.data_ptr()), ws.numel(), stages, _stream()))
     return dq, dk, dv
 
 
