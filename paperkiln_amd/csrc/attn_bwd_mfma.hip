@@ -200,6 +200,7 @@ __global__ __launch_bounds__(256) void mfma_dkdv(AttnArgs a) {
             }
             const bool full = qhi < a.T && kw0 + 31 < a.T && (!a.causal || kw0 + 31 <= qlo) &&
                               (a.window == 0 || kw0 + a.window > qhi || kw0 + 31 < a.sinks);
+            const KeyVis kvis(kw0 + c32, a.T, a.causal, a.window, a.sinks);
             // lane = key kw0+c32; element r = query qlo + (r/4)*8 + 4g + r%4
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd) {
@@ -209,11 +210,7 @@ __global__ __launch_bounds__(256) void mfma_dkdv(AttnArgs a) {
                 for (int e = 0; e < 4; ++e) {
                     const int r = qd * 4 + e;
                     float p = __builtin_amdgcn_exp2f(fmaf(s[r], cexp, nl[e]));
-                    if (!full) {
-                        const int qi = qlo + qd * 8 + g * 4 + e;
-                        if (qi >= a.T || !pk_visible(qi, kw0 + c32, a.T, a.causal, a.window, a.sinks))
-                            p = 0.0f;
-                    }
+                    if (!full) p = kvis(qlo + qd * 8 + g * 4 + e) ? p : 0.0f;
                     s[r] = p;
                     dp[r] = p * (dp[r] - dl[e]);
                 }
@@ -282,6 +279,7 @@ __global__ __launch_bounds__(256) void mfma_dq(AttnArgs a) {
         nlse = -a.lse[lrow] * LOG2E;
         dl = a.delta[lrow];
     }
+    const QueryVis qvis(qi, a.T, a.causal, a.window, a.sinks);
     f32x16 dq_acc[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db)
@@ -329,10 +327,7 @@ __global__ __launch_bounds__(256) void mfma_dq(AttnArgs a) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     float p = __builtin_amdgcn_exp2f(fmaf(s[r], cexp, nlse));
-                    if (!full) {
-                        const int kj = n0 + nb * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
-                        if (qi >= a.T || !pk_visible(qi, kj, a.T, a.causal, a.window, a.sinks)) p = 0.0f;
-                    }
+                    if (!full) p = qvis(n0 + nb * 32 + (r >> 2) * 8 + g * 4 + (r & 3)) ? p : 0.0f;
                     dp[r] = p * (dp[r] - dl);
                 }
                 const bf16x8 d0 = c_to_operand<0>(dp), d1 = c_to_operand<1>(dp);

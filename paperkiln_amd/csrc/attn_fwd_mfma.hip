@@ -18,6 +18,8 @@
 // Softmax runs in base 2 with the scale folded into one FMA per element:
 // p = exp2(s*c - m*c), c = scale*log2(e). Fully masked 32x64 blocks are
 // skipped per wavefront, fully masked key tiles are never loaded.
+#include <cstdlib>
+
 #include "mfma_common.h"
 #include "pk_internal.h"
 
@@ -65,8 +67,16 @@ __device__ inline void store_kv_lds(uint16_t* Ks, uint16_t* Vs, const u32x4* kr,
     }
 }
 
-template <int D, int NQ>
-__global__ __launch_bounds__(256) void mfma_fwd(AttnArgs a) {
+// Rescaling the O accumulators costs three VALU ops per element on this
+// machine (they live in accumulation registers), so it is done lazily: the
+// running reference max only moves when some row's new max exceeds it by more
+// than LAZY_T in log2 units. Between moves P = exp2(s*c - m*c) may reach
+// 2^LAZY_T, which bf16 P and the fp32 accumulators hold without loss; the
+// final O = acc / l and LSE = m*scale + ln(l) are exact for any reference m.
+constexpr float LAZY_T = 6.0f;
+
+template <int D, int NQ, int OCC>
+__global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
     using C = FwdCfg<D>;
     constexpr int BM = 128 * NQ;
     constexpr int KK = D / 16;  // k-chunks of the QK^T contraction
@@ -151,13 +161,13 @@ __global__ __launch_bounds__(256) void mfma_fwd(AttnArgs a) {
             const bool full = (n0 + BN - 1 < a.T) && (!a.causal || n0 + BN - 1 <= qlo) &&
                               (a.window == 0 || n0 + a.window > qhi || n0 + BN - 1 < a.sinks);
             if (!full) {
-                const int qi = qlo + c32;
+                const QueryVis vis(qlo + c32, a.T, a.causal, a.window, a.sinks);
 #pragma unroll
                 for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const int kj = n0 + nb * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
-                        if (!pk_visible(qi, kj, a.T, a.causal, a.window, a.sinks)) s[nb][r] = -INFINITY;
+                        s[nb][r] = vis(kj) ? s[nb][r] : -INFINITY;
                     }
             }
             float mx = -INFINITY;
@@ -166,9 +176,17 @@ __global__ __launch_bounds__(256) void mfma_fwd(AttnArgs a) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[nb][r]);
             mx = xhalf_max(mx);
-            const float mn = fmaxf(m[qb], mx);
-            const float alpha = __builtin_amdgcn_exp2f((m[qb] - mn) * cexp);
-            const float mc = mn * cexp;
+            if (__any((mx - m[qb]) * cexp > a.lazy_t)) {  // wavefront-uniform, rare after the first tiles
+                const float mn = fmaxf(m[qb], mx);
+                const float alpha = __builtin_amdgcn_exp2f((m[qb] - mn) * cexp);
+                l[qb] *= alpha;
+                m[qb] = mn;
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc_o[qb][db][r] *= alpha;
+            }
+            const float mc = m[qb] * cexp;
             float psum = 0.0f;
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb)
@@ -178,12 +196,7 @@ __global__ __launch_bounds__(256) void mfma_fwd(AttnArgs a) {
                     s[nb][r] = p;
                     psum += p;
                 }
-            l[qb] = l[qb] * alpha + psum;  // per-lane partial; the two halves meet in the epilogue
-            m[qb] = mn;
-#pragma unroll
-            for (int db = 0; db < DB; ++db)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc_o[qb][db][r] *= alpha;
+            l[qb] += psum;  // per-lane partial; the two halves meet in the epilogue
 
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) {
@@ -226,11 +239,11 @@ __global__ __launch_bounds__(256) void mfma_fwd(AttnArgs a) {
     }
 }
 
-template <int D, int NQ>
+template <int D, int NQ, int OCC>
 int launch(const AttnArgs& a, hipStream_t st) {
     constexpr int BM = 128 * NQ;
     dim3 grid((a.T + BM - 1) / BM, a.Hq, a.B);
-    hipLaunchKernelGGL((mfma_fwd<D, NQ>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((mfma_fwd<D, NQ, OCC>), grid, dim3(256), 0, st, a);
     PK_HIP(hipGetLastError());
     return PK_OK;
 }
@@ -258,12 +271,22 @@ bool mfma_supported(const AttnArgs& a) {
     return true;
 }
 
-int launch_mfma_fwd(const AttnArgs& a, hipStream_t st) {
+int launch_mfma_fwd(const AttnArgs& a0, hipStream_t st) {
+    AttnArgs a = a0;
+    a.lazy_t = getenv("PK_LAZY_T") ? atof(getenv("PK_LAZY_T")) : LAZY_T;
     // Two 32-query blocks per wavefront halve the LDS traffic per MFMA; short
     // sequences keep one so that the grid still covers the chip.
+    static const int variant = getenv("PK_FWD_VARIANT") ? atoi(getenv("PK_FWD_VARIANT")) : 0;
     const bool big = static_cast<int64_t>(a.T) * a.Hq * a.B >= 256 * 256 * 2;
-    if (a.dk_dim == 128) return big ? launch<128, 2>(a, st) : launch<128, 1>(a, st);
-    return big ? launch<64, 2>(a, st) : launch<64, 1>(a, st);
+    if (a.dk_dim == 128) {
+        if (variant == 1) return launch<128, 1, 2>(a, st);
+        if (variant == 2) return launch<128, 1, 1>(a, st);
+        if (variant == 3) return launch<128, 2, 1>(a, st);
+        return launch<128, 1, 2>(a, st);
+    }
+    if (variant == 1) return launch<64, 1, 2>(a, st);
+    if (variant == 3) return launch<64, 2, 1>(a, st);
+    return launch<64, 1, 2>(a, st);
 }
 
 }  // namespace pk

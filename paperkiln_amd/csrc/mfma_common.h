@@ -86,4 +86,31 @@ __device__ inline bf16x8 lds_read_tr_operand(const uint16_t* tile, int stride, i
     return *reinterpret_cast<bf16x8*>(&v);
 }
 
+// Branch-free visibility tests (the reference's two ranges, paperkiln
+// src/ops.cpp:879-880, 960-965). Written with non-short-circuit & and | so
+// that each element costs a few compares and one select, never a branch.
+//
+// QueryVis: fixed query, varying key (lane = query kernels).
+struct QueryVis {
+    int hi;      // keys [0, hi) pass the causal / length test
+    int win_lo;  // keys >= win_lo are inside the band
+    int sinks;   // keys < sinks are always visible (0 without a band)
+    __device__ QueryVis(int qi, int T, int causal, int window, int sinks_)
+        : hi(qi < T ? (causal ? min(qi + 1, T) : T) : 0),
+          win_lo(window > 0 ? qi + 1 - window : -0x40000000),
+          sinks(window > 0 ? sinks_ : 0) {}
+    __device__ bool operator()(int kj) const { return (kj < hi) & ((kj >= win_lo) | (kj < sinks)); }
+};
+// KeyVis: fixed key, varying query (lane = key kernels).
+struct KeyVis {
+    int q_lo;    // queries >= q_lo pass the causal test
+    int q_hi;    // queries < q_hi are inside the band (or the key is a sink)
+    int T;
+    __device__ KeyVis(int kj, int T_, int causal, int window, int sinks)
+        : q_lo(kj < T_ ? (causal ? kj : 0) : 0x40000000),
+          q_hi((window > 0 && kj >= sinks) ? kj + window : 0x40000000),
+          T(T_) {}
+    __device__ bool operator()(int qi) const { return (qi >= q_lo) & (qi < q_hi) & (qi < T); }
+};
+
 }  // namespace pk

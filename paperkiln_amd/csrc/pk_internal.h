@@ -45,6 +45,7 @@ struct AttnArgs {
     int causal, window, sinks;
     int grad_f32; // dq/dk/dv element type: 1 = fp32, 0 = bf16
     float scale;
+    float lazy_t; // debug
 };
 
 // Visible-set test shared by every kernel: the reference's two ranges
