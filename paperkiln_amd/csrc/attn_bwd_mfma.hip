@@ -126,10 +126,11 @@ __global__ __launch_bounds__(256) void mfma_dkdv(AttnArgs a) {
 
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int g = lane >> 5, c32 = lane & 31;
-    const int kblk = gridDim.x - 1 - blockIdx.x;  // fewest visible queries last
-    const int k0 = kblk * BNK, hk = blockIdx.y, b = blockIdx.z;
+    const int nkb = (a.T + BNK - 1) / BNK, rep = a.Hq / a.Hkv;
+    int kblk, rr, kvu;
+    if (!xcd_map(nkb, 1, a.Hkv * a.B, kblk, rr, kvu)) return;  // key block 0 sees the most queries: first
+    const int k0 = kblk * BNK, hk = kvu % a.Hkv, b = kvu / a.Hkv;
     const int kw0 = k0 + w * 32;  // this wavefront's keys
-    const int rep = a.Hq / a.Hkv;
     const float cexp = a.scale * LOG2E;
 
     bf16x8 kreg[KK], vreg[KK];
@@ -220,13 +221,13 @@ __global__ __launch_bounds__(256) void mfma_dkdv(AttnArgs a) {
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 // dV^T += dO^T P ; dK^T += Q^T dS   (A = transposed LDS tiles)
-                const bf16x8 g0 = lds_read_tr_operand(dOs, QT::S, qb * 32, db * 32, lane);
+                const bf16x8 g0 = lds_read_tr_operand_perm<D>(dOs, QT::S, qb * 32, db, lane);
                 dv_acc[db] = mfma32(g0, p0, dv_acc[db]);
-                const bf16x8 g1 = lds_read_tr_operand(dOs, QT::S, qb * 32 + 16, db * 32, lane);
+                const bf16x8 g1 = lds_read_tr_operand_perm<D>(dOs, QT::S, qb * 32 + 16, db, lane);
                 dv_acc[db] = mfma32(g1, p1, dv_acc[db]);
-                const bf16x8 q0f = lds_read_tr_operand(Qs, QT::S, qb * 32, db * 32, lane);
+                const bf16x8 q0f = lds_read_tr_operand_perm<D>(Qs, QT::S, qb * 32, db, lane);
                 dk_acc[db] = mfma32(q0f, d0, dk_acc[db]);
-                const bf16x8 q1f = lds_read_tr_operand(Qs, QT::S, qb * 32 + 16, db * 32, lane);
+                const bf16x8 q1f = lds_read_tr_operand_perm<D>(Qs, QT::S, qb * 32 + 16, db, lane);
                 dk_acc[db] = mfma32(q1f, d1, dk_acc[db]);
             }
         }
@@ -243,7 +244,7 @@ __global__ __launch_bounds__(256) void mfma_dkdv(AttnArgs a) {
         for (int db = 0; db < DB; ++db)
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd) {
-                const int d0 = db * 32 + qd * 8 + g * 4;
+                const int d0 = TrMap<D>::col0(db, qd, g);
                 store4<GF32>(a.dk, kb + d0, dk_acc[db][qd * 4] * a.scale, dk_acc[db][qd * 4 + 1] * a.scale,
                              dk_acc[db][qd * 4 + 2] * a.scale, dk_acc[db][qd * 4 + 3] * a.scale);
                 store4<GF32>(a.dv, vb + d0, dv_acc[db][qd * 4], dv_acc[db][qd * 4 + 1],
@@ -263,9 +264,12 @@ __global__ __launch_bounds__(256) void mfma_dq(AttnArgs a) {
 
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int g = lane >> 5, c32 = lane & 31;
-    const int qblk = gridDim.x - 1 - blockIdx.x;
-    const int q0 = qblk * BM, h = blockIdx.y, b = blockIdx.z;
-    const int hk = h / (a.Hq / a.Hkv);
+    const int nqb = (a.T + BM - 1) / BM, rep = a.Hq / a.Hkv;
+    int blk, rr, kvu;
+    if (!xcd_map(nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
+    const int qblk = nqb - 1 - blk;
+    const int hk = kvu % a.Hkv, b = kvu / a.Hkv, h = hk * rep + rr;
+    const int q0 = qblk * BM;
     const int qlo = q0 + w * 32, qhi = qlo + 31, qi = qlo + c32;
     const int64_t kb = b * a.k_sb + hk * a.k_sh, vb = b * a.v_sb + hk * a.v_sh;
     const float cexp = a.scale * LOG2E;
@@ -334,9 +338,9 @@ __global__ __launch_bounds__(256) void mfma_dq(AttnArgs a) {
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
                     // dQ^T += K^T dS^T
-                    const bf16x8 k0f = lds_read_tr_operand(Ks, KT::S, nb * 32, db * 32, lane);
+                    const bf16x8 k0f = lds_read_tr_operand_perm<D>(Ks, KT::S, nb * 32, db, lane);
                     dq_acc[db] = mfma32(k0f, d0, dq_acc[db]);
-                    const bf16x8 k1f = lds_read_tr_operand(Ks, KT::S, nb * 32 + 16, db * 32, lane);
+                    const bf16x8 k1f = lds_read_tr_operand_perm<D>(Ks, KT::S, nb * 32 + 16, db, lane);
                     dq_acc[db] = mfma32(k1f, d1, dq_acc[db]);
                 }
             }
@@ -356,7 +360,7 @@ __global__ __launch_bounds__(256) void mfma_dq(AttnArgs a) {
         for (int db = 0; db < DB; ++db)
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd)
-                store4<GF32>(a.dq, ob + db * 32 + qd * 8 + g * 4, dq_acc[db][qd * 4] * a.scale,
+                store4<GF32>(a.dq, ob + TrMap<D>::col0(db, qd, g), dq_acc[db][qd * 4] * a.scale,
                              dq_acc[db][qd * 4 + 1] * a.scale, dq_acc[db][qd * 4 + 2] * a.scale,
                              dq_acc[db][qd * 4 + 3] * a.scale);
     }
@@ -371,11 +375,12 @@ int launch(const AttnArgs& a, int stages, hipStream_t st) {
         PK_HIP(hipGetLastError());
     }
     if (stages & PK_BWD_DKDV) {
-        hipLaunchKernelGGL((mfma_dkdv<D, GF32>), dim3((a.T + 127) / 128, a.Hkv, a.B), dim3(256), 0, st, a);
+        hipLaunchKernelGGL((mfma_dkdv<D, GF32>), dim3(xcd_grid((a.T + 127) / 128, 1, a.Hkv * a.B)), dim3(256), 0, st, a);
         PK_HIP(hipGetLastError());
     }
     if (stages & PK_BWD_DQ) {
-        hipLaunchKernelGGL((mfma_dq<D, GF32>), dim3((a.T + 127) / 128, a.Hq, a.B), dim3(256), 0, st, a);
+        hipLaunchKernelGGL((mfma_dq<D, GF32>), dim3(xcd_grid((a.T + 127) / 128, a.Hq / a.Hkv, a.Hkv * a.B)), dim3(256), 0, st,
+                           a);
         PK_HIP(hipGetLastError());
     }
     return PK_OK;

@@ -81,15 +81,19 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
     constexpr int BM = 128 * NQ;
     constexpr int KK = D / 16;  // k-chunks of the QK^T contraction
     constexpr int DB = D / 32;  // 32-row blocks of O^T
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[BN * C::KS];
-    __shared__ __attribute__((aligned(16))) uint16_t Vs[BN * C::VS];
+    // two K/V tile buffers: tile t+1 is stored while tile t is being read, one barrier per tile
+    __shared__ __attribute__((aligned(16))) uint16_t Kbuf[2][BN * C::KS];
+    __shared__ __attribute__((aligned(16))) uint16_t Vbuf[2][BN * C::VS];
 
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int g = lane >> 5, c32 = lane & 31;
+    const int nqb = (a.T + BM - 1) / BM, rep = a.Hq / a.Hkv;
+    int blk, rr, kvu;
+    if (!xcd_map(nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
     // Heaviest query blocks (most visible keys) are dispatched first.
-    const int qblk = gridDim.x - 1 - blockIdx.x;
-    const int q0 = qblk * BM, h = blockIdx.y, b = blockIdx.z;
-    const int hk = h / (a.Hq / a.Hkv);
+    const int qblk = nqb - 1 - blk;
+    const int hk = kvu % a.Hkv, b = kvu / a.Hkv, h = hk * rep + rr;
+    const int q0 = qblk * BM;
     const int64_t qb_off = b * a.q_sb + h * a.q_sh;
     const int64_t kb = b * a.k_sb + hk * a.k_sh, vb = b * a.v_sb + hk * a.v_sh;
     const float cexp = a.scale * 1.4426950408889634f;
@@ -131,13 +135,16 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
 
     u32x4 kr[C::CPT], vr[C::CPT];
     load_kv_regs<D>(a, kb, vb, t * BN, kr, vr);
-    store_kv_lds<D>(Ks, Vs, kr, vr);
+    store_kv_lds<D>(Kbuf[0], Vbuf[0], kr, vr);
     __syncthreads();
+    int cur = 0;
 
     while (t <= hi) {
         const int n0 = t * BN;
         const int tn = (t + 1 == ns) ? lo : t + 1;
         if (tn <= hi) load_kv_regs<D>(a, kb, vb, tn * BN, kr, vr);  // in flight during the math
+        const uint16_t* Ks = Kbuf[cur];
+        const uint16_t* Vs = Vbuf[cur];
 
 #pragma unroll
         for (int qb = 0; qb < NQ; ++qb) {
@@ -152,11 +159,11 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
             for (int nb = 0; nb < 2; ++nb) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s[nb][r] = 0.0f;
+                bf16x8 kf[KK];
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) {
-                    bf16x8 kf = lds_read8(Ks + (nb * 32 + c32) * C::KS + kk * 16 + g * 8);
-                    s[nb] = mfma32(kf, qreg[qb][kk], s[nb]);
-                }
+                for (int kk = 0; kk < KK; ++kk) kf[kk] = lds_read8(Ks + (nb * 32 + c32) * C::KS + kk * 16 + g * 8);
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) s[nb] = mfma32(kf[kk], qreg[qb][kk], s[nb]);
             }
             const bool full = (n0 + BN - 1 < a.T) && (!a.causal || n0 + BN - 1 <= qlo) &&
                               (a.window == 0 || n0 + a.window > qhi || n0 + BN - 1 < a.sinks);
@@ -212,9 +219,10 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
             }
         }
 
-        __syncthreads();  // every wavefront is done reading this tile
-        if (tn <= hi) store_kv_lds<D>(Ks, Vs, kr, vr);
+        // The other buffer was last read one iteration ago, before the previous barrier.
+        if (tn <= hi) store_kv_lds<D>(Kbuf[cur ^ 1], Vbuf[cur ^ 1], kr, vr);
         __syncthreads();
+        cur ^= 1;
         t = tn;
     }
 
@@ -242,7 +250,7 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
 template <int D, int NQ, int OCC>
 int launch(const AttnArgs& a, hipStream_t st) {
     constexpr int BM = 128 * NQ;
-    dim3 grid((a.T + BM - 1) / BM, a.Hq, a.B);
+    dim3 grid(xcd_grid((a.T + BM - 1) / BM, a.Hq / a.Hkv, a.Hkv * a.B));
     hipLaunchKernelGGL((mfma_fwd<D, NQ, OCC>), grid, dim3(256), 0, st, a);
     PK_HIP(hipGetLastError());
     return PK_OK;

@@ -86,6 +86,59 @@ __device__ inline bf16x8 lds_read_tr_operand(const uint16_t* tile, int stride, i
     return *reinterpret_cast<bf16x8*>(&v);
 }
 
+// The same operand read from a tile whose row pitch is 4 banks past a multiple
+// of 64 (the pitch that keeps 16-byte row reads conflict-free). With that
+// pitch the natural column order would put two of the four rows of a
+// transposing read on the same banks, so for head_dim 128 the 32 columns of
+// MFMA block `db` are taken in a permuted order: lane 16u + 4a + c reads
+// column 4*(8a + u + 2db) + c. Every 32-lane half then touches all 64 banks
+// exactly once. The permutation only renames the rows of the product; tr_col0
+// gives, for accumulator element group qd (= r/4) of block db on half g, the
+// first of the 4 consecutive true columns that elements 4qd..4qd+3 hold.
+template <int D>
+struct TrMap;
+template <>
+struct TrMap<128> {
+    __device__ static int src_col(int db, int u, int a) { return 4 * (8 * a + u + 2 * db); }
+    __device__ static int col0(int db, int qd, int g) { return 32 * (2 * (qd & 1) + g) + 4 * (qd >> 1) + 8 * db; }
+};
+template <>
+struct TrMap<64> {  // natural order
+    __device__ static int src_col(int db, int u, int a) { return 32 * db + 16 * u + 4 * a; }
+    __device__ static int col0(int db, int qd, int g) { return 32 * db + 8 * qd + 4 * g; }
+};
+template <int D>
+__device__ inline bf16x8 lds_read_tr_operand_perm(const uint16_t* tile, int stride, int row0, int db,
+                                                  int lane) {
+    const int g = lane >> 5, u = (lane >> 4) & 1, j = lane & 15;
+    const uint16_t* p = tile + (row0 + 4 * g + (j >> 2)) * stride + TrMap<D>::src_col(db, u, j & 3);
+    s16x4 lo = lds_read_tr4(p);
+    s16x4 hi = lds_read_tr4(p + 8 * stride);
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return *reinterpret_cast<bf16x8*>(&v);
+}
+
+// XCD-aware workgroup -> tile mapping. The 256 CUs sit in 8 XCDs, each with
+// its own 4 MB L2, and consecutive workgroup ids go round-robin over the XCDs.
+// Every block of a (batch, KV head) unit re-reads that unit's K/V (or Q/dO),
+// so all blocks of a unit -- and of the `rep` query heads sharing the KV head --
+// are given ids that are congruent mod 8: one unit's tensors then live in ONE
+// L2 instead of being fetched into all eight.
+// Launch with grid.x = xcd_grid(nblk, rep, kv_units).
+__host__ __device__ inline int xcd_grid(int nblk, int rep, int kv_units) {
+    return nblk * rep * ((kv_units + 7) / 8) * 8;
+}
+// blk: block index inside the unit (0 = dispatched first); r: query head inside
+// the GQA group; kvu: (batch, KV head) unit. Returns false for padding ids.
+__device__ inline bool xcd_map(int nblk, int rep, int kv_units, int& blk, int& r, int& kvu) {
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    blk = j % nblk;
+    r = (j / nblk) % rep;
+    kvu = (j / (nblk * rep)) * 8 + xcd;
+    return kvu < kv_units;
+}
+
 // Branch-free visibility tests (the reference's two ranges, paperkiln
 // src/ops.cpp:879-880, 960-965). Written with non-short-circuit & and | so
 // that each element costs a few compares and one select, never a branch.
