@@ -29,6 +29,9 @@ namespace pk {
 namespace {
 
 constexpr float LOG2E = 1.4426950408889634f;
+#ifndef PK_DKDV_OCC
+#define PK_DKDV_OCC 1
+#endif
 
 // ---- delta --------------------------------------------------------------
 template <int D>
@@ -114,7 +117,7 @@ __device__ inline void store4(void* base, int64_t idx, float x0, float x1, float
 
 // ---- dK, dV ---------------------------------------------------------------
 template <int D, bool GF32>
-__global__ __launch_bounds__(256) void mfma_dkdv(AttnArgs a) {
+__global__ __launch_bounds__(256, PK_DKDV_OCC) void mfma_dkdv(AttnArgs a) {
     constexpr int BMQ = 64;   // queries per step
     constexpr int BNK = 128;  // keys per workgroup
     constexpr int KK = D / 16, DB = D / 32;
@@ -127,9 +130,16 @@ __global__ __launch_bounds__(256) void mfma_dkdv(AttnArgs a) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int g = lane >> 5, c32 = lane & 31;
     const int nkb = (a.T + BNK - 1) / BNK, rep = a.Hq / a.Hkv;
-    int kblk, rr, kvu;
-    if (!xcd_map(nkb, 1, a.Hkv * a.B, kblk, rr, kvu)) return;  // key block 0 sees the most queries: first
-    const int k0 = kblk * BNK, hk = kvu % a.Hkv, b = kvu / a.Hkv;
+    // Full-causal: key block i is seen by T - 128i queries; blocks i and nkb-1-i
+    // are taken back to back so that every workgroup carries the same work.
+    const bool paired = a.causal && a.window == 0;
+    int blk, rr, kvu;
+    if (!xcd_map(paired ? (nkb + 1) / 2 : nkb, 1, a.Hkv * a.B, blk, rr, kvu)) return;
+    const int hk = kvu % a.Hkv, b = kvu / a.Hkv;
+    const int npass = (paired && blk != nkb - 1 - blk) ? 2 : 1;
+  for (int pass = 0; pass < npass; ++pass) {
+    const int kblk = pass == 0 ? blk : nkb - 1 - blk;  // heavy block first
+    const int k0 = kblk * BNK;
     const int kw0 = k0 + w * 32;  // this wavefront's keys
     const float cexp = a.scale * LOG2E;
 
@@ -218,17 +228,17 @@ __global__ __launch_bounds__(256) void mfma_dkdv(AttnArgs a) {
             }
             const bf16x8 p0 = c_to_operand<0>(s), p1 = c_to_operand<1>(s);
             const bf16x8 d0 = c_to_operand<0>(dp), d1 = c_to_operand<1>(dp);
+            // dV^T += dO^T P ; dK^T += Q^T dS (A = transposed LDS tiles). Consecutive
+            // MFMAs go to different accumulators (a dependent pair costs 52 cycles, not 32).
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                // dV^T += dO^T P ; dK^T += Q^T dS   (A = transposed LDS tiles)
-                const bf16x8 g0 = lds_read_tr_operand_perm<D>(dOs, QT::S, qb * 32, db, lane);
-                dv_acc[db] = mfma32(g0, p0, dv_acc[db]);
-                const bf16x8 g1 = lds_read_tr_operand_perm<D>(dOs, QT::S, qb * 32 + 16, db, lane);
-                dv_acc[db] = mfma32(g1, p1, dv_acc[db]);
-                const bf16x8 q0f = lds_read_tr_operand_perm<D>(Qs, QT::S, qb * 32, db, lane);
-                dk_acc[db] = mfma32(q0f, d0, dk_acc[db]);
-                const bf16x8 q1f = lds_read_tr_operand_perm<D>(Qs, QT::S, qb * 32 + 16, db, lane);
-                dk_acc[db] = mfma32(q1f, d1, dk_acc[db]);
+                dv_acc[db] = mfma32(lds_read_tr_operand_perm<D>(dOs, QT::S, qb * 32, db, lane), p0, dv_acc[db]);
+                dk_acc[db] = mfma32(lds_read_tr_operand_perm<D>(Qs, QT::S, qb * 32, db, lane), d0, dk_acc[db]);
+            }
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                dv_acc[db] = mfma32(lds_read_tr_operand_perm<D>(dOs, QT::S, qb * 32 + 16, db, lane), p1, dv_acc[db]);
+                dk_acc[db] = mfma32(lds_read_tr_operand_perm<D>(Qs, QT::S, qb * 32 + 16, db, lane), d1, dk_acc[db]);
             }
         }
         __syncthreads();
@@ -251,11 +261,13 @@ __global__ __launch_bounds__(256) void mfma_dkdv(AttnArgs a) {
                              dv_acc[db][qd * 4 + 2], dv_acc[db][qd * 4 + 3]);
             }
     }
+    __syncthreads();  // the next pass refills the tile buffers
+  }
 }
 
 // ---- dQ -------------------------------------------------------------------
 template <int D, bool GF32>
-__global__ __launch_bounds__(256) void mfma_dq(AttnArgs a) {
+__global__ __launch_bounds__(256, 2) void mfma_dq(AttnArgs a) {
     constexpr int BM = 128, BN = 64;
     constexpr int KK = D / 16, DB = D / 32;
     using KT = Tile<D, BN>;
@@ -265,10 +277,13 @@ __global__ __launch_bounds__(256) void mfma_dq(AttnArgs a) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int g = lane >> 5, c32 = lane & 31;
     const int nqb = (a.T + BM - 1) / BM, rep = a.Hq / a.Hkv;
+    const bool paired = a.causal && a.window == 0;  // as in the forward kernel
     int blk, rr, kvu;
-    if (!xcd_map(nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
-    const int qblk = nqb - 1 - blk;
+    if (!xcd_map(paired ? (nqb + 1) / 2 : nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv, h = hk * rep + rr;
+    const int npass = (paired && blk != nqb - 1 - blk) ? 2 : 1;
+  for (int pass = 0; pass < npass; ++pass) {
+    const int qblk = pass == 0 ? nqb - 1 - blk : blk;
     const int q0 = qblk * BM;
     const int qlo = q0 + w * 32, qhi = qlo + 31, qi = qlo + c32;
     const int64_t kb = b * a.k_sb + hk * a.k_sh, vb = b * a.v_sb + hk * a.v_sh;
@@ -335,14 +350,13 @@ __global__ __launch_bounds__(256) void mfma_dq(AttnArgs a) {
                     dp[r] = p * (dp[r] - dl);
                 }
                 const bf16x8 d0 = c_to_operand<0>(dp), d1 = c_to_operand<1>(dp);
+                // dQ^T += K^T dS^T, DB independent chains per k-chunk
 #pragma unroll
-                for (int db = 0; db < DB; ++db) {
-                    // dQ^T += K^T dS^T
-                    const bf16x8 k0f = lds_read_tr_operand_perm<D>(Ks, KT::S, nb * 32, db, lane);
-                    dq_acc[db] = mfma32(k0f, d0, dq_acc[db]);
-                    const bf16x8 k1f = lds_read_tr_operand_perm<D>(Ks, KT::S, nb * 32 + 16, db, lane);
-                    dq_acc[db] = mfma32(k1f, d1, dq_acc[db]);
-                }
+                for (int db = 0; db < DB; ++db)
+                    dq_acc[db] = mfma32(lds_read_tr_operand_perm<D>(Ks, KT::S, nb * 32, db, lane), d0, dq_acc[db]);
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                    dq_acc[db] = mfma32(lds_read_tr_operand_perm<D>(Ks, KT::S, nb * 32 + 16, db, lane), d1, dq_acc[db]);
             }
         }
         __syncthreads();
@@ -364,23 +378,28 @@ __global__ __launch_bounds__(256) void mfma_dq(AttnArgs a) {
                              dq_acc[db][qd * 4 + 1] * a.scale, dq_acc[db][qd * 4 + 2] * a.scale,
                              dq_acc[db][qd * 4 + 3] * a.scale);
     }
+    __syncthreads();  // the next pass refills the tile buffers
+  }
 }
 
 template <int D, bool GF32>
 int launch(const AttnArgs& a, int stages, hipStream_t st) {
     const int64_t rows = static_cast<int64_t>(a.B) * a.Hq * a.T;
     constexpr int RPB = 256 / (D / 8);
+    const int nb128 = (a.T + 127) / 128;
+    const bool paired = a.causal && a.window == 0;
     if (stages & PK_BWD_DELTA) {
         hipLaunchKernelGGL((mfma_delta<D>), dim3((rows + RPB - 1) / RPB), dim3(256), 0, st, a);
         PK_HIP(hipGetLastError());
     }
     if (stages & PK_BWD_DKDV) {
-        hipLaunchKernelGGL((mfma_dkdv<D, GF32>), dim3(xcd_grid((a.T + 127) / 128, 1, a.Hkv * a.B)), dim3(256), 0, st, a);
+        hipLaunchKernelGGL((mfma_dkdv<D, GF32>), dim3(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, 1, a.Hkv * a.B)), dim3(256),
+                           0, st, a);
         PK_HIP(hipGetLastError());
     }
     if (stages & PK_BWD_DQ) {
-        hipLaunchKernelGGL((mfma_dq<D, GF32>), dim3(xcd_grid((a.T + 127) / 128, a.Hq / a.Hkv, a.Hkv * a.B)), dim3(256), 0, st,
-                           a);
+        hipLaunchKernelGGL((mfma_dq<D, GF32>), dim3(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, a.Hq / a.Hkv, a.Hkv * a.B)),
+                           dim3(256), 0, st, a);
         PK_HIP(hipGetLastError());
     }
     return PK_OK;

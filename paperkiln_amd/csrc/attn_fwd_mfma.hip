@@ -88,11 +88,17 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int g = lane >> 5, c32 = lane & 31;
     const int nqb = (a.T + BM - 1) / BM, rep = a.Hq / a.Hkv;
+    // Full-causal work per query block grows linearly with its index, so a
+    // workgroup takes blocks i and nqb-1-i back to back: every workgroup then
+    // carries the same number of key tiles and the last wave of workgroups
+    // does not idle three quarters of the chip.
+    const bool paired = a.causal && a.window == 0;
     int blk, rr, kvu;
-    if (!xcd_map(nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
-    // Heaviest query blocks (most visible keys) are dispatched first.
-    const int qblk = nqb - 1 - blk;
+    if (!xcd_map(paired ? (nqb + 1) / 2 : nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv, h = hk * rep + rr;
+    const int npass = (paired && blk != nqb - 1 - blk) ? 2 : 1;
+  for (int pass = 0; pass < npass; ++pass) {
+    const int qblk = pass == 0 ? nqb - 1 - blk : blk;
     const int q0 = qblk * BM;
     const int64_t qb_off = b * a.q_sb + h * a.q_sh;
     const int64_t kb = b * a.k_sb + hk * a.k_sh, vb = b * a.v_sb + hk * a.v_sh;
@@ -139,6 +145,13 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
     __syncthreads();
     int cur = 0;
 
+#ifdef PK_TIMING
+    long long tacc[5] = {0, 0, 0, 0, 0};
+    long long tprev = __builtin_readcyclecounter();
+#define PK_TICK(i) { long long now = __builtin_readcyclecounter(); tacc[i] += now - tprev; tprev = now; }
+#else
+#define PK_TICK(i)
+#endif
     while (t <= hi) {
         const int n0 = t * BN;
         const int tn = (t + 1 == ns) ? lo : t + 1;
@@ -154,17 +167,19 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
             if (a.causal && n0 > qhi) continue;
             if (a.window > 0 && n0 + BN - 1 + a.window <= qlo && n0 >= a.sinks) continue;
 
+            // Two independent accumulator chains, issued alternately: a dependent
+            // v_mfma_32x32x16 pair costs 52 cycles, an independent one 32.
             f32x16 s[2];
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) {
+            for (int r = 0; r < 16; ++r) s[0][r] = s[1][r] = 0.0f;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) s[nb][r] = 0.0f;
-                bf16x8 kf[KK];
-#pragma unroll
-                for (int kk = 0; kk < KK; ++kk) kf[kk] = lds_read8(Ks + (nb * 32 + c32) * C::KS + kk * 16 + g * 8);
-#pragma unroll
-                for (int kk = 0; kk < KK; ++kk) s[nb] = mfma32(kf[kk], qreg[qb][kk], s[nb]);
+            for (int kk = 0; kk < KK; ++kk) {
+                const bf16x8 k0f = lds_read8(Ks + c32 * C::KS + kk * 16 + g * 8);
+                const bf16x8 k1f = lds_read8(Ks + (32 + c32) * C::KS + kk * 16 + g * 8);
+                s[0] = mfma32(k0f, qreg[qb][kk], s[0]);
+                s[1] = mfma32(k1f, qreg[qb][kk], s[1]);
             }
+            PK_TICK(0)
             const bool full = (n0 + BN - 1 < a.T) && (!a.causal || n0 + BN - 1 <= qlo) &&
                               (a.window == 0 || n0 + a.window > qhi || n0 + BN - 1 < a.sinks);
             if (!full) {
@@ -204,28 +219,38 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
                     psum += p;
                 }
             l[qb] += psum;  // per-lane partial; the two halves meet in the epilogue
+            PK_TICK(1)
 
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) {
                 const bf16x8 p0 = c_to_operand<0>(s[nb]);
                 const bf16x8 p1 = c_to_operand<1>(s[nb]);
 #pragma unroll
-                for (int db = 0; db < DB; ++db) {
-                    bf16x8 v0 = lds_read_tr_operand(Vs, C::VS, nb * 32, db * 32, lane);
-                    acc_o[qb][db] = mfma32(v0, p0, acc_o[qb][db]);
-                    bf16x8 v1 = lds_read_tr_operand(Vs, C::VS, nb * 32 + 16, db * 32, lane);
-                    acc_o[qb][db] = mfma32(v1, p1, acc_o[qb][db]);
-                }
+                for (int db = 0; db < DB; ++db)  // DB independent chains per k-chunk
+                    acc_o[qb][db] = mfma32(lds_read_tr_operand(Vs, C::VS, nb * 32, db * 32, lane), p0, acc_o[qb][db]);
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                    acc_o[qb][db] = mfma32(lds_read_tr_operand(Vs, C::VS, nb * 32 + 16, db * 32, lane), p1, acc_o[qb][db]);
             }
         }
 
+        PK_TICK(2)
         // The other buffer was last read one iteration ago, before the previous barrier.
         if (tn <= hi) store_kv_lds<D>(Kbuf[cur ^ 1], Vbuf[cur ^ 1], kr, vr);
+        PK_TICK(3)
         __syncthreads();
+        PK_TICK(4)
         cur ^= 1;
         t = tn;
     }
 
+#ifdef PK_TIMING
+    if (a.delta && lane == 0) {
+        long long* dbg = reinterpret_cast<long long*>(a.delta) + (static_cast<long long>(blockIdx.x) * 4 + w) * 8;
+        for (int i = 0; i < 5; ++i) dbg[i] = tacc[i];
+        dbg[5] = hi + 1;
+    }
+#endif
     // Epilogue: O = acc / l, LSE = m*scale + ln(l) (natural log, scaled units).
 #pragma unroll
     for (int qb = 0; qb < NQ; ++qb) {
@@ -245,12 +270,16 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
         if (g == 0)
             a.lse[(static_cast<int64_t>(b) * a.Hq + h) * a.T + qi] = m[qb] * a.scale + logf(lt);
     }
+    __syncthreads();  // the next pass refills the tile buffers
+  }
 }
 
 template <int D, int NQ, int OCC>
 int launch(const AttnArgs& a, hipStream_t st) {
     constexpr int BM = 128 * NQ;
-    dim3 grid(xcd_grid((a.T + BM - 1) / BM, a.Hq / a.Hkv, a.Hkv * a.B));
+    const int nqb = (a.T + BM - 1) / BM;
+    const bool paired = a.causal && a.window == 0;
+    dim3 grid(xcd_grid(paired ? (nqb + 1) / 2 : nqb, a.Hq / a.Hkv, a.Hkv * a.B));
     hipLaunchKernelGGL((mfma_fwd<D, NQ, OCC>), grid, dim3(256), 0, st, a);
     PK_HIP(hipGetLastError());
     return PK_OK;
@@ -282,6 +311,9 @@ bool mfma_supported(const AttnArgs& a) {
 int launch_mfma_fwd(const AttnArgs& a0, hipStream_t st) {
     AttnArgs a = a0;
     a.lazy_t = getenv("PK_LAZY_T") ? atof(getenv("PK_LAZY_T")) : LAZY_T;
+#ifdef PK_TIMING
+    if (getenv("PK_DBG_PTR")) a.delta = reinterpret_cast<float*>(strtoull(getenv("PK_DBG_PTR"), nullptr, 0));
+#endif
     // Two 32-query blocks per wavefront halve the LDS traffic per MFMA; short
     // sequences keep one so that the grid still covers the chip.
     static const int variant = getenv("PK_FWD_VARIANT") ? atoi(getenv("PK_FWD_VARIANT")) : 0;
