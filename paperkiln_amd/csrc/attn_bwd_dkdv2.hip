@@ -1,0 +1,326 @@
+// dK / dV of the recompute backward, second generation (see attn_bwd_mfma.hip
+// for the mathematics and the operand layouts).
+//
+// Measured: the one-wavefront-per-SIMD kernel that keeps K, V, dK^T and dV^T
+// of 32 keys in one wavefront's registers leaves the matrix pipe idle while
+// that wavefront does its exp2 / LDS work, and cannot be run two per SIMD
+// (it needs > 256 registers). Here the work of one 32-key block is split
+// between TWO wavefronts that share a SIMD:
+//
+//   role 0 (wavefronts 0-3):  S = Q K^T -> P = exp2(S*c - LSE) -> dV^T += dO^T P
+//   role 1 (wavefronts 4-7):  dP = dO V^T -> dS = P .* (dP - delta) -> dK^T += Q^T dS
+//
+// Each holds one operand (K or V) and one accumulator (dV^T or dK^T): ~180
+// registers, two wavefronts per SIMD, 16 MFMAs each per 32 x 32 block, no
+// recomputation. P goes from role 0 to role 1 through LDS as packed fp16 pairs in
+// the accumulator's own element order (lane-private 32 bytes, conflict-free). Role 1
+// runs ONE STEP BEHIND role 0, so the hand-over needs no extra barrier: the
+// step barrier that publishes the next Q / dO tile also publishes P.
+//
+// Step = 64 queries of one query head. Q / dO tiles sit in a three-deep LDS
+// ring (role 0 reads step s, role 1 step s-1, step s+1 is being stored).
+#include <cstdlib>
+
+#include "mfma_common.h"
+#include "pk_internal.h"
+
+namespace pk {
+namespace {
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr int BMQ = 64;   // queries per step
+constexpr int BNK = 128;  // keys per workgroup (4 blocks of 32)
+typedef __fp16 h16x2 __attribute__((ext_vector_type(2)));
+
+template <bool F32>
+__device__ inline void store4g(void* base, int64_t idx, float x0, float x1, float x2, float x3) {
+    if (F32) {
+        f32x4 v = {x0, x1, x2, x3};
+        *reinterpret_cast<f32x4*>(static_cast<float*>(base) + idx) = v;
+    } else {
+        u32x2 v = {pack_bf16(x0, x1), pack_bf16(x2, x3)};
+        *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(base) + idx) = v;
+    }
+}
+
+template <int D, bool GF32>
+__global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
+    constexpr int KK = D / 16, DB = D / 32;
+    constexpr int S = D + 8;            // tile row pitch (elements): 16-byte row reads conflict-free
+    constexpr int NCH = D / 8;          // 16-byte chunks per row
+    constexpr int CPT = BMQ * NCH / 512;  // chunks per thread per tensor per step
+    __shared__ __attribute__((aligned(16))) uint16_t Qs[3][BMQ * S];
+    __shared__ __attribute__((aligned(16))) uint16_t dOs[3][BMQ * S];
+    __shared__ __attribute__((aligned(16))) uint16_t Pbuf[2][2][4][64 * 16];  // [step parity][query block][key block][lane][16]
+    __shared__ __attribute__((aligned(16))) float nlse_s[3][BMQ];            // -LSE * log2(e)
+    __shared__ __attribute__((aligned(16))) float dl_s[3][BMQ];
+
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int role = w >> 2, kbw = w & 3;
+    const int g = lane >> 5, c32 = lane & 31;
+    const int nkb = (a.T + BNK - 1) / BNK, rep = a.Hq / a.Hkv;
+    // Full-causal: key block i is seen by T - 128i queries; blocks i and nkb-1-i
+    // are taken back to back so that every workgroup carries the same work.
+    const bool paired = a.causal && a.window == 0;
+    int blk, rr, kvu;
+    if (!xcd_map(paired ? (nkb + 1) / 2 : nkb, 1, a.Hkv * a.B, blk, rr, kvu)) return;
+    const int hk = kvu % a.Hkv, b = kvu / a.Hkv;
+    const float cexp = a.scale * LOG2E;
+    const int npass = (paired && blk != nkb - 1 - blk) ? 2 : 1;
+
+    for (int pass = 0; pass < npass; ++pass) {
+        const int kblk = pass == 0 ? blk : nkb - 1 - blk;  // heavy block first
+        const int k0 = kblk * BNK;
+        const int kw0 = k0 + kbw * 32;  // this wavefront's 32 keys
+        const int kj = kw0 + c32;
+
+        // The wavefront's resident operand: K for role 0, V for role 1 (B operand,
+        // lane = key, chunk kk covers d = 16kk + 8g .. +7). Keys past the end
+        // re-read the last row; their P is masked to zero and nothing is stored.
+        bf16x8 kv[KK];
+        {
+            const void* src = role == 0 ? a.k : a.v;
+            const int64_t off = role == 0 ? b * a.k_sb + hk * a.k_sh : b * a.v_sb + hk * a.v_sh;
+            const int64_t st = role == 0 ? a.k_st : a.v_st;
+            const int t = min(kj, a.T - 1);
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+                const u32x4 z = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(src) + off + t * st +
+                                                                kk * 16 + g * 8);
+                kv[kk] = *reinterpret_cast<const bf16x8*>(&z);
+            }
+        }
+        f32x16 acc[DB];  // dV^T (role 0) or dK^T (role 1)
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[db][r] = 0.0f;
+        const KeyVis kvis(kj, a.T, a.causal, a.window, a.sinks);
+
+        // Query tiles that can see keys [k0, k0+127] (paperkiln src/ops.cpp:960-965 inverted).
+        const int khi = min(k0 + BNK, a.T) - 1;
+        const int qt_lo = a.causal ? k0 / BMQ : 0;
+        const int qt_hi = (a.window > 0 && k0 >= a.sinks) ? min(a.T - 1, khi + a.window - 1) / BMQ : (a.T - 1) / BMQ;
+        const int nqt = qt_hi - qt_lo + 1;
+        const int steps = nqt * rep;
+
+        u32x4 qr[CPT], gr[CPT];
+        float lse_r = 0.0f, dl_r = 0.0f;
+        auto fetch = [&](int step) {  // global -> registers, rows past the end clamped
+            const int h = hk * rep + step / nqt, q0 = (qt_lo + step % nqt) * BMQ;
+#pragma unroll
+            for (int i = 0; i < CPT; ++i) {
+                const int c = threadIdx.x + 512 * i;
+                const int row = c / NCH, ch = c % NCH;
+                const int t = min(q0 + row, a.T - 1);
+                qr[i] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.q) + b * a.q_sb + h * a.q_sh +
+                                                        t * a.q_st + ch * 8);
+                gr[i] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.d_o) + b * a.do_sb +
+                                                        h * a.do_sh + t * a.do_st + ch * 8);
+            }
+            if (threadIdx.x < BMQ) {
+                const int t = min(q0 + static_cast<int>(threadIdx.x), a.T - 1);
+                const int64_t lrow = (static_cast<int64_t>(b) * a.Hq + h) * a.T + t;
+                lse_r = -a.lse[lrow] * LOG2E;
+                dl_r = a.delta[lrow];
+            }
+        };
+        auto commit = [&](int slot) {  // registers -> LDS ring slot
+#pragma unroll
+            for (int i = 0; i < CPT; ++i) {
+                const int c = threadIdx.x + 512 * i;
+                const int row = c / NCH, ch = c % NCH;
+                *reinterpret_cast<u32x4*>(Qs[slot] + row * S + ch * 8) = qr[i];
+                *reinterpret_cast<u32x4*>(dOs[slot] + row * S + ch * 8) = gr[i];
+            }
+            if (threadIdx.x < BMQ) {
+                nlse_s[slot][threadIdx.x] = lse_r;
+                dl_s[slot][threadIdx.x] = dl_r;
+            }
+        };
+        // wavefront-uniform: is anything of (query block qb of step `step`) x (this key block) visible?
+        auto block_live = [&](int step, int qb, int& qlo) {
+            qlo = (qt_lo + step % nqt) * BMQ + qb * 32;
+            const int qhi = qlo + 31;
+            if (qlo >= a.T || kw0 >= a.T) return false;
+            if (a.causal && kw0 > qhi) return false;
+            if (a.window > 0 && kw0 + 31 + a.window <= qlo && kw0 >= a.sinks) return false;
+            return true;
+        };
+
+        if (steps > 0) {
+            fetch(0);
+            commit(0);
+            if (steps > 1) fetch(1);
+        }
+        __syncthreads();
+
+#ifdef PK_TIMING
+        long long tacc[4] = {0, 0, 0, 0};
+        long long tprev = __builtin_readcyclecounter();
+#define PK_TICK(i) { long long now = __builtin_readcyclecounter(); tacc[i] += now - tprev; tprev = now; }
+#else
+#define PK_TICK(i)
+#endif
+        // iteration s: role 0 works on step s, role 1 on step s-1
+        for (int s = 0; s <= steps; ++s) {
+            PK_TICK(3)
+            if (s + 1 < steps) {
+                commit((s + 1) % 3);  // slot last read (by role 1) before the previous barrier
+                if (s + 2 < steps) fetch(s + 2);
+            }
+            PK_TICK(0)
+            if (role == 0) {
+                if (s < steps) {
+                    const uint16_t* Qt = Qs[s % 3];
+                    const uint16_t* Gt = dOs[s % 3];
+#pragma unroll
+                    for (int qb = 0; qb < 2; ++qb) {
+                        int qlo;
+                        if (!block_live(s, qb, qlo)) continue;
+                        // two accumulator chains (even / odd k-chunks): a dependent MFMA pair
+                        // costs 52 cycles, an independent one 32
+                        f32x16 sc, sc2;
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) sc[r] = sc2[r] = 0.0f;
+#pragma unroll
+                        for (int kk = 0; kk < KK; kk += 2) {
+                            sc = mfma32(lds_read8(Qt + (qb * 32 + c32) * S + kk * 16 + g * 8), kv[kk], sc);
+                            sc2 = mfma32(lds_read8(Qt + (qb * 32 + c32) * S + (kk + 1) * 16 + g * 8), kv[kk + 1], sc2);
+                        }
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) sc[r] += sc2[r];
+                        const int qhi = qlo + 31;
+                        const bool full = qhi < a.T && kw0 + 31 < a.T && (!a.causal || kw0 + 31 <= qlo) &&
+                                          (a.window == 0 || kw0 + a.window > qhi || kw0 + 31 < a.sinks);
+                        // lane = key kj; element r = query qlo + (r/4)*8 + 4g + r%4
+#pragma unroll
+                        for (int qd = 0; qd < 4; ++qd) {
+                            const f32x4 nl = *reinterpret_cast<const f32x4*>(&nlse_s[s % 3][qb * 32 + qd * 8 + g * 4]);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                float p = __builtin_amdgcn_exp2f(fmaf(sc[qd * 4 + e], cexp, nl[e]));
+                                if (!full) p = kvis(qlo + qd * 8 + g * 4 + e) ? p : 0.0f;
+                                sc[qd * 4 + e] = p;
+                            }
+                        }
+                        const bf16x8 p0 = c_to_operand<0>(sc), p1 = c_to_operand<1>(sc);
+                        // hand-over copy in fp16: P is in [0, 1], where fp16 carries 11 significant
+                        // bits against bf16's 8, so dS is built from a P as good as the old fp32 one
+                        uint16_t* pb = Pbuf[s & 1][qb][kbw] + lane * 16;
+                        h16x2 ph[8];
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) {
+                            const f32x2 pr = {sc[2 * i], sc[2 * i + 1]};
+                            ph[i] = __builtin_convertvector(pr, h16x2);  // round to nearest even
+                        }
+                        *reinterpret_cast<u32x4*>(pb) = *reinterpret_cast<u32x4*>(&ph[0]);
+                        *reinterpret_cast<u32x4*>(pb + 8) = *reinterpret_cast<u32x4*>(&ph[4]);
+                        // dV^T += dO^T P
+#pragma unroll
+                        for (int db = 0; db < DB; ++db)
+                            acc[db] = mfma32(lds_read_tr_operand_perm<D>(Gt, S, qb * 32, db, lane), p0, acc[db]);
+#pragma unroll
+                        for (int db = 0; db < DB; ++db)
+                            acc[db] = mfma32(lds_read_tr_operand_perm<D>(Gt, S, qb * 32 + 16, db, lane), p1, acc[db]);
+                    }
+                }
+            } else {
+                if (s >= 1) {
+                    const int sp = s - 1;
+                    const uint16_t* Qt = Qs[sp % 3];
+                    const uint16_t* Gt = dOs[sp % 3];
+#pragma unroll
+                    for (int qb = 0; qb < 2; ++qb) {
+                        int qlo;
+                        if (!block_live(sp, qb, qlo)) continue;
+                        f32x16 dp, dp2;
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) dp[r] = dp2[r] = 0.0f;
+#pragma unroll
+                        for (int kk = 0; kk < KK; kk += 2) {
+                            dp = mfma32(lds_read8(Gt + (qb * 32 + c32) * S + kk * 16 + g * 8), kv[kk], dp);
+                            dp2 = mfma32(lds_read8(Gt + (qb * 32 + c32) * S + (kk + 1) * 16 + g * 8), kv[kk + 1], dp2);
+                        }
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) dp[r] += dp2[r];
+                        const uint16_t* pb = Pbuf[sp & 1][qb][kbw] + lane * 16;
+                        u32x4 praw[2];
+                        praw[0] = *reinterpret_cast<const u32x4*>(pb);
+                        praw[1] = *reinterpret_cast<const u32x4*>(pb + 8);
+                        const h16x2* ph = reinterpret_cast<const h16x2*>(praw);
+                        // dS = P .* (dP - delta); P arrives as fp16 pairs of elements (2i, 2i+1)
+#pragma unroll
+                        for (int qd = 0; qd < 4; ++qd) {
+                            const f32x4 dl = *reinterpret_cast<const f32x4*>(&dl_s[sp % 3][qb * 32 + qd * 8 + g * 4]);
+                            dp[qd * 4 + 0] = static_cast<float>(ph[2 * qd][0]) * (dp[qd * 4 + 0] - dl[0]);
+                            dp[qd * 4 + 1] = static_cast<float>(ph[2 * qd][1]) * (dp[qd * 4 + 1] - dl[1]);
+                            dp[qd * 4 + 2] = static_cast<float>(ph[2 * qd + 1][0]) * (dp[qd * 4 + 2] - dl[2]);
+                            dp[qd * 4 + 3] = static_cast<float>(ph[2 * qd + 1][1]) * (dp[qd * 4 + 3] - dl[3]);
+                        }
+                        const bf16x8 d0 = c_to_operand<0>(dp), d1 = c_to_operand<1>(dp);
+                        // dK^T += Q^T dS
+#pragma unroll
+                        for (int db = 0; db < DB; ++db)
+                            acc[db] = mfma32(lds_read_tr_operand_perm<D>(Qt, S, qb * 32, db, lane), d0, acc[db]);
+#pragma unroll
+                        for (int db = 0; db < DB; ++db)
+                            acc[db] = mfma32(lds_read_tr_operand_perm<D>(Qt, S, qb * 32 + 16, db, lane), d1, acc[db]);
+                    }
+                }
+            }
+            PK_TICK(1)
+            __syncthreads();
+            PK_TICK(2)
+        }
+#ifdef PK_TIMING
+        if (a.lazy_t != 0.0f && lane == 0) {
+            long long* dbg = reinterpret_cast<long long*>(a.dq) + (static_cast<long long>(blockIdx.x) * 8 + w) * 8;
+            for (int q = 0; q < 4; ++q) dbg[q] += tacc[q];
+            dbg[4] += steps;
+        }
+#endif
+
+        if (kj < a.T) {
+            void* dst = role == 0 ? a.dv : a.dk;
+            const int64_t ob = role == 0 ? b * a.dv_sb + hk * a.dv_sh + kj * a.dv_st
+                                         : b * a.dk_sb + hk * a.dk_sh + kj * a.dk_st;
+            const float sc = role == 0 ? 1.0f : a.scale;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int qd = 0; qd < 4; ++qd)
+                    store4g<GF32>(dst, ob + TrMap<D>::col0(db, qd, g), acc[db][qd * 4] * sc, acc[db][qd * 4 + 1] * sc,
+                                  acc[db][qd * 4 + 2] * sc, acc[db][qd * 4 + 3] * sc);
+        }
+        __syncthreads();  // the next pass refills the ring
+    }
+}
+
+template <int D, bool GF32>
+int launch(const AttnArgs& a, hipStream_t st) {
+    const int nb128 = (a.T + 127) / 128;
+    const bool paired = a.causal && a.window == 0;
+    hipLaunchKernelGGL((mfma_dkdv2<D, GF32>), dim3(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, 1, a.Hkv * a.B)),
+                       dim3(512), 0, st, a);
+    PK_HIP(hipGetLastError());
+    return PK_OK;
+}
+
+}  // namespace
+
+int launch_mfma_dkdv2(const AttnArgs& a0, hipStream_t st) {
+    AttnArgs a = a0;
+    a.lazy_t = 0.0f;
+#ifdef PK_TIMING
+    // timing build only: the dq pointer (unused by this kernel) carries the debug buffer
+    if (getenv("PK_DBG_PTR")) {
+        a.dq = reinterpret_cast<void*>(strtoull(getenv("PK_DBG_PTR"), nullptr, 0));
+        a.lazy_t = 1.0f;
+    }
+#endif
+    if (a.dk_dim == 128) return a.grad_f32 ? launch<128, true>(a, st) : launch<128, false>(a, st);
+    return a.grad_f32 ? launch<64, true>(a, st) : launch<64, false>(a, st);
+}
+
+}  // namespace pk

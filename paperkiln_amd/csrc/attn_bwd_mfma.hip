@@ -22,6 +22,8 @@
 //                 wavefront, Q and dO in registers), loops over the visible
 //                 key tiles: S^T = K Q^T, dP^T = V dO^T (lane = query, so LSE
 //                 and delta are per-lane scalars), dQ^T += K^T dS^T.
+#include <cstdlib>
+
 #include "mfma_common.h"
 #include "pk_internal.h"
 
@@ -392,7 +394,10 @@ int launch(const AttnArgs& a, int stages, hipStream_t st) {
         hipLaunchKernelGGL((mfma_delta<D>), dim3((rows + RPB - 1) / RPB), dim3(256), 0, st, a);
         PK_HIP(hipGetLastError());
     }
-    if (stages & PK_BWD_DKDV) {
+    static const bool old_dkdv = getenv("PK_DKDV_OLD") != nullptr;
+    if ((stages & PK_BWD_DKDV) && !old_dkdv) {
+        if (int rc = launch_mfma_dkdv2(a, st)) return rc;
+    } else if (stages & PK_BWD_DKDV) {
         hipLaunchKernelGGL((mfma_dkdv<D, GF32>), dim3(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, 1, a.Hkv * a.B)), dim3(256),
                            0, st, a);
         PK_HIP(hipGetLastError());

@@ -69,5 +69,6 @@ bool mfma_supported(const AttnArgs& a);
 int launch_mfma_fwd(const AttnArgs& a, hipStream_t st);
 int launch_mfma_fwd_pipe(const AttnArgs& a, hipStream_t st);
 int launch_mfma_bwd(const AttnArgs& a, int stages, hipStream_t st);
+int launch_mfma_dkdv2(const AttnArgs& a, hipStream_t st);
 
 }  // namespace pk
