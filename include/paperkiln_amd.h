@@ -99,6 +99,60 @@ int pk_attn_bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_ten
                        const pk_tensor4* dv, void* workspace, size_t workspace_bytes, int stages,
                        void* stream);
 
+/* ---- device memory ------------------------------------------------------
+ * Caching allocator with a byte-level high-water mark: the HIP counterpart of
+ * the per-call cudaMalloc/cudaFree in src/cuda_resident.cu:226-263 and
+ * src/cuda_ops.cu:63-72, and the byte receipt that the reference's
+ * live_variables() (include/microtorch/autograd.hpp:61-64) cannot give. */
+int pk_alloc(size_t bytes, void** out);
+int pk_free(void* p);
+size_t pk_live_bytes(void);
+size_t pk_peak_bytes(void);
+void pk_reset_peak(void);
+void pk_trim(void);
+
+/* ---- activation-checkpointed Llama step ---------------------------------
+ * nn::Llama (include/microtorch/llama.hpp:14-51, src/llama.cpp) on the
+ * device-resident tape. Parameters are fp32 master copies named exactly as the
+ * reference names them ("layers.N.self_attn.q_proj.weight", ...; Linear
+ * weights are [in, out], y = x W). compute_dtype PK_BF16 runs activations and
+ * GEMM operands in bf16 with fp32 accumulation. */
+typedef struct pk_llama_config {
+    int32_t vocab, d, n_layers, n_heads, d_ff;
+    float rope_theta;
+    int32_t tie_embeddings;  /* must be 1: the tied head of llama.cpp:88 */
+    int32_t compute_dtype;   /* PK_F32 | PK_BF16 */
+    int32_t rope_all_heads;  /* 0 = the reference as written: apply_rope(concat, pos, theta, dk) rotates only
+                                the first head of q and of k (src/ops.cpp:498-499, called at llama.cpp:36) */
+    int32_t window, sinks;   /* 0,0 = causal fused_attention; window>=1 = swa_attention in every block */
+} pk_llama_config;
+
+typedef struct pk_llama_stats {
+    int64_t live_vars_after_forward;        /* the reference's receipt (tests/test_checkpointing.cpp:46-60) */
+    int64_t activation_bytes_after_forward; /* allocator bytes held by the tape between forward and backward */
+    int64_t peak_activation_bytes;          /* high-water mark over forward + backward, parameters, gradients,
+                                               optimizer state and bf16 parameter shadows excluded */
+} pk_llama_stats;
+
+/* Llama::Llama(cfg, seed): N(0, 0.02) Linear / Embedding weights, unit norm gains. */
+int pk_llama_create(const pk_llama_config* cfg, unsigned seed, void** handle);
+int pk_llama_destroy(void* handle);
+int pk_llama_num_params(void* handle);
+int pk_llama_param_info(void* handle, int i, char* name, size_t name_len, int64_t* rows, int64_t* cols);
+int pk_llama_set_param(void* handle, int i, const float* host);
+int pk_llama_get_param(void* handle, int i, float* host);
+int pk_llama_get_grad(void* handle, int i, float* host);
+/* zero_grad -> forward -> mean cross-entropy -> backward: the step of tools/mtstudio.cpp:456-471.
+ * ids/targets are host arrays of n tokens, B = n/seq_len stacked sequences (seq_len 0 = one).
+ * checkpoint_blocks: Llama::checkpoint_blocks (llama.hpp:45). fused_head 1 evaluates the tied head
+ * and the loss in row chunks (no [n, vocab] matrix); 0 materialises the logits as the reference does. */
+int pk_llama_loss_backward(void* handle, const int* host_ids, const int* host_targets, int64_t n, int64_t seq_len,
+                           int checkpoint_blocks, int do_backward, int fused_head, float* loss,
+                           pk_llama_stats* stats, void* stream);
+/* ops::clip_grad_norm (src/ops.cpp:1046-1064; skipped when max_norm <= 0) then nn::AdamW::step (src/nn.cpp:301-321). */
+int pk_llama_adamw_step(void* handle, float lr, float b1, float b2, float eps, float wd, float max_norm,
+                        float* total_norm);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,6 +25,18 @@ class AttnShape(C.Structure):
                 ("dtype", C.c_int32), ("grad_dtype", C.c_int32)]
 
 
+class LlamaConfig(C.Structure):
+    _fields_ = [("vocab", C.c_int32), ("d", C.c_int32), ("n_layers", C.c_int32), ("n_heads", C.c_int32),
+                ("d_ff", C.c_int32), ("rope_theta", C.c_float), ("tie_embeddings", C.c_int32),
+                ("compute_dtype", C.c_int32), ("rope_all_heads", C.c_int32), ("window", C.c_int32),
+                ("sinks", C.c_int32)]
+
+
+class LlamaStats(C.Structure):
+    _fields_ = [("live_vars_after_forward", C.c_int64), ("activation_bytes_after_forward", C.c_int64),
+                ("peak_activation_bytes", C.c_int64)]
+
+
 class PkError(RuntimeError):
     def __init__(self, code: int, msg: str):
         super().__init__(f"paperkiln_amd error {code}: {msg}")
@@ -34,7 +46,10 @@ class PkError(RuntimeError):
 _lib = None
 
 # every symbol include/paperkiln_amd.h declares
-EXPORTS = ["pk_last_error", "pk_init", "pk_attn_fwd", "pk_attn_bwd_workspace_bytes", "pk_attn_bwd", "pk_attn_bwd_stages"]
+EXPORTS = ["pk_last_error", "pk_init", "pk_attn_fwd", "pk_attn_bwd_workspace_bytes", "pk_attn_bwd", "pk_attn_bwd_stages",
+           "pk_alloc", "pk_free", "pk_live_bytes", "pk_peak_bytes", "pk_reset_peak", "pk_trim",
+           "pk_llama_create", "pk_llama_destroy", "pk_llama_num_params", "pk_llama_param_info", "pk_llama_set_param",
+           "pk_llama_get_param", "pk_llama_get_grad", "pk_llama_loss_backward", "pk_llama_adamw_step"]
 
 
 def lib() -> C.CDLL:
@@ -54,6 +69,24 @@ def lib() -> C.CDLL:
         L.pk_attn_bwd.argtypes = [SH, T4, T4, T4, T4, C.c_void_p, T4, T4, T4, T4, C.c_void_p, C.c_size_t, C.c_void_p]
         L.pk_attn_bwd_stages.argtypes = [SH, T4, T4, T4, T4, C.c_void_p, T4, T4, T4, T4, C.c_void_p, C.c_size_t,
                                          C.c_int, C.c_void_p]
+        f32p, i32p = C.POINTER(C.c_float), C.POINTER(C.c_int)
+        L.pk_alloc.argtypes = [C.c_size_t, C.POINTER(C.c_void_p)]
+        L.pk_free.argtypes = [C.c_void_p]
+        for fn in (L.pk_live_bytes, L.pk_peak_bytes):
+            fn.restype = C.c_size_t
+        L.pk_reset_peak.restype = None
+        L.pk_trim.restype = None
+        L.pk_llama_create.argtypes = [C.POINTER(LlamaConfig), C.c_uint, C.POINTER(C.c_void_p)]
+        L.pk_llama_destroy.argtypes = [C.c_void_p]
+        L.pk_llama_num_params.argtypes = [C.c_void_p]
+        L.pk_llama_param_info.argtypes = [C.c_void_p, C.c_int, C.c_char_p, C.c_size_t, C.POINTER(C.c_int64),
+                                          C.POINTER(C.c_int64)]
+        L.pk_llama_set_param.argtypes = [C.c_void_p, C.c_int, f32p]
+        L.pk_llama_get_param.argtypes = [C.c_void_p, C.c_int, f32p]
+        L.pk_llama_get_grad.argtypes = [C.c_void_p, C.c_int, f32p]
+        L.pk_llama_loss_backward.argtypes = [C.c_void_p, i32p, i32p, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int,
+                                             f32p, C.POINTER(LlamaStats), C.c_void_p]
+        L.pk_llama_adamw_step.argtypes = [C.c_void_p] + [C.c_float] * 6 + [f32p]
         _lib = L
     return _lib
 

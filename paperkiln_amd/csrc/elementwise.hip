@@ -1,0 +1,508 @@
+// Allocator, elementwise / rowwise kernels and the GEMM wrapper behind the
+// host-side tape. They stand where the reference's device op set does
+// (paperkiln src/cuda_ops.cu:76-381, write-through host->device->host per call)
+// but are device-resident: operands and results stay in HBM between ops.
+// Formulas are those of the CPU tape in src/ops.cpp, cited per kernel.
+#include <rocblas/rocblas.h>
+
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "tensor.h"
+
+namespace pk {
+
+void hip_check(hipError_t e, const char* what) {
+    if (e != hipSuccess) throw std::runtime_error(std::string("HIP error: ") + hipGetErrorString(e) + " in " + what);
+}
+#define HIPCHK(x) ::pk::hip_check((x), #x)
+
+// ---- allocator -------------------------------------------------------------
+namespace {
+struct Pool {
+    std::mutex mu;
+    std::multimap<size_t, void*> free_blocks;         // size -> block
+    std::unordered_map<void*, size_t> sizes;          // every block handed out or cached
+    size_t live = 0, peak = 0, reserved = 0;
+};
+Pool& pool() {
+    static Pool p;
+    return p;
+}
+size_t round_up(size_t n) {
+    if (n < 512) return 512;
+    if (n < (1u << 20)) return (n + 511) & ~size_t(511);
+    return (n + ((1u << 20) - 1)) & ~size_t((1u << 20) - 1);  // 1 MiB granules above 1 MiB
+}
+hipStream_t g_stream = nullptr;
+}  // namespace
+
+hipStream_t tape_stream() { return g_stream; }
+void set_tape_stream(hipStream_t s) { g_stream = s; }
+
+void* dev_alloc(size_t bytes) {
+    const size_t n = round_up(bytes);
+    Pool& P = pool();
+    std::lock_guard<std::mutex> lk(P.mu);
+    void* p = nullptr;
+    auto it = P.free_blocks.lower_bound(n);
+    if (it != P.free_blocks.end() && it->first <= n + n / 4 + 512) {  // reuse only near-fitting blocks
+        p = it->second;
+        P.live += it->first;
+        P.free_blocks.erase(it);
+    } else {
+        hipError_t e = hipMalloc(&p, n);
+        if (e != hipSuccess) {  // give cached blocks back and retry once
+            for (auto& kv : P.free_blocks) {
+                (void)hipFree(kv.second);
+                P.reserved -= kv.first;
+                P.sizes.erase(kv.second);
+            }
+            P.free_blocks.clear();
+            hip_check(hipMalloc(&p, n), "hipMalloc");
+        }
+        P.sizes[p] = n;
+        P.reserved += n;
+        P.live += n;
+    }
+    if (P.live > P.peak) P.peak = P.live;
+    return p;
+}
+
+void dev_free(void* p) {
+    if (!p) return;
+    Pool& P = pool();
+    std::lock_guard<std::mutex> lk(P.mu);
+    auto it = P.sizes.find(p);
+    if (it == P.sizes.end()) return;
+    P.live -= it->second;
+    P.free_blocks.emplace(it->second, p);
+}
+
+size_t dev_live_bytes() { return pool().live; }
+size_t dev_peak_bytes() { return pool().peak; }
+void dev_reset_peak() { pool().peak = pool().live; }
+void dev_trim() {
+    Pool& P = pool();
+    std::lock_guard<std::mutex> lk(P.mu);
+    (void)hipDeviceSynchronize();
+    for (auto& kv : P.free_blocks) {
+        (void)hipFree(kv.second);
+        P.reserved -= kv.first;
+        P.sizes.erase(kv.second);
+    }
+    P.free_blocks.clear();
+}
+
+// ---- element access --------------------------------------------------------
+namespace {
+
+__device__ inline float ldf(const float* p, int64_t i) { return p[i]; }
+__device__ inline float ldf(const uint16_t* p, int64_t i) { return __uint_as_float(static_cast<uint32_t>(p[i]) << 16); }
+__device__ inline void stf(float* p, int64_t i, float x) { p[i] = x; }
+__device__ inline void stf(uint16_t* p, int64_t i, float x) {
+    uint32_t u = __float_as_uint(x);
+    u += 0x7FFFu + ((u >> 16) & 1u);  // round to nearest even
+    p[i] = static_cast<uint16_t>(u >> 16);
+}
+
+constexpr int NT = 256;
+inline dim3 ew_grid(int64_t n) { return dim3(static_cast<unsigned>(std::min<int64_t>((n + NT - 1) / NT, 65535 * 16))); }
+
+// dispatch one or two storage types
+#define PK_DISPATCH1(T_, dt, ...)               \
+    if ((dt) == PK_F32) {                       \
+        using T_ = float;                       \
+        __VA_ARGS__;                            \
+    } else {                                    \
+        using T_ = uint16_t;                    \
+        __VA_ARGS__;                            \
+    }
+
+template <typename TA, typename TB, typename TY, int OP>
+__global__ void ew_binary(const TA* a, const TB* b, TY* y, int64_t n) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT) {
+        const float x = ldf(a, i), z = ldf(b, i);
+        stf(y, i, OP == 0 ? x + z : x * z);
+    }
+}
+template <typename TA, typename TY>
+__global__ void ew_scale(const TA* a, float s, TY* y, int64_t n) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT)
+        stf(y, i, ldf(a, i) * s);
+}
+template <typename TY, typename TX>
+__global__ void ew_axpy(TY* y, float a, const TX* x, int64_t n) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT)
+        stf(y, i, ldf(y, i) + a * ldf(x, i));
+}
+template <typename TY>
+__global__ void ew_fill(TY* y, float v, int64_t n) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT)
+        stf(y, i, v);
+}
+template <typename T>
+__global__ void ew_silu_fwd(const T* x, T* y, int64_t n) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT) {
+        const float v = ldf(x, i);
+        stf(y, i, v / (1.0f + expf(-v)));  // ops.cpp:409
+    }
+}
+template <typename T>
+__global__ void ew_silu_bwd(const T* x, const T* dy, T* dx, int64_t n) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT) {
+        const float v = ldf(x, i);
+        const float s = 1.0f / (1.0f + expf(-v));
+        stf(dx, i, ldf(dy, i) * s * (1.0f + v * (1.0f - s)));  // ops.cpp:419-420
+    }
+}
+
+__device__ inline float wave_sum(float x) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) x += __shfl_xor(x, o, 64);
+    return x;
+}
+
+// One wavefront per row. y = x * rinv * w, rinv = 1/sqrt(mean(x^2) + eps).
+template <typename T>
+__global__ void rms_fwd(const T* x, const float* w, float eps, T* y, float* rinv, int64_t R, int C) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= R) return;
+    const T* xr = x + row * C;
+    float ss = 0.0f;
+    for (int j = lane; j < C; j += 64) {
+        const float v = ldf(xr, j);
+        ss = fmaf(v, v, ss);
+    }
+    ss = wave_sum(ss) / static_cast<float>(C);
+    const float ri = 1.0f / sqrtf(ss + eps);
+    if (lane == 0) rinv[row] = ri;
+    for (int j = lane; j < C; j += 64) stf(y + row * C, j, ldf(xr, j) * ri * w[j]);
+}
+// dx = rinv * (dY*w - x * rinv^2 * sum_j(dY*w*x) / C)
+template <typename T>
+__global__ void rms_bwd_dx(const T* dy, const T* x, const float* rinv, const float* w, T* dx, int64_t R, int C) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= R) return;
+    const T* xr = x + row * C;
+    const T* gr = dy + row * C;
+    float term = 0.0f;
+    for (int j = lane; j < C; j += 64) term = fmaf(ldf(gr, j) * w[j], ldf(xr, j), term);
+    term = wave_sum(term);
+    const float ri = rinv[row], k = ri * ri * term / static_cast<float>(C);
+    for (int j = lane; j < C; j += 64) stf(dx + row * C, j, ri * (ldf(gr, j) * w[j] - ldf(xr, j) * k));
+}
+// dw_j = sum_i dY_ij x_ij rinv_i, in two deterministic stages: each block sums
+// ROWS_PB rows into part[block][C], then one block per column chunk adds the parts.
+constexpr int ROWS_PB = 128;
+template <typename T>
+__global__ void rms_bwd_dw_part(const T* dy, const T* x, const float* rinv, float* part, int64_t R, int C) {
+    const int64_t r0 = static_cast<int64_t>(blockIdx.x) * ROWS_PB;
+    for (int j = threadIdx.x; j < C; j += NT) {
+        float s = 0.0f;
+        for (int64_t i = r0; i < min(r0 + ROWS_PB, R); ++i) s = fmaf(ldf(dy, i * C + j) * ldf(x, i * C + j), rinv[i], s);
+        part[static_cast<int64_t>(blockIdx.x) * C + j] = s;
+    }
+}
+__global__ void colsum_parts(const float* part, float* dw, int nparts, int C) {
+    const int j = blockIdx.x * NT + threadIdx.x;
+    if (j >= C) return;
+    float s = 0.0f;
+    for (int p = 0; p < nparts; ++p) s += part[static_cast<int64_t>(p) * C + j];
+    dw[j] += s;
+}
+
+// apply_rope (ops.cpp:497-509 forward, :519-533 backward = rotation by -theta).
+template <typename T>
+__global__ void rope_k(const T* x, const int* pos, float theta_base, int d, int head_dim, int rot_heads, float sign,
+                       T* y, int64_t N) {
+    const int d3 = 3 * d;
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < N * (d3 / 2);
+         i += static_cast<int64_t>(gridDim.x) * NT) {
+        const int64_t row = i / (d3 / 2);
+        const int c = static_cast<int>(i % (d3 / 2)) * 2;  // even column of the pair
+        const int third = c / d, within = c % d;
+        float x0 = ldf(x, row * d3 + c), x1 = ldf(x, row * d3 + c + 1);
+        if (third < 2 && within < rot_heads * head_dim) {
+            const int dim = within % head_dim;
+            const float inv_freq = 1.0f / powf(theta_base, static_cast<float>(dim) / head_dim);
+            const float th = sign * static_cast<float>(pos[row]) * inv_freq;
+            const float c_ = cosf(th), s_ = sinf(th);
+            const float r0 = x0 * c_ - x1 * s_, r1 = x0 * s_ + x1 * c_;
+            x0 = r0;
+            x1 = r1;
+        }
+        stf(y, row * d3 + c, x0);
+        stf(y, row * d3 + c + 1, x1);
+    }
+}
+
+template <typename T>
+__global__ void emb_fwd(const float* table, const int* ids, T* y, int64_t n, int d) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n * d; i += static_cast<int64_t>(gridDim.x) * NT)
+        stf(y, i, table[static_cast<int64_t>(ids[i / d]) * d + i % d]);
+}
+template <typename T>
+__global__ void emb_bwd(const T* dy, const int* ids, float* dtable, int64_t n, int d) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n * d; i += static_cast<int64_t>(gridDim.x) * NT)
+        atomicAdd(dtable + static_cast<int64_t>(ids[i / d]) * d + i % d, ldf(dy, i));
+}
+
+__device__ inline float block_reduce(float x, bool is_max, float* sh) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        const float y = __shfl_xor(x, o, 64);
+        x = is_max ? fmaxf(x, y) : x + y;
+    }
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = x;
+    __syncthreads();
+    float r = sh[0];
+    for (int i = 1; i < NT / 64; ++i) r = is_max ? fmaxf(r, sh[i]) : r + sh[i];
+    __syncthreads();
+    return r;
+}
+// One block per row: softmax, nll with the 1e-12 clamp, dlogits in place.
+template <typename T>
+__global__ void ce_rows(T* logits, const int* targets, float gscale, float* nll, int C) {
+    __shared__ float sh[NT / 64];
+    T* row = logits + static_cast<int64_t>(blockIdx.x) * C;
+    const int t = targets[blockIdx.x];
+    const float lt = ldf(row, t);  // read before any thread overwrites the row with dlogits
+    float mx = -INFINITY;
+    for (int j = threadIdx.x; j < C; j += NT) mx = fmaxf(mx, ldf(row, j));
+    mx = block_reduce(mx, true, sh);
+    float z = 0.0f;
+    for (int j = threadIdx.x; j < C; j += NT) z += expf(ldf(row, j) - mx);
+    z = block_reduce(z, false, sh);
+    const float inv = 1.0f / z;
+    if (threadIdx.x == 0) nll[blockIdx.x] = -logf(fmaxf(expf(lt - mx) * inv, 1e-12f));
+    for (int j = threadIdx.x; j < C; j += NT) {
+        const float p = expf(ldf(row, j) - mx) * inv;
+        stf(row, j, (p - (j == t ? 1.0f : 0.0f)) * gscale);
+    }
+}
+
+__global__ void sum_f32_k(const float* x, int64_t n, double* out) {
+    __shared__ double sh[NT];
+    double s = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += NT) s += static_cast<double>(x[i]);
+    sh[threadIdx.x] = s;
+    __syncthreads();
+    for (int o = NT / 2; o >= 1; o >>= 1) {
+        if (threadIdx.x < o) sh[threadIdx.x] += sh[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *out = sh[0];
+}
+__global__ void sumsq_part(const float* x, int64_t n, double* part) {
+    __shared__ double sh[NT];
+    double s = 0.0;
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT)
+        s += static_cast<double>(x[i]) * x[i];
+    sh[threadIdx.x] = s;
+    __syncthreads();
+    for (int o = NT / 2; o >= 1; o >>= 1) {
+        if (threadIdx.x < o) sh[threadIdx.x] += sh[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) part[blockIdx.x] = sh[0];
+}
+__global__ void adamw_k(float* p, const float* g, float* m, float* v, float lr, float b1, float b2, float eps, float wd,
+                        float c1, float c2, int64_t n) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT) {
+        const float gi = g[i];
+        const float mi = b1 * m[i] + (1.0f - b1) * gi;
+        const float vi = b2 * v[i] + (1.0f - b2) * gi * gi;
+        m[i] = mi;
+        v[i] = vi;
+        const float upd = (mi / c1) / (sqrtf(vi / c2) + eps);  // nn.cpp:317
+        p[i] -= lr * (upd + wd * p[i]);
+    }
+}
+
+void same_shape(const Tensor& a, const Tensor& b, const char* who) {
+    if (a.rows != b.rows || a.cols != b.cols) throw std::runtime_error(std::string(who) + ": shape mismatch");
+}
+void post() { HIPCHK(hipGetLastError()); }
+
+}  // namespace
+
+void k_fill(const Tensor& y, float v) {
+    PK_DISPATCH1(T, y.dtype, hipLaunchKernelGGL((ew_fill<T>), ew_grid(y.numel()), dim3(NT), 0, tape_stream(),
+                                                static_cast<T*>(y.ptr()), v, y.numel()));
+    post();
+}
+void k_cast(const Tensor& src, const Tensor& dst) {
+    same_shape(src, dst, "cast");
+    PK_DISPATCH1(TA, src.dtype, PK_DISPATCH1(TY, dst.dtype,
+                 hipLaunchKernelGGL((ew_scale<TA, TY>), ew_grid(src.numel()), dim3(NT), 0, tape_stream(),
+                                    static_cast<const TA*>(src.ptr()), 1.0f, static_cast<TY*>(dst.ptr()), src.numel())));
+    post();
+}
+template <int OP>
+static void binary(const Tensor& a, const Tensor& b, const Tensor& y, const char* who) {
+    same_shape(a, b, who);
+    same_shape(a, y, who);
+    PK_DISPATCH1(TA, a.dtype, PK_DISPATCH1(TB, b.dtype, PK_DISPATCH1(TY, y.dtype,
+                 hipLaunchKernelGGL((ew_binary<TA, TB, TY, OP>), ew_grid(a.numel()), dim3(NT), 0, tape_stream(),
+                                    static_cast<const TA*>(a.ptr()), static_cast<const TB*>(b.ptr()),
+                                    static_cast<TY*>(y.ptr()), a.numel()))));
+    post();
+}
+void k_add(const Tensor& a, const Tensor& b, const Tensor& y) { binary<0>(a, b, y, "add"); }
+void k_mul(const Tensor& a, const Tensor& b, const Tensor& y) { binary<1>(a, b, y, "mul"); }
+void k_scale(const Tensor& a, float s, const Tensor& y) {
+    same_shape(a, y, "scale");
+    PK_DISPATCH1(TA, a.dtype, PK_DISPATCH1(TY, y.dtype,
+                 hipLaunchKernelGGL((ew_scale<TA, TY>), ew_grid(a.numel()), dim3(NT), 0, tape_stream(),
+                                    static_cast<const TA*>(a.ptr()), s, static_cast<TY*>(y.ptr()), a.numel())));
+    post();
+}
+void k_axpy(const Tensor& y, float a, const Tensor& x) {
+    if (x.rows != y.rows || x.cols != y.cols) throw std::runtime_error("accumulate: gradient shape mismatch");  // autograd.cpp:20-22
+    PK_DISPATCH1(TY, y.dtype, PK_DISPATCH1(TX, x.dtype,
+                 hipLaunchKernelGGL((ew_axpy<TY, TX>), ew_grid(y.numel()), dim3(NT), 0, tape_stream(),
+                                    static_cast<TY*>(y.ptr()), a, static_cast<const TX*>(x.ptr()), y.numel())));
+    post();
+}
+void k_silu_fwd(const Tensor& x, const Tensor& y) {
+    same_shape(x, y, "silu");
+    PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((ew_silu_fwd<T>), ew_grid(x.numel()), dim3(NT), 0, tape_stream(),
+                                                static_cast<const T*>(x.ptr()), static_cast<T*>(y.ptr()), x.numel()));
+    post();
+}
+void k_silu_bwd(const Tensor& x, const Tensor& dy, const Tensor& dx) {
+    same_shape(x, dy, "silu");
+    PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((ew_silu_bwd<T>), ew_grid(x.numel()), dim3(NT), 0, tape_stream(),
+                                                static_cast<const T*>(x.ptr()), static_cast<const T*>(dy.ptr()),
+                                                static_cast<T*>(dx.ptr()), x.numel()));
+    post();
+}
+void k_rmsnorm_fwd(const Tensor& x, const Tensor& w, float eps, const Tensor& y, float* rinv) {
+    if (w.rows != 1 || w.cols != x.cols || w.dtype != PK_F32) throw std::runtime_error("rmsnorm: w must be [1, cols(x)]");
+    PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((rms_fwd<T>), dim3((x.rows + 3) / 4), dim3(NT), 0, tape_stream(),
+                                                static_cast<const T*>(x.ptr()), static_cast<const float*>(w.ptr()), eps,
+                                                static_cast<T*>(y.ptr()), rinv, x.rows, static_cast<int>(x.cols)));
+    post();
+}
+void k_rmsnorm_bwd(const Tensor& dy, const Tensor& x, const float* rinv, const Tensor& w, const Tensor* dw,
+                   const Tensor* dx) {
+    const int C = static_cast<int>(x.cols);
+    if (dx) {
+        PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((rms_bwd_dx<T>), dim3((x.rows + 3) / 4), dim3(NT), 0, tape_stream(),
+                                                    static_cast<const T*>(dy.ptr()), static_cast<const T*>(x.ptr()), rinv,
+                                                    static_cast<const float*>(w.ptr()), static_cast<T*>(dx->ptr()),
+                                                    x.rows, C));
+        post();
+    }
+    if (dw) {
+        const int nparts = static_cast<int>((x.rows + ROWS_PB - 1) / ROWS_PB);
+        Buffer part(sizeof(float) * static_cast<size_t>(nparts) * C);
+        PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((rms_bwd_dw_part<T>), dim3(nparts), dim3(NT), 0, tape_stream(),
+                                                    static_cast<const T*>(dy.ptr()), static_cast<const T*>(x.ptr()), rinv,
+                                                    static_cast<float*>(part.p), x.rows, C));
+        post();
+        hipLaunchKernelGGL(colsum_parts, dim3((C + NT - 1) / NT), dim3(NT), 0, tape_stream(),
+                           static_cast<const float*>(part.p), static_cast<float*>(dw->ptr()), nparts, C);
+        post();
+    }
+}
+void k_rope(const Tensor& x, const int* pos, float theta, int d, int head_dim, int rot_heads, bool inverse,
+            const Tensor& y) {
+    if (x.cols != 3 * d) throw std::runtime_error("apply_rope: cols must be divisible by 3");
+    if (head_dim % 2 != 0 || head_dim > d) throw std::runtime_error("apply_rope: head_dim must be even and <= d");
+    PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((rope_k<T>), ew_grid(x.numel() / 2), dim3(NT), 0, tape_stream(),
+                                                static_cast<const T*>(x.ptr()), pos, theta, d, head_dim, rot_heads,
+                                                inverse ? -1.0f : 1.0f, static_cast<T*>(y.ptr()), x.rows));
+    post();
+}
+void k_embedding_fwd(const Tensor& table, const int* ids, const Tensor& y) {
+    PK_DISPATCH1(T, y.dtype, hipLaunchKernelGGL((emb_fwd<T>), ew_grid(y.numel()), dim3(NT), 0, tape_stream(),
+                                                static_cast<const float*>(table.ptr()), ids, static_cast<T*>(y.ptr()),
+                                                y.rows, static_cast<int>(y.cols)));
+    post();
+}
+void k_embedding_bwd(const Tensor& dy, const int* ids, const Tensor& dtable) {
+    PK_DISPATCH1(T, dy.dtype, hipLaunchKernelGGL((emb_bwd<T>), ew_grid(dy.numel()), dim3(NT), 0, tape_stream(),
+                                                 static_cast<const T*>(dy.ptr()), ids, static_cast<float*>(dtable.ptr()),
+                                                 dy.rows, static_cast<int>(dy.cols)));
+    post();
+}
+void k_ce_rows(const Tensor& logits, const int* targets, float gscale, float* nll_rows) {
+    PK_DISPATCH1(T, logits.dtype, hipLaunchKernelGGL((ce_rows<T>), dim3(logits.rows), dim3(NT), 0, tape_stream(),
+                                                     static_cast<T*>(logits.ptr()), targets, gscale, nll_rows,
+                                                     static_cast<int>(logits.cols)));
+    post();
+}
+double k_sum_f32_to_host(const float* x, int64_t n) {
+    Buffer out(sizeof(double));
+    hipLaunchKernelGGL(sum_f32_k, dim3(1), dim3(NT), 0, tape_stream(), x, n, static_cast<double*>(out.p));
+    post();
+    double h = 0.0;
+    HIPCHK(hipMemcpyAsync(&h, out.p, sizeof(double), hipMemcpyDeviceToHost, tape_stream()));
+    HIPCHK(hipStreamSynchronize(tape_stream()));
+    return h;
+}
+double k_sumsq_to_host(const Tensor& g) {
+    if (g.dtype != PK_F32) throw std::runtime_error("clip_grad_norm: gradients must be fp32");
+    const int nb = static_cast<int>(std::min<int64_t>((g.numel() + NT - 1) / NT, 1024));
+    Buffer part(sizeof(double) * nb);
+    hipLaunchKernelGGL(sumsq_part, dim3(nb), dim3(NT), 0, tape_stream(), static_cast<const float*>(g.ptr()), g.numel(),
+                       static_cast<double*>(part.p));
+    post();
+    std::vector<double> h(nb);
+    HIPCHK(hipMemcpyAsync(h.data(), part.p, sizeof(double) * nb, hipMemcpyDeviceToHost, tape_stream()));
+    HIPCHK(hipStreamSynchronize(tape_stream()));
+    double s = 0.0;
+    for (double v : h) s += v;
+    return s;
+}
+void k_adamw(const Tensor& p, const Tensor& g, const Tensor& m, const Tensor& v, float lr, float b1, float b2,
+             float eps, float wd, float c1, float c2) {
+    hipLaunchKernelGGL(adamw_k, ew_grid(p.numel()), dim3(NT), 0, tape_stream(), static_cast<float*>(p.ptr()),
+                       static_cast<const float*>(g.ptr()), static_cast<float*>(m.ptr()), static_cast<float*>(v.ptr()), lr,
+                       b1, b2, eps, wd, c1, c2, p.numel());
+    post();
+}
+
+// ---- GEMM -------------------------------------------------------------------
+namespace {
+rocblas_handle blas() {
+    static rocblas_handle h = [] {
+        rocblas_handle x;
+        if (rocblas_create_handle(&x) != rocblas_status_success) throw std::runtime_error("rocblas_create_handle failed");
+        // no atomics-based split-K: a recomputed (checkpointed) block must reproduce its first forward bit for bit
+        rocblas_set_atomics_mode(x, rocblas_atomics_not_allowed);
+        return x;
+    }();
+    return h;
+}
+}  // namespace
+
+void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dtype, int64_t M, int64_t N, int64_t ldc,
+          float beta) {
+    const int64_t Ka = tA ? A.rows : A.cols, Kb = tB ? B.cols : B.rows;
+    const int64_t Ma = tA ? A.cols : A.rows, Nb = tB ? B.rows : B.cols;
+    if (Ka != Kb) throw std::runtime_error("gemm: inner dimensions disagree");  // device.cpp:97
+    if (Ma != M || Nb != N) throw std::runtime_error("gemm: output shape mismatch");
+    if (A.dtype != B.dtype) throw std::runtime_error("gemm: operand dtypes differ");
+    // Row-major C = op(A) op(B)  <=>  column-major C^T = op(B)^T op(A)^T.
+    const rocblas_datatype ab = A.dtype == PK_F32 ? rocblas_datatype_f32_r : rocblas_datatype_bf16_r;
+    const rocblas_datatype ct = c_dtype == PK_F32 ? rocblas_datatype_f32_r : rocblas_datatype_bf16_r;
+    const float alpha = 1.0f;
+    rocblas_set_stream(blas(), tape_stream());
+    const rocblas_status st = rocblas_gemm_ex(
+        blas(), tB ? rocblas_operation_transpose : rocblas_operation_none,
+        tA ? rocblas_operation_transpose : rocblas_operation_none, static_cast<rocblas_int>(N),
+        static_cast<rocblas_int>(M), static_cast<rocblas_int>(Ka), &alpha, B.ptr(), ab, static_cast<rocblas_int>(B.cols),
+        A.ptr(), ab, static_cast<rocblas_int>(A.cols), &beta, C, ct, static_cast<rocblas_int>(ldc), C, ct,
+        static_cast<rocblas_int>(ldc), rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+    if (st != rocblas_status_success)
+        throw std::runtime_error(std::string("rocblas_gemm_ex failed: ") + rocblas_status_to_string(st));
+}
+
+}  // namespace pk

@@ -1,0 +1,320 @@
+// Llama-family model, AdamW and the training step on the device-resident
+// tape, plus their C ABI. Mirrors paperkiln src/llama.cpp (LlamaBlock::forward
+// :25-60, Llama::forward :71-89), nn::AdamW (src/nn.cpp:301-321) and the step
+// shape of tools/mtstudio.cpp:456-480. The per-block activation checkpoint is
+// the reference's checkpoint() (src/autograd.cpp:68-102) on HBM tensors; its
+// receipt here is bytes from the allocator's high-water mark, not a node count.
+#include <cmath>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "pk_internal.h"
+#include "tape.h"
+
+namespace pk {
+namespace {
+
+// splitmix64 + Box-Muller, the same stream as paperkiln_amd/synth.py randn():
+// the reference initialises from libstdc++'s mt19937 + normal_distribution
+// (nn.cpp:14-21), which is not reproducible outside libstdc++.
+struct Rng {
+    uint64_t seed;
+    static uint64_t mix(uint64_t z) {
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return z ^ (z >> 31);
+    }
+    double u01(uint64_t idx) const {  // idx is 1-based
+        const uint64_t z = mix(seed + idx * 0x9E3779B97F4A7C15ull);
+        return (static_cast<double>(z >> 11) + 0.5) * (1.0 / 9007199254740992.0);
+    }
+};
+std::vector<float> randn_host(uint64_t seed, size_t n, float std_) {
+    const size_t m = (n + 1) / 2;
+    Rng r{seed};
+    std::vector<float> out(2 * m);
+    for (size_t i = 0; i < m; ++i) {
+        const double u1 = r.u01(i + 1), u2 = r.u01(m + i + 1);
+        const double rad = std::sqrt(-2.0 * std::log(u1)), th = 2.0 * M_PI * u2;
+        out[2 * i] = static_cast<float>(rad * std::cos(th) * std_);
+        out[2 * i + 1] = static_cast<float>(rad * std::sin(th) * std_);
+    }
+    out.resize(n);
+    return out;
+}
+
+Var make_param(int64_t r, int64_t c, const std::vector<float>& host) {
+    Tensor t = Tensor::make(r, c, PK_F32);
+    hip_check(hipMemcpy(t.ptr(), host.data(), sizeof(float) * r * c, hipMemcpyHostToDevice), "hipMemcpy");
+    Var v = make_var(std::move(t), true);
+    v->is_param = true;
+    return v;
+}
+
+std::shared_ptr<Buffer> ints_to_dev(const int* h, size_t n) {
+    auto b = std::make_shared<Buffer>(sizeof(int) * n);
+    hip_check(hipMemcpyAsync(b->p, h, sizeof(int) * n, hipMemcpyHostToDevice, tape_stream()), "hipMemcpyAsync");
+    hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+    return b;
+}
+
+struct Block {
+    Var ln1_w, ln2_w, q, k, v, o, gate, up, down;
+};
+
+struct Model {
+    pk_llama_config cfg;
+    Var embed, norm_w;
+    std::vector<Block> blocks;
+    std::vector<std::pair<std::string, Var>> named;
+    bool checkpoint_blocks = false;
+    // AdamW state (nn.cpp:293-299)
+    std::vector<Tensor> m, v;
+    long t = 0;
+
+    void reg(const std::string& name, const Var& p) { named.emplace_back(name, p); }
+
+    Model(const pk_llama_config& c, unsigned seed) : cfg(c) {
+        if (c.d % c.n_heads != 0) throw std::runtime_error("llama: d must divide by n_heads");
+        const int64_t d = c.d, ff = c.d_ff;
+        auto lin = [&](int64_t in, int64_t out, unsigned s) {
+            return make_param(in, out, randn_host(static_cast<uint64_t>(s) * 7919u + 1u, in * out, 0.02f));
+        };
+        const std::vector<float> ones(d, 1.0f);
+        embed = make_param(c.vocab, d, randn_host(static_cast<uint64_t>(seed + 11) * 104729u + 3u, c.vocab * d, 0.02f));
+        reg("embed_tokens.weight", embed);
+        for (int i = 0; i < c.n_layers; ++i) {
+            const unsigned s = seed + 100u * static_cast<unsigned>(i + 1);
+            const std::string p = "layers." + std::to_string(i) + ".";
+            Block b;
+            b.ln1_w = make_param(1, d, ones);
+            b.ln2_w = make_param(1, d, ones);
+            b.q = lin(d, d, s + 1);
+            b.k = lin(d, d, s + 2);
+            b.v = lin(d, d, s + 3);
+            b.o = lin(d, d, s + 4);
+            b.gate = lin(d, ff, s + 5);
+            b.up = lin(d, ff, s + 6);
+            b.down = lin(ff, d, s + 7);
+            reg(p + "input_layernorm.weight", b.ln1_w);
+            reg(p + "post_attention_layernorm.weight", b.ln2_w);
+            reg(p + "self_attn.q_proj.weight", b.q);
+            reg(p + "self_attn.k_proj.weight", b.k);
+            reg(p + "self_attn.v_proj.weight", b.v);
+            reg(p + "self_attn.o_proj.weight", b.o);
+            reg(p + "mlp.gate_proj.weight", b.gate);
+            reg(p + "mlp.up_proj.weight", b.up);
+            reg(p + "mlp.down_proj.weight", b.down);
+            blocks.push_back(b);
+        }
+        norm_w = make_param(1, d, ones);
+        reg("norm.weight", norm_w);
+        if (!c.tie_embeddings) throw std::runtime_error("llama: only the tied head (lm_head = embed_tokens) is built");
+    }
+
+    std::vector<Var> parameters() const {
+        std::vector<Var> out;
+        for (const auto& kv : named) out.push_back(kv.second);
+        return out;
+    }
+
+    // LlamaBlock::forward, llama.cpp:25-60. The 3H slice_cols + H fused_attention +
+    // concat_cols nodes of :47-53 are one attention node reading heads in place.
+    Var block_forward(const Block& b, const Var& x, const std::shared_ptr<Buffer>& pos, int64_t seq_len) const {
+        const int dk = cfg.d / cfg.n_heads;
+        Var h = ops::rmsnorm(x, b.ln1_w);
+        Var qkv = ops::linear3(h, b.q, b.k, b.v);
+        qkv = ops::apply_rope(qkv, pos, cfg.rope_theta, dk, cfg.rope_all_heads ? cfg.n_heads : 1);
+        const float sc = 1.0f / std::sqrt(static_cast<float>(dk));
+        Var attn = ops::linear(ops::attention_qkv(qkv, cfg.n_heads, sc, seq_len, true, cfg.window, cfg.sinks), b.o);
+        Var x1 = ops::add(x, attn);
+        Var h2 = ops::rmsnorm(x1, b.ln2_w);
+        Var ffn = ops::linear(ops::mul(ops::silu(ops::linear(h2, b.gate)), ops::linear(h2, b.up)), b.down);
+        return ops::add(x1, ffn);
+    }
+
+    // Llama::forward (llama.cpp:71-89) up to the final norm; positions restart per sequence.
+    Var hidden(const std::shared_ptr<Buffer>& ids, int64_t n, int64_t seq_len) const {
+        const int64_t sl = seq_len == 0 ? n : seq_len;
+        if (n % sl != 0) throw std::runtime_error("ids not a multiple of seq_len");
+        std::vector<int> pos(n);
+        for (int64_t i = 0; i < n; ++i) pos[i] = static_cast<int>(i % sl);
+        auto pos_dev = ints_to_dev(pos.data(), pos.size());
+        Var h = ops::embedding(embed, ids, n);
+        for (const Block& blk : blocks) {
+            if (checkpoint_blocks && grad_enabled()) {
+                const Block* bp = &blk;
+                h = checkpoint([this, bp, pos_dev, seq_len](const Var& in) { return block_forward(*bp, in, pos_dev, seq_len); },
+                               h);
+            } else {
+                h = block_forward(blk, h, pos_dev, seq_len);
+            }
+        }
+        return ops::rmsnorm(h, norm_w);
+    }
+};
+
+thread_local std::string g_llama_err;
+template <typename F>
+int guarded(F&& f) {
+    try {
+        f();
+        return PK_OK;
+    } catch (const std::exception& e) {
+        g_llama_err = e.what();
+        set_error(g_llama_err);
+        return PK_ERR_ARGUMENT;
+    }
+}
+
+}  // namespace
+}  // namespace pk
+
+using namespace pk;
+
+extern "C" {
+
+int pk_alloc(size_t bytes, void** out) {
+    return guarded([&] { *out = dev_alloc(bytes); });
+}
+int pk_free(void* p) {
+    return guarded([&] { dev_free(p); });
+}
+size_t pk_live_bytes(void) { return dev_live_bytes(); }
+size_t pk_peak_bytes(void) { return dev_peak_bytes(); }
+void pk_reset_peak(void) { dev_reset_peak(); }
+void pk_trim(void) { dev_trim(); }
+
+int pk_llama_create(const pk_llama_config* cfg, unsigned seed, void** handle) {
+    return guarded([&] {
+        if (!cfg || !handle) throw std::runtime_error("pk_llama_create: null argument");
+        set_compute_dtype(cfg->compute_dtype);
+        *handle = new Model(*cfg, seed);
+    });
+}
+int pk_llama_destroy(void* h) {
+    return guarded([&] { delete static_cast<Model*>(h); });
+}
+int pk_llama_num_params(void* h) { return static_cast<int>(static_cast<Model*>(h)->named.size()); }
+int pk_llama_param_info(void* h, int i, char* name, size_t name_len, int64_t* rows, int64_t* cols) {
+    return guarded([&] {
+        Model* m = static_cast<Model*>(h);
+        if (i < 0 || i >= static_cast<int>(m->named.size())) throw std::runtime_error("parameter index out of range");
+        if (name && name_len) std::snprintf(name, name_len, "%s", m->named[i].first.c_str());
+        *rows = m->named[i].second->data.rows;
+        *cols = m->named[i].second->data.cols;
+    });
+}
+int pk_llama_set_param(void* h, int i, const float* host) {
+    return guarded([&] {
+        Model* m = static_cast<Model*>(h);
+        const Tensor& t = m->named.at(i).second->data;
+        hip_check(hipMemcpy(t.ptr(), host, sizeof(float) * t.numel(), hipMemcpyHostToDevice), "hipMemcpy");
+        invalidate_shadows();
+    });
+}
+int pk_llama_get_param(void* h, int i, float* host) {
+    return guarded([&] {
+        Model* m = static_cast<Model*>(h);
+        const Tensor& t = m->named.at(i).second->data;
+        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+        hip_check(hipMemcpy(host, t.ptr(), sizeof(float) * t.numel(), hipMemcpyDeviceToHost), "hipMemcpy");
+    });
+}
+int pk_llama_get_grad(void* h, int i, float* host) {
+    return guarded([&] {
+        Model* m = static_cast<Model*>(h);
+        const Var& p = m->named.at(i).second;
+        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+        if (p->grad.empty())
+            std::memset(host, 0, sizeof(float) * p->data.numel());
+        else
+            hip_check(hipMemcpy(host, p->grad.ptr(), sizeof(float) * p->data.numel(), hipMemcpyDeviceToHost), "hipMemcpy");
+    });
+}
+
+int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets, int64_t n, int64_t seq_len,
+                           int checkpoint_blocks, int do_backward, int fused_head, float* loss, pk_llama_stats* stats,
+                           void* stream) {
+    return guarded([&] {
+        Model* m = static_cast<Model*>(h);
+        set_tape_stream(static_cast<hipStream_t>(stream));
+        for (int64_t i = 0; i < n; ++i)
+            if (host_ids[i] < 0 || host_ids[i] >= m->cfg.vocab) throw std::runtime_error("embedding: id out of range");
+        for (int64_t i = 0; i < n; ++i)
+            if (host_targets[i] < 0 || host_targets[i] >= m->cfg.vocab)
+                throw std::runtime_error("cross_entropy: target out of range");
+        m->checkpoint_blocks = checkpoint_blocks != 0;
+        auto params = m->parameters();
+        zero_grad(params);
+        for (const auto& p : params) p->ensure_grad();  // persistent state, kept out of the activation receipt
+        auto ids = ints_to_dev(host_ids, n);
+        auto tg = ints_to_dev(host_targets, n);
+        // Everything allocated from here on, until backward returns, is activation memory.
+        if (compute_dtype() != PK_F32) {  // build the bf16 parameter shadows first: they are not activations
+            NoGrad ng;
+            Tensor probe = Tensor::make(1, m->cfg.d, compute_dtype());
+            k_fill(probe, 0.0f);
+            for (const auto& b : m->blocks) {
+                Var x = make_var(probe);
+                (void)ops::linear3(x, b.q, b.k, b.v);
+                (void)ops::linear(x, b.o);
+                (void)ops::linear(x, b.gate);
+                (void)ops::linear(x, b.up);
+                Tensor pf = Tensor::make(1, m->cfg.d_ff, compute_dtype());
+                k_fill(pf, 0.0f);
+                (void)ops::linear(make_var(pf), b.down);
+            }
+            (void)ops::matmul_nt(make_var(probe), m->embed);
+        }
+        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+        const size_t base = dev_live_bytes();
+        dev_reset_peak();
+        const size_t live0 = live_variables();
+        Var hid = m->hidden(ids, n, seq_len);
+        Var l = fused_head ? ops::linear_cross_entropy(hid, m->embed, tg, 1024)
+                           : ops::cross_entropy(ops::matmul_nt(hid, m->embed), tg);
+        hid.reset();
+        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+        if (stats) {
+            stats->live_vars_after_forward = static_cast<int64_t>(live_variables() - live0);
+            stats->activation_bytes_after_forward = static_cast<int64_t>(dev_live_bytes() - base);
+        }
+        if (do_backward) backward(l);
+        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+        if (stats) stats->peak_activation_bytes = static_cast<int64_t>(dev_peak_bytes() - base);
+        float hl = 0.0f;
+        hip_check(hipMemcpy(&hl, l->data.ptr(), 4, hipMemcpyDeviceToHost), "hipMemcpy");
+        *loss = hl;
+    });
+}
+
+int pk_llama_adamw_step(void* h, float lr, float b1, float b2, float eps, float wd, float max_norm, float* total_norm) {
+    return guarded([&] {
+        Model* m = static_cast<Model*>(h);
+        auto params = m->parameters();
+        if (m->m.empty()) {
+            for (const auto& p : params) {
+                m->m.push_back(Tensor::make(p->data.rows, p->data.cols, PK_F32));
+                m->v.push_back(Tensor::make(p->data.rows, p->data.cols, PK_F32));
+                k_fill(m->m.back(), 0.0f);
+                k_fill(m->v.back(), 0.0f);
+            }
+        }
+        double tn = 0.0;
+        if (max_norm > 0.0f) tn = ops::clip_grad_norm(params, max_norm);
+        if (total_norm) *total_norm = static_cast<float>(tn);
+        ++m->t;
+        const float c1 = 1.0f - std::pow(b1, static_cast<float>(m->t));
+        const float c2 = 1.0f - std::pow(b2, static_cast<float>(m->t));
+        for (size_t k = 0; k < params.size(); ++k) {
+            if (params[k]->grad.empty()) continue;  // never accumulated (nn.cpp:309)
+            k_adamw(params[k]->data, params[k]->grad, m->m[k], m->v[k], lr, b1, b2, eps, wd, c1, c2);
+        }
+        invalidate_shadows();
+        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+    });
+}
+
+}  // extern "C"

@@ -1,0 +1,532 @@
+// Host side of the device-resident tape: see tape.h. Plain C++ driving the
+// kernels of elementwise.hip and the attention entry points of the C ABI.
+#include "tape.h"
+
+#include <cmath>
+#include <cstring>
+#include <unordered_map>
+#include <unordered_set>
+
+namespace pk {
+
+namespace detail {
+std::atomic<size_t> g_live_vars{0};
+}
+size_t live_variables() { return detail::g_live_vars.load(); }
+
+namespace {
+thread_local bool g_grad_enabled = true;
+int g_compute = PK_F32;
+// compute-dtype copies of fp32 parameters, valid until the next optimizer step
+std::unordered_map<const Variable*, Tensor> g_shadow;
+
+const Tensor& shadow_of(const Var& W) {
+    if (g_compute == PK_F32 || W->data.dtype != PK_F32) return W->data;
+    auto it = g_shadow.find(W.get());
+    if (it == g_shadow.end()) {
+        Tensor t = Tensor::make(W->data.rows, W->data.cols, g_compute);
+        k_cast(W->data, t);
+        it = g_shadow.emplace(W.get(), std::move(t)).first;
+    }
+    return it->second;
+}
+
+// Post-order DFS over parents, iterative (autograd.cpp:31-45).
+void topo(const Var& root, std::vector<Variable*>& order) {
+    std::unordered_set<Variable*> seen;
+    std::vector<std::pair<Variable*, size_t>> stack{{root.get(), 0}};
+    seen.insert(root.get());
+    while (!stack.empty()) {
+        auto& [node, next] = stack.back();
+        if (next < node->parents.size()) {
+            Variable* p = node->parents[next++].get();
+            if (seen.insert(p).second) stack.emplace_back(p, 0);
+        } else {
+            order.push_back(node);
+            stack.pop_back();
+        }
+    }
+}
+
+void run_backward(const Var& root) {
+    std::vector<Variable*> order;
+    topo(root, order);
+    for (auto it = order.rbegin(); it != order.rend(); ++it) {
+        if ((*it)->backward_fn && !(*it)->grad.empty()) (*it)->backward_fn();
+    }
+}
+
+float scalar_to_host(const Tensor& t) {
+    float h = 0.0f;
+    if (t.dtype == PK_F32) {
+        hip_check(hipMemcpyAsync(&h, t.ptr(), 4, hipMemcpyDeviceToHost, tape_stream()), "hipMemcpyAsync");
+        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+    } else {
+        uint16_t u = 0;
+        hip_check(hipMemcpyAsync(&u, t.ptr(), 2, hipMemcpyDeviceToHost, tape_stream()), "hipMemcpyAsync");
+        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+        uint32_t w = static_cast<uint32_t>(u) << 16;
+        std::memcpy(&h, &w, 4);
+    }
+    return h;
+}
+
+pk_tensor4 view4(const void* base, int64_t elem_off, size_t esize, int64_t sb, int64_t st, int64_t sh) {
+    pk_tensor4 t;
+    t.ptr = const_cast<char*>(static_cast<const char*>(base)) + elem_off * static_cast<int64_t>(esize);
+    t.stride_b = sb;
+    t.stride_t = st;
+    t.stride_h = sh;
+    return t;
+}
+void attn_check(int rc) {
+    if (rc != PK_OK) throw std::runtime_error(pk_last_error());
+}
+
+}  // namespace
+
+void set_compute_dtype(int dtype) {
+    if (dtype != PK_F32 && dtype != PK_BF16) throw std::runtime_error("compute dtype must be PK_F32 or PK_BF16");
+    g_compute = dtype;
+    g_shadow.clear();
+}
+int compute_dtype() { return g_compute; }
+void invalidate_shadows() { g_shadow.clear(); }
+
+Tensor& Variable::ensure_grad() {
+    if (grad.empty()) {
+        grad = Tensor::make(data.rows, data.cols, is_param ? PK_F32 : data.dtype);
+        k_fill(grad, 0.0f);
+    }
+    return grad;
+}
+
+void Variable::accumulate(const Tensor& g, float a) {
+    if (g.rows != data.rows || g.cols != data.cols) throw std::runtime_error("accumulate: gradient shape mismatch");
+    if (grad.empty()) {
+        grad = Tensor::make(data.rows, data.cols, is_param ? PK_F32 : data.dtype);
+        k_scale(g, a, grad);  // first contribution: grad = a * g, no zero fill
+        return;
+    }
+    k_axpy(grad, a, g);
+}
+
+bool grad_enabled() { return g_grad_enabled; }
+NoGrad::NoGrad() : prev_(g_grad_enabled) { g_grad_enabled = false; }
+NoGrad::~NoGrad() { g_grad_enabled = prev_; }
+
+Var record(Tensor result, std::vector<Var> parents, std::function<void(Variable*)> bw) {
+    bool needs = false;
+    if (grad_enabled())
+        for (const auto& p : parents) needs = needs || p->requires_grad;
+    Var out = make_var(std::move(result), needs);
+    if (needs) {
+        out->parents = std::move(parents);
+        Variable* self = out.get();
+        out->backward_fn = [self, bw]() { bw(self); };
+    }
+    return out;
+}
+
+void backward(const Var& root) {
+    if (root->data.rows != 1 || root->data.cols != 1)
+        throw std::runtime_error("backward: root must be a [1,1] scalar (compose with mean/sum)");
+    Tensor seed = Tensor::make(1, 1, root->data.dtype);
+    k_fill(seed, 1.0f);
+    root->accumulate(seed);
+    run_backward(root);
+}
+
+void zero_grad(const std::vector<Var>& vars) {
+    for (const auto& v : vars)
+        if (!v->grad.empty()) k_fill(v->grad, 0.0f);
+}
+
+Var checkpoint(const std::function<Var(const Var&)>& fn, const Var& x) {
+    if (!grad_enabled()) return fn(x);  // eval: nothing to rematerialise
+    Tensor out_data;
+    {
+        NoGrad ng;
+        out_data = fn(x)->data;  // the inner tape never exists
+    }
+    Var out = make_var(std::move(out_data), true);
+    out->parents = {x};
+    Variable* self = out.get();
+    auto fn_copy = fn;
+    out->backward_fn = [self, fn_copy]() {
+        const Var& xin = self->parents[0];
+        // Re-run the segment on a detached leaf that shares the input's storage: nothing
+        // writes into an activation after it is produced, so the copy the reference makes
+        // (autograd.cpp:86) is not needed on a tape whose tensors are immutable.
+        Var x2 = make_var(xin->data, /*requires_grad=*/true);
+        Var y2 = fn_copy(x2);
+        if (y2->data.rows != self->grad.rows || y2->data.cols != self->grad.cols)
+            throw std::runtime_error("checkpoint: recomputed output shape mismatch");
+        y2->accumulate(self->grad);
+        run_backward(y2);  // parameters inside fn are the model's own, their grads land in place
+        if (xin->requires_grad && !x2->grad.empty()) xin->accumulate(x2->grad);
+    };
+    return out;
+}
+
+namespace ops {
+
+Var linear(const Var& x, const Var& W) {
+    if (x->data.cols != W->data.rows) throw std::runtime_error("matmul: inner dimensions disagree");
+    const Tensor& Wc = shadow_of(W);
+    Tensor y = Tensor::make(x->data.rows, W->data.cols, x->data.dtype);
+    gemm(x->data, false, Wc, false, y.ptr(), y.dtype, y.rows, y.cols, y.cols, 0.0f);
+    return record(std::move(y), {x, W}, [](Variable* self) {
+        const Var& x = self->parents[0];
+        const Var& W = self->parents[1];
+        if (x->requires_grad) {  // dX = dY W^T  (ops.cpp:48-51)
+            Tensor dx = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
+            gemm(self->grad, false, shadow_of(W), true, dx.ptr(), dx.dtype, dx.rows, dx.cols, dx.cols, 0.0f);
+            x->accumulate(dx);
+        }
+        if (W->requires_grad) {  // dW += X^T dY (ops.cpp:52-55), straight into the fp32 grad
+            Tensor& g = W->ensure_grad();
+            gemm(x->data, true, self->grad, false, g.ptr(), g.dtype, g.rows, g.cols, g.cols, 1.0f);
+        }
+    });
+}
+
+Var linear3(const Var& x, const Var& Wq, const Var& Wk, const Var& Wv) {
+    const int64_t N = x->data.rows, d = Wq->data.cols;
+    if (Wk->data.cols != d || Wv->data.cols != d || Wq->data.rows != x->data.cols || Wk->data.rows != x->data.cols ||
+        Wv->data.rows != x->data.cols)
+        throw std::runtime_error("matmul: inner dimensions disagree");
+    Tensor y = Tensor::make(N, 3 * d, x->data.dtype);
+    const size_t es = y.esize();
+    const Var Ws[3] = {Wq, Wk, Wv};
+    for (int i = 0; i < 3; ++i)
+        gemm(x->data, false, shadow_of(Ws[i]), false, static_cast<char*>(y.ptr()) + i * d * es, y.dtype, N, d, 3 * d, 0.0f);
+    return record(std::move(y), {x, Wq, Wk, Wv}, [d](Variable* self) {
+        const Var& x = self->parents[0];
+        const int64_t N = x->data.rows;
+        // the three column slices of dY, viewed as [N, d] matrices with row pitch 3d
+        Tensor dx;
+        if (x->requires_grad) dx = Tensor::make(N, x->data.cols, x->data.dtype);
+        for (int i = 0; i < 3; ++i) {
+            const Var& W = self->parents[1 + i];
+            Tensor slice = Tensor::make(N, d, self->grad.dtype);  // contiguous copy of the slice
+            {
+                // strided copy via GEMM-free path: cast kernel works on contiguous data only, so
+                // use a 2-D memcpy
+                const size_t es = slice.esize();
+                hip_check(hipMemcpy2DAsync(slice.ptr(), d * es, static_cast<const char*>(self->grad.ptr()) + i * d * es,
+                                           3 * d * es, d * es, N, hipMemcpyDeviceToDevice, tape_stream()),
+                          "hipMemcpy2DAsync");
+            }
+            if (x->requires_grad)
+                gemm(slice, false, shadow_of(W), true, dx.ptr(), dx.dtype, N, x->data.cols, x->data.cols, i == 0 ? 0.0f : 1.0f);
+            if (W->requires_grad) {
+                Tensor& g = W->ensure_grad();
+                gemm(x->data, true, slice, false, g.ptr(), g.dtype, g.rows, g.cols, g.cols, 1.0f);
+            }
+        }
+        if (x->requires_grad) x->accumulate(dx);
+    });
+}
+
+Var add(const Var& a, const Var& b) {
+    Tensor y = Tensor::make(a->data.rows, a->data.cols, a->data.dtype);
+    k_add(a->data, b->data, y);
+    return record(std::move(y), {a, b}, [](Variable* self) {
+        if (self->parents[0]->requires_grad) self->parents[0]->accumulate(self->grad);
+        if (self->parents[1]->requires_grad) self->parents[1]->accumulate(self->grad);
+    });
+}
+
+Var mul(const Var& a, const Var& b) {
+    Tensor y = Tensor::make(a->data.rows, a->data.cols, a->data.dtype);
+    k_mul(a->data, b->data, y);
+    return record(std::move(y), {a, b}, [](Variable* self) {
+        const Var& a = self->parents[0];
+        const Var& b = self->parents[1];
+        if (a->requires_grad) {
+            Tensor t = Tensor::make(a->data.rows, a->data.cols, a->data.dtype);
+            k_mul(self->grad, b->data, t);
+            a->accumulate(t);
+        }
+        if (b->requires_grad) {
+            Tensor t = Tensor::make(a->data.rows, a->data.cols, a->data.dtype);
+            k_mul(self->grad, a->data, t);
+            b->accumulate(t);
+        }
+    });
+}
+
+Var scale(const Var& x, float s) {
+    Tensor y = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
+    k_scale(x->data, s, y);
+    return record(std::move(y), {x}, [s](Variable* self) {
+        if (self->parents[0]->requires_grad) self->parents[0]->accumulate(self->grad, s);
+    });
+}
+
+Var silu(const Var& x) {
+    Tensor y = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
+    k_silu_fwd(x->data, y);
+    return record(std::move(y), {x}, [](Variable* self) {
+        const Var& x = self->parents[0];
+        if (!x->requires_grad) return;
+        Tensor dx = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
+        k_silu_bwd(x->data, self->grad, dx);
+        x->accumulate(dx);
+    });
+}
+
+Var rmsnorm(const Var& x, const Var& w) {
+    if (w->data.rows != 1 || w->data.cols != x->data.cols) throw std::runtime_error("rmsnorm: w must be [1, cols(x)]");
+    auto rinv = std::make_shared<Buffer>(sizeof(float) * x->data.rows);
+    Tensor y = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
+    k_rmsnorm_fwd(x->data, w->data, 1e-5f, y, static_cast<float*>(rinv->p));
+    return record(std::move(y), {x, w}, [rinv](Variable* self) {
+        const Var& x = self->parents[0];
+        const Var& w = self->parents[1];
+        Tensor dx;
+        if (x->requires_grad) dx = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
+        Tensor* dw = w->requires_grad ? &w->ensure_grad() : nullptr;
+        k_rmsnorm_bwd(self->grad, x->data, static_cast<const float*>(rinv->p), w->data, dw,
+                      x->requires_grad ? &dx : nullptr);
+        if (x->requires_grad) x->accumulate(dx);
+    });
+}
+
+Var apply_rope(const Var& qkv, const std::shared_ptr<Buffer>& pos, float theta, int head_dim, int rot_heads) {
+    if (qkv->data.cols % 3 != 0) throw std::runtime_error("apply_rope: cols must be divisible by 3");
+    const int d = static_cast<int>(qkv->data.cols / 3);
+    Tensor y = Tensor::make(qkv->data.rows, qkv->data.cols, qkv->data.dtype);
+    k_rope(qkv->data, static_cast<const int*>(pos->p), theta, d, head_dim, rot_heads, false, y);
+    return record(std::move(y), {qkv}, [pos, theta, head_dim, rot_heads, d](Variable* self) {
+        const Var& x = self->parents[0];
+        if (!x->requires_grad) return;
+        Tensor dx = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
+        k_rope(self->grad, static_cast<const int*>(pos->p), theta, d, head_dim, rot_heads, true, dx);
+        x->accumulate(dx);
+    });
+}
+
+Var embedding(const Var& table, const std::shared_ptr<Buffer>& ids, int64_t n) {
+    Tensor y = Tensor::make(n, table->data.cols, compute_dtype());
+    k_embedding_fwd(table->data, static_cast<const int*>(ids->p), y);
+    return record(std::move(y), {table}, [ids](Variable* self) {
+        const Var& t = self->parents[0];
+        if (!t->requires_grad) return;
+        k_embedding_bwd(self->grad, static_cast<const int*>(ids->p), t->ensure_grad());  // scatter-add, ops.cpp:338-347
+    });
+}
+
+namespace {
+
+struct AttnGeom {
+    int64_t B, T;
+    int H, dk;
+    float scale;
+    bool causal;
+    int window, sinks;
+};
+
+pk_attn_shape shape_of(const AttnGeom& g, int dtype) {
+    pk_attn_shape s;
+    s.B = static_cast<int32_t>(g.B);
+    s.T = static_cast<int32_t>(g.T);
+    s.Hq = s.Hkv = g.H;
+    s.dk = g.dk;
+    s.causal = g.causal;
+    s.window = g.window;
+    s.sinks = g.sinks;
+    s.scale = g.scale;
+    s.dtype = s.grad_dtype = dtype;
+    return s;
+}
+
+}  // namespace
+
+Var attention_qkv(const Var& qkv, int n_heads, float scale, int64_t seq_len, bool causal, int window, int sinks) {
+    const int64_t N = qkv->data.rows, d3 = qkv->data.cols;
+    if (d3 % 3 != 0 || (d3 / 3) % n_heads != 0) throw std::runtime_error("fused_attention: shape mismatch");
+    const int64_t d = d3 / 3, sl = seq_len == 0 ? N : seq_len;
+    if (N % sl != 0) throw std::runtime_error("fused_attention: rows not a multiple of seq_len");
+    AttnGeom g{N / sl, sl, n_heads, static_cast<int>(d / n_heads), scale, causal, window, sinks};
+    const int dt = qkv->data.dtype;
+    const size_t es = qkv->data.esize();
+    Tensor o = Tensor::make(N, d, dt);
+    auto lse = std::make_shared<Buffer>(sizeof(float) * g.B * g.H * g.T);
+    const pk_attn_shape sh = shape_of(g, dt);
+    const pk_tensor4 q4 = view4(qkv->data.ptr(), 0, es, sl * d3, d3, g.dk), k4 = view4(qkv->data.ptr(), d, es, sl * d3, d3, g.dk),
+                     v4 = view4(qkv->data.ptr(), 2 * d, es, sl * d3, d3, g.dk), o4 = view4(o.ptr(), 0, es, sl * d, d, g.dk);
+    attn_check(pk_attn_fwd(&sh, &q4, &k4, &v4, &o4, static_cast<float*>(lse->p), tape_stream()));
+    // The node keeps O (its own data) and LSE; P is rebuilt from Q, K and LSE in backward.
+    return record(std::move(o), {qkv}, [g, lse](Variable* self) {
+        const Var& qkv = self->parents[0];
+        if (!qkv->requires_grad) return;
+        const int64_t N = qkv->data.rows, d3 = qkv->data.cols, d = d3 / 3, sl = g.T;
+        const int dt = qkv->data.dtype;
+        const size_t es = qkv->data.esize();
+        Tensor dqkv = Tensor::make(N, d3, dt);
+        const pk_attn_shape sh = shape_of(g, dt);
+        Buffer ws(pk_attn_bwd_workspace_bytes(&sh));
+        const pk_tensor4 q4 = view4(qkv->data.ptr(), 0, es, sl * d3, d3, g.dk), k4 = view4(qkv->data.ptr(), d, es, sl * d3, d3, g.dk),
+                         v4 = view4(qkv->data.ptr(), 2 * d, es, sl * d3, d3, g.dk),
+                         o4 = view4(self->data.ptr(), 0, es, sl * d, d, g.dk), g4 = view4(self->grad.ptr(), 0, es, sl * d, d, g.dk),
+                         dq4 = view4(dqkv.ptr(), 0, es, sl * d3, d3, g.dk), dk4 = view4(dqkv.ptr(), d, es, sl * d3, d3, g.dk),
+                         dv4 = view4(dqkv.ptr(), 2 * d, es, sl * d3, d3, g.dk);
+        attn_check(pk_attn_bwd(&sh, &q4, &k4, &v4, &o4, static_cast<const float*>(lse->p), &g4, &dq4, &dk4, &dv4, ws.p,
+                               ws.bytes, tape_stream()));
+        qkv->accumulate(dqkv);
+    });
+}
+
+namespace {
+Var head_attention(const Var& q, const Var& k, const Var& v, float scale, int64_t seq_len, bool causal, int window,
+                   int sinks, const char* who) {
+    const int64_t T = q->data.rows;
+    if (k->data.rows != T || v->data.rows != T || q->data.cols != k->data.cols || v->data.cols != k->data.cols)
+        throw std::runtime_error(std::string(who) + ": shape mismatch");
+    const int64_t sl = seq_len == 0 ? T : seq_len;
+    if (T % sl != 0) throw std::runtime_error(std::string(who) + ": rows not a multiple of seq_len");
+    const int dk = static_cast<int>(q->data.cols);
+    AttnGeom g{T / sl, sl, 1, dk, scale, causal, window, sinks};
+    const int dt = q->data.dtype;
+    const size_t es = q->data.esize();
+    Tensor o = Tensor::make(T, dk, dt);
+    auto lse = std::make_shared<Buffer>(sizeof(float) * T);
+    const pk_attn_shape sh = shape_of(g, dt);
+    auto v4of = [&](const Tensor& t) { return view4(t.ptr(), 0, es, sl * dk, dk, dk); };
+    const pk_tensor4 q4 = v4of(q->data), k4 = v4of(k->data), vv4 = v4of(v->data), o4 = v4of(o);
+    attn_check(pk_attn_fwd(&sh, &q4, &k4, &vv4, &o4, static_cast<float*>(lse->p), tape_stream()));
+    return record(std::move(o), {q, k, v}, [g, lse](Variable* self) {
+        const Var& q = self->parents[0];
+        const Var& k = self->parents[1];
+        const Var& v = self->parents[2];
+        if (!q->requires_grad && !k->requires_grad && !v->requires_grad) return;
+        const int dt = q->data.dtype, dk = g.dk;
+        const size_t es = q->data.esize();
+        const int64_t T = q->data.rows, sl = g.T;
+        Tensor dq = Tensor::make(T, dk, dt), dkk = Tensor::make(T, dk, dt), dv = Tensor::make(T, dk, dt);
+        const pk_attn_shape sh = shape_of(g, dt);
+        Buffer ws(pk_attn_bwd_workspace_bytes(&sh));
+        auto v4of = [&](const Tensor& t) { return view4(t.ptr(), 0, es, sl * dk, dk, dk); };
+        const pk_tensor4 q4 = v4of(q->data), k4 = v4of(k->data), vv4 = v4of(v->data), o4 = v4of(self->data),
+                         g4 = v4of(self->grad), dq4 = v4of(dq), dk4 = v4of(dkk), dv4 = v4of(dv);
+        attn_check(pk_attn_bwd(&sh, &q4, &k4, &vv4, &o4, static_cast<const float*>(lse->p), &g4, &dq4, &dk4, &dv4, ws.p,
+                               ws.bytes, tape_stream()));
+        if (q->requires_grad) q->accumulate(dq);
+        if (k->requires_grad) k->accumulate(dkk);
+        if (v->requires_grad) v->accumulate(dv);
+    });
+}
+}  // namespace
+
+Var fused_attention(const Var& q, const Var& k, const Var& v, float scale, int64_t seq_len, bool causal) {
+    return head_attention(q, k, v, scale, seq_len, causal, 0, 0, "fused_attention");
+}
+Var swa_attention(const Var& q, const Var& k, const Var& v, float scale, int64_t window, int64_t sinks, int64_t seq_len) {
+    if (window == 0) throw std::runtime_error("swa_attention: window must be >= 1");  // ops.cpp:954
+    return head_attention(q, k, v, scale, seq_len, true, static_cast<int>(window), static_cast<int>(sinks), "swa_attention");
+}
+
+Var matmul_nt(const Var& h, const Var& E) {
+    if (h->data.cols != E->data.cols) throw std::runtime_error("matmul: inner dimensions disagree");
+    Tensor y = Tensor::make(h->data.rows, E->data.rows, PK_F32);  // logits stay fp32, as in the reference
+    gemm(h->data, false, shadow_of(E), true, y.ptr(), y.dtype, y.rows, y.cols, y.cols, 0.0f);
+    return record(std::move(y), {h, E}, [](Variable* self) {
+        const Var& h = self->parents[0];
+        const Var& E = self->parents[1];
+        Tensor dl = self->grad;
+        if (dl.dtype != h->data.dtype) {
+            dl = Tensor::make(self->grad.rows, self->grad.cols, h->data.dtype);
+            k_cast(self->grad, dl);
+        }
+        if (h->requires_grad) {
+            Tensor dh = Tensor::make(h->data.rows, h->data.cols, h->data.dtype);
+            gemm(dl, false, shadow_of(E), false, dh.ptr(), dh.dtype, dh.rows, dh.cols, dh.cols, 0.0f);
+            h->accumulate(dh);
+        }
+        if (E->requires_grad) {
+            Tensor& g = E->ensure_grad();
+            gemm(dl, true, h->data, false, g.ptr(), g.dtype, g.rows, g.cols, g.cols, 1.0f);
+        }
+    });
+}
+
+Var cross_entropy(const Var& logits, const std::shared_ptr<Buffer>& targets) {
+    const int64_t R = logits->data.rows;
+    // softmax copy for the fused backward, as the reference caches P (ops.cpp:357)
+    auto P = std::make_shared<Tensor>(Tensor::make(R, logits->data.cols, logits->data.dtype));
+    k_cast(logits->data, *P);
+    Buffer nll(sizeof(float) * R);
+    k_ce_rows(*P, static_cast<const int*>(targets->p), 1.0f / static_cast<float>(R), static_cast<float*>(nll.p));
+    const double total = k_sum_f32_to_host(static_cast<const float*>(nll.p), R);
+    Tensor out = Tensor::make(1, 1, PK_F32);
+    k_fill(out, static_cast<float>(total / static_cast<double>(R)));
+    return record(std::move(out), {logits}, [P](Variable* self) {
+        const Var& l = self->parents[0];
+        if (!l->requires_grad) return;
+        l->accumulate(*P, scalar_to_host(self->grad));  // (P - onehot) * g / R, ops.cpp:371-374
+    });
+}
+
+Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffer>& targets, int64_t chunk_rows) {
+    const int64_t N = h->data.rows, V = E->data.rows;
+    if (h->data.cols != E->data.cols) throw std::runtime_error("matmul: inner dimensions disagree");
+    if (chunk_rows <= 0) chunk_rows = 1024;
+    const int* tg = static_cast<const int*>(targets->p);
+    const size_t hes = h->data.esize();
+    // one pass over row chunks; with_grad also produces dh and accumulates dE
+    auto pass = [N, V, chunk_rows, tg, hes](const Var& h, const Var& E, float gscale, Tensor* dh, Tensor* dE) {
+        const Tensor& Ec = shadow_of(E);
+        Buffer nll(sizeof(float) * N);
+        for (int64_t r0 = 0; r0 < N; r0 += chunk_rows) {
+            const int64_t rows = std::min(chunk_rows, N - r0);
+            const Tensor hview = h->data.row_range(r0, rows);
+            Tensor logits = Tensor::make(rows, V, PK_F32);
+            gemm(hview, false, Ec, true, logits.ptr(), PK_F32, rows, V, V, 0.0f);
+            k_ce_rows(logits, tg + r0, gscale, static_cast<float*>(nll.p) + r0);
+            if (dh || dE) {
+                Tensor dl = logits;
+                if (h->data.dtype != PK_F32) {
+                    dl = Tensor::make(rows, V, h->data.dtype);
+                    k_cast(logits, dl);
+                }
+                if (dh)
+                    gemm(dl, false, Ec, false, static_cast<char*>(dh->ptr()) + r0 * h->data.cols * hes, dh->dtype, rows,
+                         h->data.cols, h->data.cols, 0.0f);
+                if (dE) gemm(dl, true, hview, false, dE->ptr(), dE->dtype, V, h->data.cols, h->data.cols, 1.0f);
+            }
+        }
+        return k_sum_f32_to_host(static_cast<const float*>(nll.p), N);
+    };
+    const double total = pass(h, E, 0.0f, nullptr, nullptr);
+    Tensor out = Tensor::make(1, 1, PK_F32);
+    k_fill(out, static_cast<float>(total / static_cast<double>(N)));
+    // Backward recomputes each chunk of logits: nothing of size [N, vocab] is kept.
+    return record(std::move(out), {h, E}, [pass, N](Variable* self) {
+        const Var& h = self->parents[0];
+        const Var& E = self->parents[1];
+        const float g = scalar_to_host(self->grad) / static_cast<float>(N);
+        Tensor dh;
+        if (h->requires_grad) dh = Tensor::make(h->data.rows, h->data.cols, h->data.dtype);
+        Tensor* dE = E->requires_grad ? &E->ensure_grad() : nullptr;
+        pass(h, E, g, h->requires_grad ? &dh : nullptr, dE);
+        if (h->requires_grad) h->accumulate(dh);
+    });
+}
+
+double clip_grad_norm(const std::vector<Var>& params, float max_norm) {
+    double sq = 0.0;
+    for (const auto& p : params)
+        if (!p->grad.empty()) sq += k_sumsq_to_host(p->grad);
+    const double total = std::sqrt(sq);
+    if (total > max_norm && total > 0.0) {
+        const float s = static_cast<float>(max_norm / total);
+        for (const auto& p : params)
+            if (!p->grad.empty()) k_scale(p->grad, s, p->grad);
+    }
+    return total;
+}
+
+}  // namespace ops
+}  // namespace pk
