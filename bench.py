@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
 # HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs
 # (FETCH_SIZE, WRITE_SIZE) scaled by a copy kernel of known size; see
 # profiles/. None until measured for the current kernel.
-MEASURED_TRAFFIC_BYTES = None
+MEASURED_TRAFFIC_BYTES = {"dkdv": 5.11e8, "dq": 4.30e8, "fwd": 3.38e8}  # profiles/attn_*_pmc.txt, fetch x2.0 + write x1.0
 
 
 def cpu_baseline(B, T, H, dk, scale, seconds_budget=30.0):
@@ -69,6 +69,69 @@ def cpu_baseline(B, T, H, dk, scale, seconds_budget=30.0):
             "sample": f"1 of {B * H} (batch, head) units of the same workload, fwd+bwd, {dt:.2f} s wall; "
                       f"whole job would take ~{dt * B * H:.0f} s on one core",
             "host_cpu": cpu, "host_nproc": os.cpu_count()}
+
+
+def window_variant(ops, q, k, v, d_o, out, scale, B, H, T, dk, warmup, steps):
+    """Same shape, window=256 + 4 sink keys (BASELINE config 4b): 12% of the causal pairs are live, every
+    byte still moves once, so this one is priced against the HBM roofline."""
+    import torch
+    from paperkiln_amd import synth
+    W, S = 256, 4
+
+    def step():
+        o, lse = ops.attn_fwd(q, k, v, scale, True, W, S)
+        ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, W, S, out=out)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    pairs = synth.visible_pairs(T, True, W, S)
+    nbytes = 12.0 * B * T * H * dk * 2 + 2.0 * B * H * T * 4
+    return {"workload": "same shape, window=256, sinks=4", "ms_per_step": round(ms, 4),
+            "tflops": round(14.0 * dk * pairs * B * H / (ms * 1e-3) / 1e12, 2),
+            "roofline": {"bound": "hbm", "achieved": round(nbytes / (ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}}
+
+
+def llama_step():
+    """Activation-checkpointed Llama training step (BASELINE config 5): 6 layers, d=512, 8 heads, SwiGLU 1376,
+    vocab 32000 tied, B=8 x T=1024 tokens, bf16 compute with fp32 master weights. Reports tokens/s, the loss
+    with and without per-block checkpointing, and the allocator's peak activation bytes for both."""
+    from paperkiln_amd import synth
+    from paperkiln_amd.llama import Llama
+    cfg = dict(vocab=32000, d=512, n_layers=6, n_heads=8, d_ff=1376)
+    B, T = 8, 1024
+    m = Llama(compute_dtype="bf16", seed=0, **cfg)
+    toks = synth.randint(9, B * T + 1, cfg["vocab"])
+    x, y = toks[:-1], toks[1:]
+    out = {"workload": "Llama L6 d512 H8 d_ff1376 V32000 tied, B=8 T=1024, bf16 compute / fp32 master, fwd+bwd+AdamW",
+           "params": m.parameter_count()}
+    for ck in (False, True):
+        for _ in range(2):
+            m.loss_backward(x, y, T, checkpoint=ck)
+        t0 = time.perf_counter()
+        n = 3
+        for _ in range(n):
+            loss, st = m.loss_backward(x, y, T, checkpoint=ck)
+        dt = (time.perf_counter() - t0) / n
+        tag = "checkpointed" if ck else "plain"
+        out[tag] = {"loss": round(loss, 6), "ms_fwd_bwd": round(dt * 1e3, 2), "tokens_per_s_fwd_bwd": round(B * T / dt, 0),
+                    "peak_activation_bytes": st["peak_activation_bytes"],
+                    "activation_bytes_after_forward": st["activation_bytes_after_forward"],
+                    "live_vars_after_forward": st["live_vars_after_forward"]}
+    t0 = time.perf_counter()
+    m.adamw_step(1e-3, max_norm=1.0)
+    out["ms_clip_adamw"] = round((time.perf_counter() - t0) * 1e3, 2)
+    out["loss_abs_diff"] = abs(out["plain"]["loss"] - out["checkpointed"]["loss"])
+    out["peak_activation_ratio"] = round(out["plain"]["peak_activation_bytes"] / out["checkpointed"]["peak_activation_bytes"], 2)
+    out["tokens_per_s_step_checkpointed"] = round(B * T / (out["checkpointed"]["ms_fwd_bwd"] * 1e-3 + out["ms_clip_adamw"] * 1e-3), 0)
+    m.close()
+    return out
 
 
 def main():
@@ -163,8 +226,10 @@ def main():
         "kernel_ms": {n: round(t, 4) for n, t in kern_ms.items()},
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(dominant)},
     }
+    res["window_variant"] = window_variant(ops, q, k, v, d_o, out, scale, B, H, T, dk, args.warmup, max(args.steps // 2, 1))
+    res["llama_step"] = llama_step()
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(B, T, H, dk, scale)
     print(json.dumps(res), flush=True)
