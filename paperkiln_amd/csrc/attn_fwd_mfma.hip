@@ -319,7 +319,6 @@ int launch_mfma_fwd(const AttnArgs& a0, hipStream_t st) {
     static const int variant = getenv("PK_FWD_VARIANT") ? atoi(getenv("PK_FWD_VARIANT")) : 0;
     const bool big = static_cast<int64_t>(a.T) * a.Hq * a.B >= 256 * 256 * 2;
     if (a.dk_dim == 128) {
-        if (variant == 4) return launch_mfma_fwd_pipe(a, st);  // a is the copy that carries the debug pointer
         if (variant == 1) return launch<128, 1, 2>(a, st);
         if (variant == 2) return launch<128, 1, 1>(a, st);
         if (variant == 3) return launch<128, 2, 1>(a, st);

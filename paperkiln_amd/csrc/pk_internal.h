@@ -67,7 +67,6 @@ int launch_generic_bwd(const AttnArgs& a, bool bf16_in, int stages, hipStream_t 
 // attn_fwd_mfma.hip / attn_bwd_mfma.hip: bf16 MFMA kernels, head_dim 64 or 128.
 bool mfma_supported(const AttnArgs& a);
 int launch_mfma_fwd(const AttnArgs& a, hipStream_t st);
-int launch_mfma_fwd_pipe(const AttnArgs& a, hipStream_t st);
 int launch_mfma_bwd(const AttnArgs& a, int stages, hipStream_t st);
 int launch_mfma_dkdv2(const AttnArgs& a, hipStream_t st);
 
