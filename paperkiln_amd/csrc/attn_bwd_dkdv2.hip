@@ -63,7 +63,11 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
     // are taken back to back so that every workgroup carries the same work.
     const bool paired = a.causal && a.window == 0;
     int blk, rr, kvu;
-    if (!xcd_map(paired ? (nkb + 1) / 2 : nkb, 1, a.Hkv * a.B, blk, rr, kvu)) return;
+    if (a.window > 0 && a.sinks > 0 && nkb > 1) {
+        if (!xcd_map_block0_first(nkb, a.Hkv * a.B, blk, kvu)) return;
+    } else if (!xcd_map(paired ? (nkb + 1) / 2 : nkb, 1, a.Hkv * a.B, blk, rr, kvu)) {
+        return;
+    }
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv;
     const float cexp = a.scale * LOG2E;
     const int npass = (paired && blk != nkb - 1 - blk) ? 2 : 1;

@@ -139,6 +139,23 @@ __device__ inline bool xcd_map(int nblk, int rep, int kv_units, int& blk, int& r
     return kvu < kv_units;
 }
 
+// The same mapping with block 0 of EVERY unit dispatched before any other block (rep = 1). With a
+// band mask plus sink keys the workgroup that owns key block 0 walks all query tiles while the others
+// walk a handful; started last it is the tail of the launch, started first it runs beside them.
+__device__ inline bool xcd_map_block0_first(int nblk, int kv_units, int& blk, int& kvu) {
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    const int upx = (kv_units + 7) / 8;  // units per XCD
+    if (j < upx) {
+        blk = 0;
+        kvu = j * 8 + xcd;
+    } else {
+        const int jj = j - upx;
+        blk = 1 + jj % (nblk - 1);
+        kvu = (jj / (nblk - 1)) * 8 + xcd;
+    }
+    return kvu < kv_units;
+}
+
 // Branch-free visibility tests (the reference's two ranges, paperkiln
 // src/ops.cpp:879-880, 960-965). Written with non-short-circuit & and | so
 // that each element costs a few compares and one select, never a branch.
