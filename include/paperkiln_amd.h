@@ -153,6 +153,54 @@ int pk_llama_loss_backward(void* handle, const int* host_ids, const int* host_ta
 int pk_llama_adamw_step(void* handle, float lr, float b1, float b2, float eps, float wd, float max_norm,
                         float* total_norm);
 
+/* ---- block operators -------------------------------------------------------
+ * The operators of one Llama block as single calls on device memory: row-major
+ * contiguous matrices, dtype PK_F32 or PK_BF16 storage, fp32 arithmetic. They
+ * stand where the reference's devops entry points do
+ * (include/microtorch/device_cache.hpp:97-127: add, mul, scale, axpy, fill,
+ * rmsnorm_fwd, rmsnorm_bwd) and add the ones the reference still runs as host
+ * loops. Calls only enqueue on `stream` unless a host result is named. */
+int pk_op_add(const void* a, const void* b, void* y, int64_t n, int dtype, void* stream);   /* ops::add, src/ops.cpp:60-65 */
+int pk_op_mul(const void* a, const void* b, void* y, int64_t n, int dtype, void* stream);   /* ops::mul, src/ops.cpp:76-83 */
+int pk_op_scale(const void* a, float s, void* y, int64_t n, int dtype, void* stream);       /* devops::scale */
+int pk_op_axpy(void* y, float a, const void* x, int64_t n, int dtype, void* stream);        /* Variable::accumulate, src/autograd.cpp:16-24 */
+int pk_op_fill(void* y, float v, int64_t n, int dtype, void* stream);                       /* devops::fill */
+/* ops::silu and its closure (src/ops.cpp:404-424). */
+int pk_op_silu_fwd(const void* x, void* y, int64_t n, int dtype, void* stream);
+int pk_op_silu_bwd(const void* x, const void* dy, void* dx, int64_t n, int dtype, void* stream);
+/* ops::rmsnorm (src/ops.cpp:426-479; devops::rmsnorm_fwd / rmsnorm_bwd). w, rms_inv[rows] and dw are fp32;
+ * dw and dx may be NULL (the reference's want_dw / want_dx) and are overwritten, not accumulated. */
+int pk_op_rmsnorm_fwd(const void* x, const float* w, float eps, void* y, float* rms_inv, int64_t rows, int64_t cols,
+                      int dtype, void* stream);
+int pk_op_rmsnorm_bwd(const void* dy, const void* x, const float* rms_inv, const float* w, float* dw, void* dx,
+                      int64_t rows, int64_t cols, int dtype, void* stream);
+/* ops::apply_rope (src/ops.cpp:481-537) on a fused [rows, 3d] projection; pos[rows] on the device. all_heads = 0
+ * rotates only the first head of the q and k thirds, as the reference's loop does; 1 rotates every head.
+ * inverse = 1 is the backward closure. y may alias qkv. */
+int pk_op_rope(const void* qkv, const int* pos, float theta, int64_t rows, int64_t d, int head_dim, int all_heads,
+               int inverse, void* y, int dtype, void* stream);
+/* ops::embedding (src/ops.cpp:329-348): gather from an fp32 table; the backward scatter-ADDS into dtable (fp32),
+ * which the caller zeroes. ids[n] on the device; an id outside the table is the caller's to reject (the reference
+ * throws, src/ops.cpp:333). */
+int pk_op_embedding_fwd(const float* table, const int* ids, void* y, int64_t n, int64_t vocab, int64_t d, int dtype,
+                        void* stream);
+int pk_op_embedding_bwd(const void* dy, const int* ids, float* dtable, int64_t n, int64_t vocab, int64_t d, int dtype,
+                        void* stream);
+/* ops::cross_entropy (src/ops.cpp:350-376), fused: logits[rows, vocab] are REPLACED by dlogits =
+ * (P - onehot) * upstream / rows; nll_rows[rows] (device, fp32) receives -log(max(p_target, 1e-12)). When loss is
+ * non-NULL the call waits for the stream and returns the mean there (double accumulation, as the reference). */
+int pk_op_cross_entropy(void* logits, const int* targets, int64_t rows, int64_t vocab, float upstream, float* nll_rows,
+                        float* loss, int dtype, void* stream);
+/* nn::AdamW::step for one fp32 parameter at step t >= 1 (src/nn.cpp:301-321). */
+int pk_op_adamw(float* p, const float* g, float* m, float* v, int64_t n, float lr, float b1, float b2, float eps,
+                float wd, int t, void* stream);
+/* The sum of squares ops::clip_grad_norm accumulates in double (src/ops.cpp:1047-1053); waits for the stream. */
+int pk_op_sumsq(const float* g, int64_t n, double* host_out, void* stream);
+/* device::gemm (src/device.cpp:91-125; include/microtorch/device_cache.hpp:63-71): C[m,n] (+)= op(A) op(B), row-major,
+ * op = transpose when the flag is set (A is [k,m] then, B is [n,k]); operands dtype, output c_dtype, fp32 accumulate. */
+int pk_op_gemm(const void* a, int trans_a, const void* b, int trans_b, void* c, int64_t m, int64_t n, int64_t k,
+               int dtype, int c_dtype, int accumulate, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

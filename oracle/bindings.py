@@ -40,6 +40,23 @@ class Oracle:
         L.pko_attention_mask.argtypes = [sz, sz, C.c_int, _f32p]
         L.pko_visible_pairs.argtypes = [sz, C.c_int, sz, sz]
         L.pko_visible_pairs.restype = C.c_ulonglong
+        f = C.c_float
+        L.pko_rmsnorm_fwd.argtypes = [_f32p, _f32p, sz, sz, f, _f32p, _f32p]
+        L.pko_rmsnorm_fwd.restype = None
+        L.pko_rmsnorm_bwd.argtypes = [_f32p] * 4 + [sz, sz, _f32p, _f32p]
+        L.pko_rmsnorm_bwd.restype = None
+        L.pko_silu_fwd.argtypes = [_f32p, sz, _f32p]
+        L.pko_silu_fwd.restype = None
+        L.pko_silu_bwd.argtypes = [_f32p, _f32p, sz, _f32p]
+        L.pko_silu_bwd.restype = None
+        L.pko_rope.argtypes = [_f32p, _i32p, sz, sz, f, sz, C.c_int, _f32p]
+        L.pko_embedding_fwd.argtypes = [_f32p, sz, sz, _i32p, sz, _f32p]
+        L.pko_embedding_bwd.argtypes = [_f32p, _i32p, sz, sz, sz, _f32p]
+        L.pko_cross_entropy.argtypes = [_f32p, _i32p, sz, sz, _f32p, _f32p]
+        L.pko_adamw.argtypes = [_f32p, _f32p, _f32p, _f32p, sz, f, f, f, f, f, C.c_int]
+        L.pko_adamw.restype = None
+        L.pko_clip_grad_norm.argtypes = [C.POINTER(_f32p), C.POINTER(sz), sz, f]
+        L.pko_clip_grad_norm.restype = f
 
     def head_fwd(self, q, k, v, scale, seq_len=0, causal=True, window=0, sinks=0):
         q, k, v = _c(q), _c(k), _c(v)
@@ -102,6 +119,80 @@ class Oracle:
 
     def visible_pairs(self, T, causal=True, window=0, sinks=0):
         return int(self.lib.pko_visible_pairs(T, int(causal), window, sinks))
+
+    # ---- Llama block ops --------------------------------------------------
+    def rmsnorm(self, x, w, dy=None, eps=1e-5):
+        """y, rms_inv (and dx, dw when dy is given)."""
+        x, w = _c(x), _c(w).reshape(-1)
+        R, Cc = x.shape
+        y, ri = np.empty_like(x), np.empty(R, np.float32)
+        self.lib.pko_rmsnorm_fwd(_fp(x), _fp(w), R, Cc, eps, _fp(y), _fp(ri))
+        if dy is None:
+            return y, ri
+        dy = _c(dy)
+        dx, dw = np.empty_like(x), np.empty(Cc, np.float32)
+        self.lib.pko_rmsnorm_bwd(_fp(dy), _fp(x), _fp(ri), _fp(w), R, Cc, _fp(dw), _fp(dx))
+        return y, ri, dx, dw
+
+    def silu(self, x, dy=None):
+        x = _c(x)
+        y = np.empty_like(x)
+        self.lib.pko_silu_fwd(_fp(x), x.size, _fp(y))
+        if dy is None:
+            return y
+        dy = _c(dy)
+        dx = np.empty_like(x)
+        self.lib.pko_silu_bwd(_fp(x), _fp(dy), x.size, _fp(dx))
+        return y, dx
+
+    def rope(self, x, pos, theta, head_dim, inverse=False):
+        x = _c(x)
+        pos = np.ascontiguousarray(pos, np.int32)
+        y = np.empty_like(x)
+        rc = self.lib.pko_rope(_fp(x), pos.ctypes.data_as(_i32p), x.shape[0], x.shape[1], theta, head_dim,
+                               int(inverse), _fp(y))
+        if rc:
+            raise RuntimeError("apply_rope: bad cols / head_dim")
+        return y
+
+    def embedding(self, table, ids, dy=None):
+        table = _c(table)
+        ids = np.ascontiguousarray(ids, np.int32)
+        V, d = table.shape
+        y = np.empty((len(ids), d), np.float32)
+        if self.lib.pko_embedding_fwd(_fp(table), V, d, ids.ctypes.data_as(_i32p), len(ids), _fp(y)):
+            raise RuntimeError("embedding: id out of range")
+        if dy is None:
+            return y
+        dy = _c(dy)
+        dt = np.empty_like(table)
+        self.lib.pko_embedding_bwd(_fp(dy), ids.ctypes.data_as(_i32p), len(ids), V, d, _fp(dt))
+        return y, dt
+
+    def cross_entropy(self, logits, targets):
+        logits = _c(logits)
+        targets = np.ascontiguousarray(targets, np.int32)
+        loss = C.c_float()
+        dl = np.empty_like(logits)
+        rc = self.lib.pko_cross_entropy(_fp(logits), targets.ctypes.data_as(_i32p), logits.shape[0], logits.shape[1],
+                                        C.byref(loss), _fp(dl))
+        if rc:
+            raise RuntimeError("cross_entropy: target out of range")
+        return loss.value, dl
+
+    def adamw(self, p, g, m, v, lr, b1=0.9, b2=0.999, eps=1e-8, wd=0.01, t=1):
+        """Returns updated copies (p, m, v)."""
+        p, g, m, v = (_c(a).copy() for a in (p, g, m, v))
+        self.lib.pko_adamw(_fp(p), _fp(g), _fp(m), _fp(v), p.size, lr, b1, b2, eps, wd, t)
+        return p, m, v
+
+    def clip_grad_norm(self, grads, max_norm):
+        """Returns (total_norm, clipped copies)."""
+        gs = [_c(g).copy() for g in grads]
+        ptrs = (_f32p * len(gs))(*[_fp(g) for g in gs])
+        sizes = (C.c_size_t * len(gs))(*[g.size for g in gs])
+        total = self.lib.pko_clip_grad_norm(ptrs, sizes, len(gs), max_norm)
+        return float(total), gs
 
 
 class Reference:

@@ -250,3 +250,135 @@ unsigned long long pko_visible_pairs(size_t T, int causal, size_t window, size_t
     }
     return n;
 }
+
+/* ---- Llama block ops ------------------------------------------------------ */
+
+void pko_rmsnorm_fwd(const float* x, const float* w, size_t R, size_t C, float eps, float* y, float* rms_inv) {
+    for (size_t i = 0; i < R; ++i) { /* src/ops.cpp:438-444 */
+        float rms_sq = 0.0f;
+        for (size_t j = 0; j < C; ++j) rms_sq += x[i * C + j] * x[i * C + j];
+        rms_sq /= (float)C;
+        rms_inv[i] = 1.0f / sqrtf(rms_sq + eps);
+        for (size_t j = 0; j < C; ++j) y[i * C + j] = x[i * C + j] * rms_inv[i] * w[j];
+    }
+}
+
+void pko_rmsnorm_bwd(const float* dy, const float* x, const float* rms_inv, const float* w, size_t R, size_t C,
+                     float* dw, float* dx) {
+    for (size_t j = 0; j < C; ++j) dw[j] = 0.0f;
+    for (size_t i = 0; i < R; ++i) /* src/ops.cpp:457-459 */
+        for (size_t j = 0; j < C; ++j) dw[j] += dy[i * C + j] * x[i * C + j] * rms_inv[i];
+    for (size_t i = 0; i < R; ++i) { /* src/ops.cpp:466-474 */
+        float term = 0.0f;
+        for (size_t j = 0; j < C; ++j) term += dy[i * C + j] * w[j] * x[i * C + j];
+        const float ri2 = rms_inv[i] * rms_inv[i];
+        const float n_inv = 1.0f / (float)C;
+        for (size_t j = 0; j < C; ++j)
+            dx[i * C + j] = rms_inv[i] * (dy[i * C + j] * w[j] - x[i * C + j] * ri2 * term * n_inv);
+    }
+}
+
+void pko_silu_fwd(const float* x, size_t n, float* y) {
+    for (size_t i = 0; i < n; ++i) y[i] = x[i] / (1.0f + expf(-x[i])); /* src/ops.cpp:408-409 */
+}
+
+void pko_silu_bwd(const float* x, const float* dy, size_t n, float* dx) {
+    for (size_t i = 0; i < n; ++i) { /* src/ops.cpp:418-420 */
+        const float s = 1.0f / (1.0f + expf(-x[i]));
+        dx[i] = dy[i] * (s * (1.0f + x[i] * (1.0f - s)));
+    }
+}
+
+int pko_rope(const float* x, const int* pos, size_t T, size_t d3, float theta_base, size_t head_dim, int inverse,
+             float* y) {
+    if (d3 % 3 != 0) return -1;                  /* src/ops.cpp:483-485 */
+    const size_t d = d3 / 3;
+    if (head_dim % 2 != 0 || head_dim > d) return -1; /* src/ops.cpp:487-489 */
+    memcpy(y, x, T * d3 * sizeof(float));
+    for (size_t i = 0; i < T; ++i) {
+        const float m = (float)pos[i];
+        for (size_t start = 0; start < 2 * d; start += d)     /* q third, k third; v untouched */
+            for (size_t dim = 0; dim < head_dim; dim += 2) {  /* only the first head's columns, as written */
+                const float inv_freq = 1.0f / powf(theta_base, (float)dim / (float)head_dim);
+                const float th = inverse ? -m * inv_freq : m * inv_freq;
+                const float c = cosf(th), s = sinf(th);
+                const float x0 = y[i * d3 + start + dim], x1 = y[i * d3 + start + dim + 1];
+                y[i * d3 + start + dim] = x0 * c - x1 * s;
+                y[i * d3 + start + dim + 1] = x0 * s + x1 * c;
+            }
+    }
+    return 0;
+}
+
+int pko_embedding_fwd(const float* table, size_t V, size_t d, const int* ids, size_t n, float* y) {
+    for (size_t i = 0; i < n; ++i) {
+        if (ids[i] < 0 || (size_t)ids[i] >= V) return -1; /* src/ops.cpp:333-335 */
+        memcpy(y + i * d, table + (size_t)ids[i] * d, d * sizeof(float));
+    }
+    return 0;
+}
+
+int pko_embedding_bwd(const float* dy, const int* ids, size_t n, size_t V, size_t d, float* dtable) {
+    memset(dtable, 0, V * d * sizeof(float));
+    for (size_t i = 0; i < n; ++i) { /* src/ops.cpp:345-346, in id order */
+        if (ids[i] < 0 || (size_t)ids[i] >= V) return -1;
+        for (size_t j = 0; j < d; ++j) dtable[(size_t)ids[i] * d + j] += dy[i * d + j];
+    }
+    return 0;
+}
+
+int pko_cross_entropy(const float* logits, const int* targets, size_t R, size_t C, float* loss, float* dlogits) {
+    float* P = (float*)malloc(R * C * sizeof(float));
+    if (!P) return -2;
+    double nll = 0.0;
+    for (size_t i = 0; i < R; ++i) { /* components.cpp:232-250 */
+        float mx = -INFINITY;
+        for (size_t j = 0; j < C; ++j) mx = fmaxf(mx, logits[i * C + j]);
+        float sum = 0.0f;
+        for (size_t j = 0; j < C; ++j) {
+            const float e = expf(logits[i * C + j] - mx);
+            P[i * C + j] = e;
+            sum += e;
+        }
+        for (size_t j = 0; j < C; ++j) P[i * C + j] /= sum;
+        if (targets[i] < 0 || (size_t)targets[i] >= C) { /* src/ops.cpp:363-365 */
+            free(P);
+            return -1;
+        }
+        nll -= log((double)fmaxf(P[i * C + targets[i]], 1e-12f)); /* std::log(float) summed into a double */
+    }
+    *loss = (float)(nll / (double)R);
+    if (dlogits) { /* src/ops.cpp:371-374 with upstream grad 1 */
+        const float g = 1.0f / (float)R;
+        for (size_t i = 0; i < R; ++i)
+            for (size_t j = 0; j < C; ++j)
+                dlogits[i * C + j] = (P[i * C + j] - ((size_t)targets[i] == j ? 1.0f : 0.0f)) * g;
+    }
+    free(P);
+    return 0;
+}
+
+void pko_adamw(float* p, const float* g, float* m, float* v, size_t n, float lr, float b1, float b2, float eps,
+               float wd, int t) {
+    const float c1 = 1.0f - powf(b1, (float)t); /* src/nn.cpp:305-306 */
+    const float c2 = 1.0f - powf(b2, (float)t);
+    for (size_t i = 0; i < n; ++i) { /* src/nn.cpp:312-318 */
+        m[i] = b1 * m[i] + (1.0f - b1) * g[i];
+        v[i] = b2 * v[i] + (1.0f - b2) * g[i] * g[i];
+        const float update = (m[i] / c1) / (sqrtf(v[i] / c2) + eps);
+        p[i] -= lr * (update + wd * p[i]);
+    }
+}
+
+float pko_clip_grad_norm(float* const* grads, const size_t* sizes, size_t nparams, float max_norm) {
+    double sq = 0.0; /* src/ops.cpp:1047-1053 */
+    for (size_t k = 0; k < nparams; ++k)
+        for (size_t i = 0; i < sizes[k]; ++i) sq += (double)grads[k][i] * grads[k][i];
+    const float total = (float)sqrt(sq);
+    if (total > max_norm && total > 0.0f) { /* src/ops.cpp:1055-1062 */
+        const float scale = max_norm / total;
+        for (size_t k = 0; k < nparams; ++k)
+            for (size_t i = 0; i < sizes[k]; ++i) grads[k][i] *= scale;
+    }
+    return total;
+}

@@ -64,6 +64,38 @@ int pko_attention_mask(size_t rows, size_t seq_len, int causal, float* out);
  * the band count of src/ops.cpp:960-965. */
 unsigned long long pko_visible_pairs(size_t T, int causal, size_t window, size_t sinks);
 
+/* ---- Llama block ops (fp32, the reference's loop order) ------------------
+ * Pinned by tests/test_oracle_blockops.py: against vectors written by the
+ * compiled reference (tests/golden/blockops_fp32.npz), against the compiled
+ * reference itself where it is present, and against fp64 finite differences
+ * and closed forms. AdamW and clip_grad_norm are pinned by the parameters the
+ * reference's own optimiser produced (tests/golden/llama_*.npz). */
+
+/* ops::rmsnorm forward (src/ops.cpp:437-445): y = x * rms_inv * w, rms_inv = 1/sqrt(mean(x^2)+eps). */
+void pko_rmsnorm_fwd(const float* x, const float* w, size_t R, size_t C, float eps, float* y, float* rms_inv);
+/* its backward (src/ops.cpp:447-478); dw and dx are overwritten. */
+void pko_rmsnorm_bwd(const float* dy, const float* x, const float* rms_inv, const float* w, size_t R, size_t C,
+                     float* dw, float* dx);
+/* ops::silu (src/ops.cpp:404-424). */
+void pko_silu_fwd(const float* x, size_t n, float* y);
+void pko_silu_bwd(const float* x, const float* dy, size_t n, float* dx);
+/* ops::apply_rope (src/ops.cpp:481-537) on a fused [T, 3d] matrix: adjacent pairs of the FIRST head_dim
+ * columns of the q third and of the k third are rotated (the reference's loop never reaches the other
+ * heads); inverse != 0 is the backward. Returns -1 on the reference's argument errors. */
+int pko_rope(const float* x, const int* pos, size_t T, size_t d3, float theta, size_t head_dim, int inverse,
+             float* y);
+/* ops::embedding (src/ops.cpp:329-348): gather; backward scatter-adds into a zeroed table. -1 = id out of range. */
+int pko_embedding_fwd(const float* table, size_t V, size_t d, const int* ids, size_t n, float* y);
+int pko_embedding_bwd(const float* dy, const int* ids, size_t n, size_t V, size_t d, float* dtable);
+/* ops::cross_entropy (src/ops.cpp:350-376) with Matrix::apply_softmax (components.cpp:229-251): mean NLL with
+ * the max(p, 1e-12) clamp, double accumulation; dlogits = (P - onehot) / R. -1 = target out of range. */
+int pko_cross_entropy(const float* logits, const int* targets, size_t R, size_t C, float* loss, float* dlogits);
+/* nn::AdamW::step for one parameter at step t >= 1 (src/nn.cpp:301-321). */
+void pko_adamw(float* p, const float* g, float* m, float* v, size_t n, float lr, float b1, float b2, float eps,
+               float wd, int t);
+/* ops::clip_grad_norm over a list of gradients (src/ops.cpp:1046-1064); returns the norm before clipping. */
+float pko_clip_grad_norm(float* const* grads, const size_t* sizes, size_t nparams, float max_norm);
+
 #ifdef __cplusplus
 }
 #endif

@@ -49,7 +49,10 @@ _lib = None
 EXPORTS = ["pk_last_error", "pk_init", "pk_attn_fwd", "pk_attn_bwd_workspace_bytes", "pk_attn_bwd", "pk_attn_bwd_stages",
            "pk_alloc", "pk_free", "pk_live_bytes", "pk_peak_bytes", "pk_reset_peak", "pk_trim",
            "pk_llama_create", "pk_llama_destroy", "pk_llama_num_params", "pk_llama_param_info", "pk_llama_set_param",
-           "pk_llama_get_param", "pk_llama_get_grad", "pk_llama_loss_backward", "pk_llama_adamw_step"]
+           "pk_llama_get_param", "pk_llama_get_grad", "pk_llama_loss_backward", "pk_llama_adamw_step",
+           "pk_op_add", "pk_op_mul", "pk_op_scale", "pk_op_axpy", "pk_op_fill", "pk_op_silu_fwd", "pk_op_silu_bwd",
+           "pk_op_rmsnorm_fwd", "pk_op_rmsnorm_bwd", "pk_op_rope", "pk_op_embedding_fwd", "pk_op_embedding_bwd",
+           "pk_op_cross_entropy", "pk_op_adamw", "pk_op_sumsq", "pk_op_gemm"]
 
 
 def lib() -> C.CDLL:
@@ -87,6 +90,23 @@ def lib() -> C.CDLL:
         L.pk_llama_loss_backward.argtypes = [C.c_void_p, i32p, i32p, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int,
                                              f32p, C.POINTER(LlamaStats), C.c_void_p]
         L.pk_llama_adamw_step.argtypes = [C.c_void_p] + [C.c_float] * 6 + [f32p]
+        vp, i64, ci, cf = C.c_void_p, C.c_int64, C.c_int, C.c_float
+        L.pk_op_add.argtypes = [vp, vp, vp, i64, ci, vp]
+        L.pk_op_mul.argtypes = [vp, vp, vp, i64, ci, vp]
+        L.pk_op_scale.argtypes = [vp, cf, vp, i64, ci, vp]
+        L.pk_op_axpy.argtypes = [vp, cf, vp, i64, ci, vp]
+        L.pk_op_fill.argtypes = [vp, cf, i64, ci, vp]
+        L.pk_op_silu_fwd.argtypes = [vp, vp, i64, ci, vp]
+        L.pk_op_silu_bwd.argtypes = [vp, vp, vp, i64, ci, vp]
+        L.pk_op_rmsnorm_fwd.argtypes = [vp, vp, cf, vp, vp, i64, i64, ci, vp]
+        L.pk_op_rmsnorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, ci, vp]
+        L.pk_op_rope.argtypes = [vp, vp, cf, i64, i64, ci, ci, ci, vp, ci, vp]
+        L.pk_op_embedding_fwd.argtypes = [vp, vp, vp, i64, i64, i64, ci, vp]
+        L.pk_op_embedding_bwd.argtypes = [vp, vp, vp, i64, i64, i64, ci, vp]
+        L.pk_op_cross_entropy.argtypes = [vp, vp, i64, i64, cf, vp, f32p, ci, vp]
+        L.pk_op_adamw.argtypes = [vp, vp, vp, vp, i64, cf, cf, cf, cf, cf, ci, vp]
+        L.pk_op_sumsq.argtypes = [vp, i64, C.POINTER(C.c_double), vp]
+        L.pk_op_gemm.argtypes = [vp, ci, vp, ci, vp, i64, i64, i64, ci, ci, ci, vp]
         _lib = L
     return _lib
 

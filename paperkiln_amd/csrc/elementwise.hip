@@ -6,6 +6,7 @@
 #include <rocblas/rocblas.h>
 
 #include <map>
+#include <cmath>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
@@ -217,9 +218,16 @@ __global__ void colsum_parts(const float* part, float* dw, int nparts, int C) {
 }
 
 // apply_rope (ops.cpp:497-509 forward, :519-533 backward = rotation by -theta).
+// The inverse frequencies come from the host, computed with the reference's own expression
+// 1 / pow(theta, dim / head_dim): the angle pos * inv_freq is then the same fp32 number the
+// reference feeds to cos / sin. An inv_freq one ulp off would be amplified by the position.
+constexpr int ROPE_MAX_PAIRS = 128;  // head_dim <= 256
+struct RopeFreq {
+    float f[ROPE_MAX_PAIRS];
+};
 template <typename T>
-__global__ void rope_k(const T* x, const int* pos, float theta_base, int d, int head_dim, int rot_heads, float sign,
-                       T* y, int64_t N) {
+__global__ void rope_k(const T* x, const int* pos, RopeFreq freq, int d, int head_dim, int rot_heads, float sign, T* y,
+                       int64_t N) {
     const int d3 = 3 * d;
     for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < N * (d3 / 2);
          i += static_cast<int64_t>(gridDim.x) * NT) {
@@ -229,8 +237,7 @@ __global__ void rope_k(const T* x, const int* pos, float theta_base, int d, int 
         float x0 = ldf(x, row * d3 + c), x1 = ldf(x, row * d3 + c + 1);
         if (third < 2 && within < rot_heads * head_dim) {
             const int dim = within % head_dim;
-            const float inv_freq = 1.0f / powf(theta_base, static_cast<float>(dim) / head_dim);
-            const float th = sign * static_cast<float>(pos[row]) * inv_freq;
+            const float th = sign * static_cast<float>(pos[row]) * freq.f[dim >> 1];
             const float c_ = cosf(th), s_ = sinf(th);
             const float r0 = x0 * c_ - x1 * s_, r1 = x0 * s_ + x1 * c_;
             x0 = r0;
@@ -415,8 +422,12 @@ void k_rope(const Tensor& x, const int* pos, float theta, int d, int head_dim, i
             const Tensor& y) {
     if (x.cols != 3 * d) throw std::runtime_error("apply_rope: cols must be divisible by 3");
     if (head_dim % 2 != 0 || head_dim > d) throw std::runtime_error("apply_rope: head_dim must be even and <= d");
+    if (head_dim > 2 * ROPE_MAX_PAIRS) throw std::runtime_error("apply_rope: head_dim above 256 is not supported");
+    RopeFreq freq;
+    for (int dim = 0; dim < head_dim; dim += 2)  // ops.cpp:499-500
+        freq.f[dim >> 1] = 1.0f / std::pow(theta, static_cast<float>(dim) / static_cast<float>(head_dim));
     PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((rope_k<T>), ew_grid(x.numel() / 2), dim3(NT), 0, tape_stream(),
-                                                static_cast<const T*>(x.ptr()), pos, theta, d, head_dim, rot_heads,
+                                                static_cast<const T*>(x.ptr()), pos, freq, d, head_dim, rot_heads,
                                                 inverse ? -1.0f : 1.0f, static_cast<T*>(y.ptr()), x.rows));
     post();
 }

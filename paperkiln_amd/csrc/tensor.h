@@ -31,8 +31,12 @@ void dev_trim();  // return cached blocks to the driver
 struct Buffer {
     void* p = nullptr;
     size_t bytes = 0;
+    bool owned = true;
     explicit Buffer(size_t n) : p(dev_alloc(n)), bytes(n) {}
-    ~Buffer() { dev_free(p); }
+    Buffer(void* caller_memory, size_t n) : p(caller_memory), bytes(n), owned(false) {}  // a view of caller memory
+    ~Buffer() {
+        if (owned) dev_free(p);
+    }
     Buffer(const Buffer&) = delete;
     Buffer& operator=(const Buffer&) = delete;
 };
@@ -55,6 +59,17 @@ struct Tensor {
         t.cols = c;
         t.dtype = dt;
         t.buf = std::make_shared<Buffer>(static_cast<size_t>(r) * c * (dt == PK_F32 ? 4 : 2));
+        return t;
+    }
+    static Tensor borrow(const void* p, int64_t r, int64_t c, int dt) {  // caller-owned device memory, never freed here
+        if (!p) throw std::runtime_error("null device pointer");
+        if (r <= 0 || c <= 0) throw std::runtime_error("Matrix: zero dimension");
+        if (dt != PK_F32 && dt != PK_BF16) throw std::runtime_error("unknown element type");
+        Tensor t;
+        t.rows = r;
+        t.cols = c;
+        t.dtype = dt;
+        t.buf = std::make_shared<Buffer>(const_cast<void*>(p), static_cast<size_t>(r) * c * (dt == PK_F32 ? 4 : 2));
         return t;
     }
     Tensor row_range(int64_t r0, int64_t n) const {  // rows [r0, r0+n) of this matrix, no copy

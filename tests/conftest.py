@@ -39,7 +39,8 @@ def reference():
 
 def golden_names():
     names = sorted(os.path.splitext(os.path.basename(p))[0] for p in glob.glob(os.path.join(GOLDEN, "*.npz")))
-    return [n for n in names if not n.startswith("llama_")]  # model-level vectors have their own loader
+    # model-level and block-op vectors have their own loaders
+    return [n for n in names if not n.startswith(("llama_", "blockops_"))]
 
 
 class Golden:

@@ -1,0 +1,185 @@
+"""GPU parity of the Llama block operators (pk_op_* through the C ABI) against
+the vectors the compiled reference wrote (tests/golden/blockops_fp32.npz,
+llama_*.npz) and against the CPU oracle on other seeded inputs.
+
+Bars: fp32 storage max-abs 1e-5 (relative to the largest expected magnitude
+where values exceed 1: row reductions run in a different order); bf16 storage
+2e-2 against the oracle run on the same bf16-rounded inputs.
+"""
+from __future__ import annotations
+
+import os
+
+import numpy as np
+import pytest
+
+from paperkiln_amd import synth
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+F32_TOL = 1e-5
+BF16_TOL = 2e-2
+
+
+@pytest.fixture(scope="module")
+def bo():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    from paperkiln_amd import _lib, blockops
+    _lib.check(_lib.lib().pk_init(0, None, 0))
+    return blockops
+
+
+@pytest.fixture(scope="module")
+def vec():
+    return np.load(os.path.join(GOLDEN, "blockops_fp32.npz"))
+
+
+def dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    return t.to(dtype) if dtype is not None else t
+
+
+def host(t):
+    return t.float().cpu().numpy()
+
+
+def close(got, want, tol):
+    want = np.asarray(want, np.float64)
+    err = np.abs(host(got).astype(np.float64) - want).max()
+    assert err <= tol * max(1.0, np.abs(want).max()), err
+
+
+def test_rmsnorm_fp32_vs_reference_vectors(bo, vec):
+    y, dx, dw = bo.rmsnorm(dev(vec["rms_x"]), dev(vec["rms_w"]), dev(vec["rms_dy"]))
+    close(y, vec["rms_y"], F32_TOL)
+    close(dx, vec["rms_dx"], F32_TOL)
+    close(dw, vec["rms_dw"], F32_TOL)
+
+
+def test_silu_fp32_vs_reference_vectors(bo, vec):
+    y, dx = bo.silu(dev(vec["silu_x"]), dev(vec["silu_dy"]))
+    close(y, vec["silu_y"], F32_TOL)
+    close(dx, vec["silu_dx"], F32_TOL)
+
+
+def test_rope_fp32_vs_reference_vectors(bo, vec):
+    th, hd = float(vec["rope_theta"]), int(vec["rope_head_dim"])
+    pos = dev(vec["rope_pos"])
+    close(bo.apply_rope(dev(vec["rope_x"]), pos, th, hd), vec["rope_y"], F32_TOL)
+    close(bo.apply_rope(dev(vec["rope_dy"]), pos, th, hd, inverse=True), vec["rope_dx"], F32_TOL)
+
+
+def test_rope_all_heads_switch(bo, oracle, vec):
+    """all_heads=True rotates every head the way the first one is rotated; the default leaves them alone."""
+    th, hd = float(vec["rope_theta"]), int(vec["rope_head_dim"])
+    x, pos = vec["rope_x"], vec["rope_pos"]
+    d = x.shape[1] // 3
+    want = x.copy()
+    for third in (0, 1):
+        for h in range(d // hd):
+            blk = np.zeros_like(x)
+            c0 = third * d + h * hd
+            blk[:, :hd] = x[:, c0:c0 + hd]  # put the head where the reference's loop rotates
+            want[:, c0:c0 + hd] = oracle.rope(blk, pos, th, hd)[:, :hd]
+    close(bo.apply_rope(dev(x), dev(pos), th, hd, all_heads=True), want, F32_TOL)
+
+
+def test_cross_entropy_fp32_vs_reference_vectors(bo, vec):
+    loss, dl = bo.cross_entropy(dev(vec["ce_logits"]), dev(vec["ce_targets"]))
+    assert abs(loss - float(vec["ce_loss"])) < 1e-5 * abs(float(vec["ce_loss"]))
+    close(dl, vec["ce_dlogits"], F32_TOL)
+
+
+def test_embedding_vs_reference_vectors(bo, vec):
+    y, dt = bo.embedding(dev(vec["emb_table"]), dev(vec["emb_ids"]), dev(vec["emb_dy"]))
+    assert np.array_equal(host(y), vec["emb_y"])
+    close(dt, vec["emb_dtable"], F32_TOL)
+
+
+@pytest.mark.parametrize("name", ["llama_T16_single"])
+def test_clip_and_adamw_vs_reference_optimiser(bo, name):
+    z = np.load(os.path.join(GOLDEN, name + ".npz"))
+    names = [k[2:] for k in z.files if k.startswith("p:")]
+    grads = [dev(z["g:" + n]).reshape(-1).contiguous() for n in names]
+    total = bo.clip_grad_norm_(grads, 1.0)
+    assert abs(total - float(z["total_norm"])) < 1e-5 * float(z["total_norm"])
+    worst = 0.0
+    for n, g in zip(names, grads):
+        p = dev(z["p:" + n]).reshape(-1).contiguous()
+        bo.adamw_(p, g, torch.zeros_like(p), torch.zeros_like(p), lr=3e-3, t=1)
+        ok = np.abs(host(g)) > 1e-5  # the first Adam step is g/(|g|+eps): ill-conditioned at |g| ~ eps
+        worst = max(worst, np.abs(host(p) - z["a:" + n].reshape(-1))[ok].max())
+    assert worst < F32_TOL, worst
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", F32_TOL), ("bfloat16", BF16_TOL)])
+def test_block_ops_vs_oracle_larger(bo, oracle, dtype, tol):
+    """Shapes of a real block (rows not a multiple of the kernels' row groups), both storage types."""
+    td = getattr(torch, dtype)
+    rnd = (lambda a: synth.bf16_round(a)) if dtype == "bfloat16" else (lambda a: a)
+    R, Cc = 301, 512
+    x, dy = rnd(synth.randn(401, (R, Cc), 1.5)), rnd(synth.randn(402, (R, Cc), 1.0))
+    w = (1.0 + 0.2 * synth.randn(403, (Cc,), 1.0)).astype(np.float32)
+    wy, _, wdx, wdw = oracle.rmsnorm(x, w, dy)
+    y, dx, dw = bo.rmsnorm(dev(x, td), dev(w), dev(dy, td))
+    close(y, wy, tol), close(dx, wdx, tol)
+    close(dw, wdw, tol if dtype == "float32" else 5e-2)  # a 301-term column sum of bf16-rounded products
+    wy, wdx = oracle.silu(x, dy)
+    y, dx = bo.silu(dev(x, td), dev(dy, td))
+    close(y, wy, tol), close(dx, wdx, tol)
+    a, b = rnd(synth.randn(404, (R, Cc), 1.0)), rnd(synth.randn(405, (R, Cc), 1.0))
+    close(bo.add(dev(a, td), dev(b, td)), a + b, tol)
+    close(bo.mul(dev(a, td), dev(b, td)), a * b, tol)
+    close(bo.scale(dev(a, td), 0.37), a * np.float32(0.37), tol)
+    close(bo.axpy_(dev(a, td), -1.5, dev(b, td)), a + np.float32(-1.5) * b, tol)
+    assert float(bo.fill_(dev(a, td), 2.5).float().min()) == 2.5
+    # rope on a Llama-shaped fused projection: 2 x 150 positions, d = 512, head_dim = 64
+    qkv = rnd(synth.randn(406, (300, 3 * 512), 1.0))
+    pos = np.concatenate([np.arange(150), np.arange(150)]).astype(np.int32)
+    close(bo.apply_rope(dev(qkv, td), dev(pos), 10000.0, 64), oracle.rope(qkv, pos, 10000.0, 64), tol)
+    # cross entropy over a 1000-word vocabulary
+    lg = rnd(synth.randn(407, (97, 1000), 2.0))
+    t = synth.randint(408, 97, 1000).astype(np.int32)
+    wl, wdl = oracle.cross_entropy(lg, t)
+    loss, dl = bo.cross_entropy(dev(lg, td), dev(t))
+    assert abs(loss - wl) < (1e-5 if dtype == "float32" else 1e-3) * abs(wl)
+    close(dl, wdl, tol if dtype == "float32" else 1e-3)  # |dlogits| <= 1/97
+    # embedding into either storage type
+    table = synth.randn(409, (500, 64), 0.5)
+    ids = synth.randint(410, 333, 500).astype(np.int32)
+    g = rnd(synth.randn(411, (333, 64), 1.0))
+    wy, wdt = oracle.embedding(table, ids, g)
+    y, dt = bo.embedding(dev(table), dev(ids), dev(g, td), dtype=td)
+    close(y, rnd(wy), tol), close(dt, wdt, 1e-5)
+
+
+def test_matmul_vs_numpy(bo):
+    a, b = synth.randn(421, (65, 130), 1.0), synth.randn(422, (130, 47), 1.0)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    close(bo.matmul(dev(a), dev(b)), want, 2e-5)
+    close(bo.matmul(dev(a.T.copy()), dev(b), trans_a=True), want, 2e-5)
+    close(bo.matmul(dev(a), dev(b.T.copy()), trans_b=True), want, 2e-5)
+    ab, bb = synth.bf16_round(a), synth.bf16_round(b)
+    close(bo.matmul(dev(ab, torch.bfloat16), dev(bb, torch.bfloat16), out_dtype=torch.float32),
+          ab.astype(np.float64) @ bb.astype(np.float64), 2e-5)
+    with pytest.raises(RuntimeError):
+        bo.matmul(dev(a), dev(a))
+
+
+def test_error_behaviour(bo):
+    x = dev(synth.randn(431, (4, 8), 1.0))
+    with pytest.raises(RuntimeError):
+        bo.rmsnorm(x, dev(np.ones(7, np.float32)))
+    with pytest.raises(RuntimeError):
+        bo.apply_rope(x, dev(np.arange(4, dtype=np.int32)), 10000.0, 2)  # 8 columns: not divisible by 3
+    with pytest.raises(RuntimeError):
+        bo.apply_rope(dev(synth.randn(432, (4, 12), 1.0)), dev(np.arange(4, dtype=np.int32)), 10000.0, 3)  # odd head_dim
+    with pytest.raises(RuntimeError):
+        bo.embedding(x, dev(np.array([4], np.int32)))
+    with pytest.raises(RuntimeError):
+        bo.cross_entropy(x, dev(np.array([0, 1, 8, 2], np.int32)))
+    with pytest.raises(RuntimeError):
+        bo.add(x, dev(synth.randn(433, (4, 9), 1.0)))
