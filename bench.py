@@ -140,6 +140,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--sections", default="window,llama",
+                    help="extra measurements beside the headline: any of window,llama (empty = headline only, "
+                         "which is what the profiles under profiles/ were taken with)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (one process, one MI355X); --gpus must be 1. "
@@ -228,8 +231,12 @@ def main():
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(dominant)},
     }
-    res["window_variant"] = window_variant(ops, q, k, v, d_o, out, scale, B, H, T, dk, args.warmup, max(args.steps // 2, 1))
-    res["llama_step"] = llama_step()
+    extras = [x for x in args.sections.split(",") if x]
+    if "window" in extras:
+        res["window_variant"] = window_variant(ops, q, k, v, d_o, out, scale, B, H, T, dk, args.warmup,
+                                               max(args.steps // 2, 1))
+    if "llama" in extras:
+        res["llama_step"] = llama_step()
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(B, T, H, dk, scale)
     print(json.dumps(res), flush=True)
