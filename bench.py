@@ -124,9 +124,11 @@ def llama_step():
                     "peak_activation_bytes": st["peak_activation_bytes"],
                     "activation_bytes_after_forward": st["activation_bytes_after_forward"],
                     "live_vars_after_forward": st["live_vars_after_forward"]}
+    m.adamw_step(1e-3, max_norm=1.0)  # the first step also allocates the moments
     t0 = time.perf_counter()
-    m.adamw_step(1e-3, max_norm=1.0)
-    out["ms_clip_adamw"] = round((time.perf_counter() - t0) * 1e3, 2)
+    for _ in range(3):
+        m.adamw_step(1e-3, max_norm=1.0)
+    out["ms_clip_adamw"] = round((time.perf_counter() - t0) / 3 * 1e3, 2)
     out["loss_abs_diff"] = abs(out["plain"]["loss"] - out["checkpointed"]["loss"])
     out["peak_activation_ratio"] = round(out["plain"]["peak_activation_bytes"] / out["checkpointed"]["peak_activation_bytes"], 2)
     out["tokens_per_s_step_checkpointed"] = round(B * T / (out["checkpointed"]["ms_fwd_bwd"] * 1e-3 + out["ms_clip_adamw"] * 1e-3), 0)

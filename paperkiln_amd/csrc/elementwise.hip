@@ -11,6 +11,7 @@
 #include <unordered_map>
 #include <vector>
 
+#include "mfma_common.h"
 #include "tensor.h"
 
 namespace pk {
@@ -199,7 +200,7 @@ __global__ void rms_bwd_dx(const T* dy, const T* x, const float* rinv, const flo
 }
 // dw_j = sum_i dY_ij x_ij rinv_i, in two deterministic stages: each block sums
 // ROWS_PB rows into part[block][C], then one block per column chunk adds the parts.
-constexpr int ROWS_PB = 128;
+constexpr int ROWS_PB = 32;  // 8192 rows -> 256 blocks, one per CU
 template <typename T>
 __global__ void rms_bwd_dw_part(const T* dy, const T* x, const float* rinv, float* part, int64_t R, int C) {
     const int64_t r0 = static_cast<int64_t>(blockIdx.x) * ROWS_PB;
@@ -210,11 +211,23 @@ __global__ void rms_bwd_dw_part(const T* dy, const T* x, const float* rinv, floa
     }
 }
 __global__ void colsum_parts(const float* part, float* dw, int nparts, int C) {
-    const int j = blockIdx.x * NT + threadIdx.x;
-    if (j >= C) return;
+    // 64 columns x 4 groups of parts per block; the groups meet in a fixed order
+    __shared__ float sh[4][64];
+    const int col = blockIdx.x * 64 + (threadIdx.x & 63), grp = threadIdx.x >> 6;
     float s = 0.0f;
-    for (int p = 0; p < nparts; ++p) s += part[static_cast<int64_t>(p) * C + j];
-    dw[j] += s;
+    if (col < C)
+        for (int p = grp; p < nparts; p += 4) s += part[static_cast<int64_t>(p) * C + col];
+    sh[grp][threadIdx.x & 63] = s;
+    __syncthreads();
+    if (grp == 0 && col < C) dw[col] += (sh[0][threadIdx.x] + sh[1][threadIdx.x]) + (sh[2][threadIdx.x] + sh[3][threadIdx.x]);
+}
+// dst[i] += sum_s part[s][i], parts added in index order
+__global__ void add_parts(const float* part, float* dst, int nparts, int64_t n) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT) {
+        float s = 0.0f;
+        for (int p = 0; p < nparts; ++p) s += part[p * n + i];
+        dst[i] += s;
+    }
 }
 
 // apply_rope (ops.cpp:497-509 forward, :519-533 backward = rotation by -theta).
@@ -290,6 +303,75 @@ __global__ void ce_rows(T* logits, const int* targets, float gscale, float* nll,
     for (int j = threadIdx.x; j < C; j += NT) {
         const float p = expf(ldf(row, j) - mx) * inv;
         stf(row, j, (p - (j == t ? 1.0f : 0.0f)) * gscale);
+    }
+}
+
+// The same row operation for the chunked head (fp32 logits, vocabulary a multiple of 4 and at most
+// 32768): 1024 threads hold the whole row in registers, so the logits are read ONCE; the forward pass
+// writes nothing but the row's nll, the backward writes dlogits straight in the GEMM's operand type.
+constexpr int CE_NT = 1024, CE_V4 = 8;  // 8 float4 per thread
+template <typename TOut, bool WRITE>
+__global__ __launch_bounds__(CE_NT) void ce_rows_reg(const float* logits, TOut* dl, const int* targets, float gscale,
+                                                     float* nll, int C) {
+    __shared__ float sh[CE_NT / 64];
+    const float* row = logits + static_cast<int64_t>(blockIdx.x) * C;
+    const int t = targets[blockIdx.x];
+    f32x4 v[CE_V4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < CE_V4; ++i) {
+        const int j = (threadIdx.x + i * CE_NT) * 4;
+        if (j < C) {
+            v[i] = *reinterpret_cast<const f32x4*>(row + j);
+            mx = fmaxf(fmaxf(mx, fmaxf(v[i][0], v[i][1])), fmaxf(v[i][2], v[i][3]));
+        }
+    }
+    auto reduce = [&](float x, bool is_max) {
+        for (int o = 32; o >= 1; o >>= 1) {
+            const float y = __shfl_xor(x, o);
+            x = is_max ? fmaxf(x, y) : x + y;
+        }
+        __syncthreads();  // sh is reused
+        if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = x;
+        __syncthreads();
+        float r = sh[0];
+        for (int w = 1; w < CE_NT / 64; ++w) r = is_max ? fmaxf(r, sh[w]) : r + sh[w];
+        return r;
+    };
+    mx = reduce(mx, true);
+    float z = 0.0f;
+#pragma unroll
+    for (int i = 0; i < CE_V4; ++i) {
+        const int j = (threadIdx.x + i * CE_NT) * 4;
+        if (j < C) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[i][e] = expf(v[i][e] - mx);
+                z += v[i][e];
+            }
+        }
+    }
+    z = reduce(z, false);
+    const float inv = 1.0f / z;
+#pragma unroll
+    for (int i = 0; i < CE_V4; ++i) {
+        const int j = (threadIdx.x + i * CE_NT) * 4;
+        if (j < C) {
+            if (t >= j && t < j + 4) nll[blockIdx.x] = -logf(fmaxf(v[i][t - j] * inv, 1e-12f));
+            if (WRITE) {
+                float o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (v[i][e] * inv - (j + e == t ? 1.0f : 0.0f)) * gscale;
+                TOut* dst = dl + static_cast<int64_t>(blockIdx.x) * C + j;
+                if (sizeof(TOut) == 4) {
+                    f32x4 w = {o[0], o[1], o[2], o[3]};
+                    *reinterpret_cast<f32x4*>(dst) = w;
+                } else {
+                    u32x2 w = {pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3])};
+                    *reinterpret_cast<u32x2*>(dst) = w;
+                }
+            }
+        }
     }
 }
 
@@ -413,7 +495,7 @@ void k_rmsnorm_bwd(const Tensor& dy, const Tensor& x, const float* rinv, const T
                                                     static_cast<const T*>(dy.ptr()), static_cast<const T*>(x.ptr()), rinv,
                                                     static_cast<float*>(part.p), x.rows, C));
         post();
-        hipLaunchKernelGGL(colsum_parts, dim3((C + NT - 1) / NT), dim3(NT), 0, tape_stream(),
+        hipLaunchKernelGGL(colsum_parts, dim3((C + 63) / 64), dim3(NT), 0, tape_stream(),
                            static_cast<const float*>(part.p), static_cast<float*>(dw->ptr()), nparts, C);
         post();
     }
@@ -449,6 +531,23 @@ void k_ce_rows(const Tensor& logits, const int* targets, float gscale, float* nl
                                                      static_cast<int>(logits.cols)));
     post();
 }
+bool k_ce_rows_once(const Tensor& logits, const int* targets, float gscale, float* nll_rows, const Tensor* dl) {
+    const int C = static_cast<int>(logits.cols);
+    if (logits.dtype != PK_F32 || C % 4 != 0 || C > CE_NT * CE_V4 * 4) return false;  // caller takes the generic kernel
+    const float* src = static_cast<const float*>(logits.ptr());
+    if (!dl) {
+        hipLaunchKernelGGL((ce_rows_reg<float, false>), dim3(logits.rows), dim3(CE_NT), 0, tape_stream(), src,
+                           static_cast<float*>(nullptr), targets, gscale, nll_rows, C);
+    } else if (dl->dtype == PK_F32) {
+        hipLaunchKernelGGL((ce_rows_reg<float, true>), dim3(logits.rows), dim3(CE_NT), 0, tape_stream(), src,
+                           static_cast<float*>(dl->ptr()), targets, gscale, nll_rows, C);
+    } else {
+        hipLaunchKernelGGL((ce_rows_reg<uint16_t, true>), dim3(logits.rows), dim3(CE_NT), 0, tape_stream(), src,
+                           static_cast<uint16_t*>(dl->ptr()), targets, gscale, nll_rows, C);
+    }
+    post();
+    return true;
+}
 double k_sum_f32_to_host(const float* x, int64_t n) {
     Buffer out(sizeof(double));
     hipLaunchKernelGGL(sum_f32_k, dim3(1), dim3(NT), 0, tape_stream(), x, n, static_cast<double*>(out.p));
@@ -458,19 +557,26 @@ double k_sum_f32_to_host(const float* x, int64_t n) {
     HIPCHK(hipStreamSynchronize(tape_stream()));
     return h;
 }
-double k_sumsq_to_host(const Tensor& g) {
+int k_sumsq_parts(const Tensor& g, double* part_dev) {
     if (g.dtype != PK_F32) throw std::runtime_error("clip_grad_norm: gradients must be fp32");
-    const int nb = static_cast<int>(std::min<int64_t>((g.numel() + NT - 1) / NT, 1024));
-    Buffer part(sizeof(double) * nb);
+    const int nb = static_cast<int>(std::min<int64_t>((g.numel() + NT - 1) / NT, SUMSQ_MAX_PARTS));
     hipLaunchKernelGGL(sumsq_part, dim3(nb), dim3(NT), 0, tape_stream(), static_cast<const float*>(g.ptr()), g.numel(),
-                       static_cast<double*>(part.p));
+                       part_dev);
     post();
-    std::vector<double> h(nb);
-    HIPCHK(hipMemcpyAsync(h.data(), part.p, sizeof(double) * nb, hipMemcpyDeviceToHost, tape_stream()));
+    return nb;
+}
+double k_sum_f64_to_host(const double* part_dev, int64_t n) {
+    std::vector<double> h(n);
+    HIPCHK(hipMemcpyAsync(h.data(), part_dev, sizeof(double) * n, hipMemcpyDeviceToHost, tape_stream()));
     HIPCHK(hipStreamSynchronize(tape_stream()));
     double s = 0.0;
     for (double v : h) s += v;
     return s;
+}
+double k_sumsq_to_host(const Tensor& g) {
+    Buffer part(sizeof(double) * SUMSQ_MAX_PARTS);
+    const int nb = k_sumsq_parts(g, static_cast<double*>(part.p));
+    return k_sum_f64_to_host(static_cast<const double*>(part.p), nb);
 }
 void k_adamw(const Tensor& p, const Tensor& g, const Tensor& m, const Tensor& v, float lr, float b1, float b2,
              float eps, float wd, float c1, float c2) {
@@ -506,6 +612,31 @@ void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dty
     const rocblas_datatype ct = c_dtype == PK_F32 ? rocblas_datatype_f32_r : rocblas_datatype_bf16_r;
     const float alpha = 1.0f;
     rocblas_set_stream(blas(), tape_stream());
+    // Weight gradients (X^T dY accumulated into an fp32 matrix): the contraction runs over every token while
+    // the output is a few hundred tiles at most, so one GEMM leaves most of the chip idle. The token axis is
+    // cut into slices that run as one strided-batched GEMM into separate partial products, which are then
+    // added in slice order: no atomics, so the sum is the same on every run.
+    if (tA && !tB && c_dtype == PK_F32 && beta == 1.0f && ldc == N && Ka >= 2048 && M * N <= (int64_t{1} << 21)) {
+        int S = 8;
+        while (S > 1 && (Ka % S != 0 || Ka / S < 256)) S >>= 1;
+        if (S > 1) {
+            const int64_t Ks = Ka / S;
+            Buffer part(sizeof(float) * static_cast<size_t>(S) * M * N);
+            const float zero = 0.0f;
+            const rocblas_status st = rocblas_gemm_strided_batched_ex(
+                blas(), rocblas_operation_none, rocblas_operation_transpose, static_cast<rocblas_int>(N),
+                static_cast<rocblas_int>(M), static_cast<rocblas_int>(Ks), &alpha, B.ptr(), ab,
+                static_cast<rocblas_int>(B.cols), Ks * B.cols, A.ptr(), ab, static_cast<rocblas_int>(A.cols), Ks * A.cols, &zero,
+                part.p, rocblas_datatype_f32_r, static_cast<rocblas_int>(N), M * N, part.p, rocblas_datatype_f32_r,
+                static_cast<rocblas_int>(N), M * N, S, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+            if (st != rocblas_status_success)
+                throw std::runtime_error(std::string("rocblas_gemm_strided_batched_ex failed: ") + rocblas_status_to_string(st));
+            hipLaunchKernelGGL(add_parts, ew_grid(M * N), dim3(NT), 0, tape_stream(), static_cast<const float*>(part.p),
+                               static_cast<float*>(C), S, M * N);
+            post();
+            return;
+        }
+    }
     const rocblas_status st = rocblas_gemm_ex(
         blas(), tB ? rocblas_operation_transpose : rocblas_operation_none,
         tA ? rocblas_operation_transpose : rocblas_operation_none, static_cast<rocblas_int>(N),

@@ -39,6 +39,9 @@ public:
 
     bool is_leaf() const { return parents.empty(); }
     void accumulate(const Tensor& g, float a = 1.0f);  // grad += a * g (autograd.cpp:16-24)
+    // The same for a temporary the caller is done with: the first contribution takes the buffer over instead of
+    // copying it (the reference's lazily sized grad, autograd.cpp:17-19, makes that first += a copy as well).
+    void accumulate_owned(Tensor&& g);
     Tensor& ensure_grad();                             // zero-filled grad of data's shape
 };
 

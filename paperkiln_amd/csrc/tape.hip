@@ -2,6 +2,7 @@
 // kernels of elementwise.hip and the attention entry points of the C ABI.
 #include "tape.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <unordered_map>
@@ -111,6 +112,17 @@ void Variable::accumulate(const Tensor& g, float a) {
     k_axpy(grad, a, g);
 }
 
+void Variable::accumulate_owned(Tensor&& g) {
+    const int want = is_param ? PK_F32 : data.dtype;
+    const bool whole = g.buf && g.off_bytes == 0 && g.buf.use_count() == 1 &&
+                       g.buf->bytes == static_cast<size_t>(g.rows) * g.cols * g.esize();
+    if (grad.empty() && whole && g.dtype == want && g.rows == data.rows && g.cols == data.cols) {
+        grad = std::move(g);
+        return;
+    }
+    accumulate(g);
+}
+
 bool grad_enabled() { return g_grad_enabled; }
 NoGrad::NoGrad() : prev_(g_grad_enabled) { g_grad_enabled = false; }
 NoGrad::~NoGrad() { g_grad_enabled = prev_; }
@@ -182,7 +194,7 @@ Var linear(const Var& x, const Var& W) {
         if (x->requires_grad) {  // dX = dY W^T  (ops.cpp:48-51)
             Tensor dx = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
             gemm(self->grad, false, shadow_of(W), true, dx.ptr(), dx.dtype, dx.rows, dx.cols, dx.cols, 0.0f);
-            x->accumulate(dx);
+            x->accumulate_owned(std::move(dx));
         }
         if (W->requires_grad) {  // dW += X^T dY (ops.cpp:52-55), straight into the fp32 grad
             Tensor& g = W->ensure_grad();
@@ -225,7 +237,7 @@ Var linear3(const Var& x, const Var& Wq, const Var& Wk, const Var& Wv) {
                 gemm(x->data, true, slice, false, g.ptr(), g.dtype, g.rows, g.cols, g.cols, 1.0f);
             }
         }
-        if (x->requires_grad) x->accumulate(dx);
+        if (x->requires_grad) x->accumulate_owned(std::move(dx));
     });
 }
 
@@ -247,12 +259,12 @@ Var mul(const Var& a, const Var& b) {
         if (a->requires_grad) {
             Tensor t = Tensor::make(a->data.rows, a->data.cols, a->data.dtype);
             k_mul(self->grad, b->data, t);
-            a->accumulate(t);
+            a->accumulate_owned(std::move(t));
         }
         if (b->requires_grad) {
             Tensor t = Tensor::make(a->data.rows, a->data.cols, a->data.dtype);
             k_mul(self->grad, a->data, t);
-            b->accumulate(t);
+            b->accumulate_owned(std::move(t));
         }
     });
 }
@@ -273,7 +285,7 @@ Var silu(const Var& x) {
         if (!x->requires_grad) return;
         Tensor dx = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
         k_silu_bwd(x->data, self->grad, dx);
-        x->accumulate(dx);
+        x->accumulate_owned(std::move(dx));
     });
 }
 
@@ -290,7 +302,7 @@ Var rmsnorm(const Var& x, const Var& w) {
         Tensor* dw = w->requires_grad ? &w->ensure_grad() : nullptr;
         k_rmsnorm_bwd(self->grad, x->data, static_cast<const float*>(rinv->p), w->data, dw,
                       x->requires_grad ? &dx : nullptr);
-        if (x->requires_grad) x->accumulate(dx);
+        if (x->requires_grad) x->accumulate_owned(std::move(dx));
     });
 }
 
@@ -304,7 +316,7 @@ Var apply_rope(const Var& qkv, const std::shared_ptr<Buffer>& pos, float theta, 
         if (!x->requires_grad) return;
         Tensor dx = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
         k_rope(self->grad, static_cast<const int*>(pos->p), theta, d, head_dim, rot_heads, true, dx);
-        x->accumulate(dx);
+        x->accumulate_owned(std::move(dx));
     });
 }
 
@@ -375,7 +387,7 @@ Var attention_qkv(const Var& qkv, int n_heads, float scale, int64_t seq_len, boo
                          dv4 = view4(dqkv.ptr(), 2 * d, es, sl * d3, d3, g.dk);
         attn_check(pk_attn_bwd(&sh, &q4, &k4, &v4, &o4, static_cast<const float*>(lse->p), &g4, &dq4, &dk4, &dv4, ws.p,
                                ws.bytes, tape_stream()));
-        qkv->accumulate(dqkv);
+        qkv->accumulate_owned(std::move(dqkv));
     });
 }
 
@@ -413,9 +425,9 @@ Var head_attention(const Var& q, const Var& k, const Var& v, float scale, int64_
                          g4 = v4of(self->grad), dq4 = v4of(dq), dk4 = v4of(dkk), dv4 = v4of(dv);
         attn_check(pk_attn_bwd(&sh, &q4, &k4, &vv4, &o4, static_cast<const float*>(lse->p), &g4, &dq4, &dk4, &dv4, ws.p,
                                ws.bytes, tape_stream()));
-        if (q->requires_grad) q->accumulate(dq);
-        if (k->requires_grad) k->accumulate(dkk);
-        if (v->requires_grad) v->accumulate(dv);
+        if (q->requires_grad) q->accumulate_owned(std::move(dq));
+        if (k->requires_grad) k->accumulate_owned(std::move(dkk));
+        if (v->requires_grad) v->accumulate_owned(std::move(dv));
     });
 }
 }  // namespace
@@ -443,7 +455,7 @@ Var matmul_nt(const Var& h, const Var& E) {
         if (h->requires_grad) {
             Tensor dh = Tensor::make(h->data.rows, h->data.cols, h->data.dtype);
             gemm(dl, false, shadow_of(E), false, dh.ptr(), dh.dtype, dh.rows, dh.cols, dh.cols, 0.0f);
-            h->accumulate(dh);
+            h->accumulate_owned(std::move(dh));
         }
         if (E->requires_grad) {
             Tensor& g = E->ensure_grad();
@@ -484,13 +496,14 @@ Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffe
             const Tensor hview = h->data.row_range(r0, rows);
             Tensor logits = Tensor::make(rows, V, PK_F32);
             gemm(hview, false, Ec, true, logits.ptr(), PK_F32, rows, V, V, 0.0f);
-            k_ce_rows(logits, tg + r0, gscale, static_cast<float*>(nll.p) + r0);
+            float* nll_r = static_cast<float*>(nll.p) + r0;
+            Tensor dl;
+            if (dh || dE) dl = h->data.dtype == PK_F32 ? logits : Tensor::make(rows, V, h->data.dtype);
+            if (!k_ce_rows_once(logits, tg + r0, gscale, nll_r, (dh || dE) ? &dl : nullptr)) {
+                k_ce_rows(logits, tg + r0, gscale, nll_r);
+                if ((dh || dE) && h->data.dtype != PK_F32) k_cast(logits, dl);
+            }
             if (dh || dE) {
-                Tensor dl = logits;
-                if (h->data.dtype != PK_F32) {
-                    dl = Tensor::make(rows, V, h->data.dtype);
-                    k_cast(logits, dl);
-                }
                 if (dh)
                     gemm(dl, false, Ec, false, static_cast<char*>(dh->ptr()) + r0 * h->data.cols * hes, dh->dtype, rows,
                          h->data.cols, h->data.cols, 0.0f);
@@ -511,14 +524,17 @@ Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffe
         if (h->requires_grad) dh = Tensor::make(h->data.rows, h->data.cols, h->data.dtype);
         Tensor* dE = E->requires_grad ? &E->ensure_grad() : nullptr;
         pass(h, E, g, h->requires_grad ? &dh : nullptr, dE);
-        if (h->requires_grad) h->accumulate(dh);
+        if (h->requires_grad) h->accumulate_owned(std::move(dh));
     });
 }
 
 double clip_grad_norm(const std::vector<Var>& params, float max_norm) {
-    double sq = 0.0;
+    // double accumulation as the reference (ops.cpp:1047-1053); one host round trip for all parameters
+    Buffer parts(sizeof(double) * SUMSQ_MAX_PARTS * std::max<size_t>(params.size(), 1));
+    int64_t n = 0;
     for (const auto& p : params)
-        if (!p->grad.empty()) sq += k_sumsq_to_host(p->grad);
+        if (!p->grad.empty()) n += k_sumsq_parts(p->grad, static_cast<double*>(parts.p) + n);
+    const double sq = n ? k_sum_f64_to_host(static_cast<const double*>(parts.p), n) : 0.0;
     const double total = std::sqrt(sq);
     if (total > max_norm && total > 0.0) {
         const float s = static_cast<float>(max_norm / total);

@@ -107,8 +107,16 @@ void k_embedding_bwd(const Tensor& dy, const int* ids, const Tensor& dtable_f32)
 // dlogits = (P - onehot) * gscale in place and the per-row nll (fp32) with the
 // reference's max(p, 1e-12) clamp.
 void k_ce_rows(const Tensor& logits, const int* targets, float gscale, float* nll_rows);
+// The same on fp32 logits that are read once and left untouched: dl == nullptr computes only the nll, otherwise
+// dlogits go to *dl (fp32 or bf16). Returns false when the shape does not fit (the caller then uses k_ce_rows).
+bool k_ce_rows_once(const Tensor& logits, const int* targets, float gscale, float* nll_rows, const Tensor* dl);
 double k_sum_f32_to_host(const float* x, int64_t n);                   // double accumulation, ops.cpp:360-367
 double k_sumsq_to_host(const Tensor& g);                               // clip_grad_norm's sum, ops.cpp:1046-1052
+// The same in two halves, so that many gradients cost one host round trip: per-block partial sums (at most
+// SUMSQ_MAX_PARTS doubles) into device memory, then one copy and a host sum over all of them.
+constexpr int SUMSQ_MAX_PARTS = 1024;
+int k_sumsq_parts(const Tensor& g, double* part_dev);
+double k_sum_f64_to_host(const double* part_dev, int64_t n);
 void k_adamw(const Tensor& p, const Tensor& g, const Tensor& m, const Tensor& v, float lr, float b1, float b2,
              float eps, float wd, float c1, float c2);                 // nn.cpp:301-321
 

@@ -169,6 +169,26 @@ def test_matmul_vs_numpy(bo):
         bo.matmul(dev(a), dev(a))
 
 
+def test_weight_gradient_gemm_long_contraction(bo):
+    """dW += X^T dY over 4096 tokens takes the sliced path (partial products added in slice order): same
+    result as one product, and the same bits on every run."""
+    import ctypes as C
+    from paperkiln_amd import _lib
+    x, dy = synth.bf16_round(synth.randn(441, (4096, 96), 1.0)), synth.bf16_round(synth.randn(442, (4096, 160), 1.0))
+    g0 = synth.randn(443, (96, 160), 1.0)
+    want = g0.astype(np.float64) + x.astype(np.float64).T @ dy.astype(np.float64)
+    outs = []
+    for _ in range(2):
+        g = dev(g0)
+        tx, tdy = dev(x, torch.bfloat16), dev(dy, torch.bfloat16)
+        _lib.check(_lib.lib().pk_op_gemm(C.c_void_p(tx.data_ptr()), 1, C.c_void_p(tdy.data_ptr()), 0,
+                                         C.c_void_p(g.data_ptr()), 96, 160, 4096, _lib.PK_BF16, _lib.PK_F32, 1,
+                                         C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        outs.append(host(g))
+    assert np.abs(outs[0] - want).max() < 2e-4 * np.abs(want).max()  # fp32 accumulation over 4096 terms
+    assert np.array_equal(outs[0], outs[1])
+
+
 def test_error_behaviour(bo):
     x = dev(synth.randn(431, (4, 8), 1.0))
     with pytest.raises(RuntimeError):
