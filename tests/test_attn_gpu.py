@@ -193,3 +193,53 @@ def test_full_size_properties_cfg4(oracle):
     got = (host(o[b, :, h]), host(lse[b, h]), host(dq[b, :, h]), host(dk_[b, :, h]), host(dv[b, :, h]))
     errs = report("cfg4 full size, unit (1,7)", got, want)
     assert max(errs[0], errs[2], errs[3], errs[4]) < BF16_TOL and errs[1] < BF16_LSE_TOL
+
+
+def test_full_size_window_unit_cfg4b(oracle):
+    """B=4, H=16, T=4096, d=128, window=256 + 4 sinks: one (batch, head) unit against the oracle at the full T."""
+    B, T, H, dk = 4, 4096, 16, 128
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
+    g = torch.Generator(device="cuda").manual_seed(5)
+    q, k, v = ((torch.randn((B, T, H, dk), generator=g, device="cuda") * 0.5).bfloat16() for _ in range(3))
+    d_o = torch.randn((B, T, H, dk), generator=g, device="cuda").bfloat16()
+    o, lse = ops.attn_fwd(q, k, v, scale, True, 256, 4)
+    dq, dk_, dv = ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, 256, 4, grad_dtype=torch.float32)
+    b, h = 3, 0
+    hq, hk, hv, hg = (host(x[b, :, h]) for x in (q, k, v, d_o))
+    want_y, want_lse, A = oracle.head_fwd(hq, hk, hv, scale, 0, True, 256, 4)
+    want = (want_y, want_lse) + oracle.head_bwd(hq, hk, hv, A, hg, scale, 0, True, 256, 4)
+    got = (host(o[b, :, h]), host(lse[b, h]), host(dq[b, :, h]), host(dk_[b, :, h]), host(dv[b, :, h]))
+    errs = report("cfg4b full size, unit (3,0)", got, want)
+    assert max(errs[0], errs[2], errs[3], errs[4]) < BF16_TOL and errs[1] < BF16_LSE_TOL
+
+
+@pytest.mark.parametrize("name,B,T,Hq,Hkv,theta", [("cfg2", 16, 512, 8, 8, 1e4), ("cfg3", 4, 2048, 14, 2, 1e6)])
+def test_full_size_cfg2_cfg3(oracle, name, B, T, Hq, Hkv, theta):
+    """BASELINE configs 2 and 3 at their full shapes (head_dim 64, N(0,1) with RoPE pre-applied): one
+    (batch, KV group) unit against the oracle, and GQA == MHA over repeated KV heads with the group's dK / dV summed."""
+    dk = 64
+    q, k, v, d_o = make(B, T, Hq, Hkv, dk, 1.0, 700, theta)
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
+    tq, tk, tv, tg = (torch.from_numpy(x).cuda().bfloat16() for x in (q, k, v, d_o))
+    o, lse = ops.attn_fwd(tq, tk, tv, scale, True)
+    dq, dk_, dv = ops.attn_bwd(tq, tk, tv, o, lse, tg, scale, True, grad_dtype=torch.float32)
+    rep = Hq // Hkv
+    b, hk = B - 1, Hkv - 1
+    hs = slice(hk * rep, (hk + 1) * rep)
+    uq, uk, uv, ug = q[b:b + 1, :, hs], k[b:b + 1, :, hk:hk + 1], v[b:b + 1, :, hk:hk + 1], d_o[b:b + 1, :, hs]
+    want_o, want_lse = oracle.attn_fwd(uq, uk, uv, scale, True, 0, 0)
+    want = (want_o, want_lse) + oracle.attn_bwd(uq, uk, uv, ug, scale, True, 0, 0)
+    got = (host(o[b:b + 1, :, hs]), host(lse[b:b + 1, hs]), host(dq[b:b + 1, :, hs]), host(dk_[b:b + 1, :, hk:hk + 1]),
+           host(dv[b:b + 1, :, hk:hk + 1]))
+    errs = report(f"{name} full size, unit (b={b}, kv head {hk})", got, want)
+    assert max(errs[0], errs[2], errs[3], errs[4]) < BF16_TOL and errs[1] < BF16_LSE_TOL
+    if rep > 1:
+        kr, vr = tk.repeat_interleave(rep, dim=2), tv.repeat_interleave(rep, dim=2)
+        o2, lse2 = ops.attn_fwd(tq, kr, vr, scale, True)
+        assert torch.equal(o2, o) and torch.equal(lse2, lse)
+        dq2, dk2, dv2 = ops.attn_bwd(tq, kr, vr, o2, lse2, tg, scale, True, grad_dtype=torch.float32)
+        assert torch.equal(dq2, dq)
+        sk = dk2.view(B, T, Hkv, rep, dk).sum(dim=3)
+        sv = dv2.view(B, T, Hkv, rep, dk).sum(dim=3)
+        assert float((sk - dk_).abs().max()) < 1e-3 * float(dk_.abs().max()) + 1e-4  # fp32 sums in another order
+        assert float((sv - dv).abs().max()) < 1e-3 * float(dv.abs().max()) + 1e-4
