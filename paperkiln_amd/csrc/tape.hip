@@ -482,49 +482,60 @@ Var cross_entropy(const Var& logits, const std::shared_ptr<Buffer>& targets) {
 }
 
 Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffer>& targets, int64_t chunk_rows) {
-    const int64_t N = h->data.rows, V = E->data.rows;
-    if (h->data.cols != E->data.cols) throw std::runtime_error("matmul: inner dimensions disagree");
+    const int64_t N = h->data.rows, V = E->data.rows, d = h->data.cols;
+    if (d != E->data.cols) throw std::runtime_error("matmul: inner dimensions disagree");
     if (chunk_rows <= 0) chunk_rows = 1024;
     const int* tg = static_cast<const int*>(targets->p);
     const size_t hes = h->data.esize();
-    // one pass over row chunks; with_grad also produces dh and accumulates dE
-    auto pass = [N, V, chunk_rows, tg, hes](const Var& h, const Var& E, float gscale, Tensor* dh, Tensor* dE) {
-        const Tensor& Ec = shadow_of(E);
-        Buffer nll(sizeof(float) * N);
-        for (int64_t r0 = 0; r0 < N; r0 += chunk_rows) {
-            const int64_t rows = std::min(chunk_rows, N - r0);
-            const Tensor hview = h->data.row_range(r0, rows);
-            Tensor logits = Tensor::make(rows, V, PK_F32);
-            gemm(hview, false, Ec, true, logits.ptr(), PK_F32, rows, V, V, 0.0f);
-            float* nll_r = static_cast<float*>(nll.p) + r0;
-            Tensor dl;
-            if (dh || dE) dl = h->data.dtype == PK_F32 ? logits : Tensor::make(rows, V, h->data.dtype);
-            if (!k_ce_rows_once(logits, tg + r0, gscale, nll_r, (dh || dE) ? &dl : nullptr)) {
-                k_ce_rows(logits, tg + r0, gscale, nll_r);
-                if ((dh || dE) && h->data.dtype != PK_F32) k_cast(logits, dl);
-            }
-            if (dh || dE) {
-                if (dh)
-                    gemm(dl, false, Ec, false, static_cast<char*>(dh->ptr()) + r0 * h->data.cols * hes, dh->dtype, rows,
-                         h->data.cols, h->data.cols, 0.0f);
-                if (dE) gemm(dl, true, hview, false, dE->ptr(), dE->dtype, V, h->data.cols, h->data.cols, 1.0f);
-            }
+    // One pass over row chunks. The loss is a scalar, so its gradient with respect to the logits is known up to
+    // the upstream factor as soon as a chunk's softmax is: when a gradient will be asked for, the same pass also
+    // produces dh and dE for an upstream gradient of 1 (dlogits = (P - onehot) / N), and the backward closure only
+    // scales them. Nothing of size [N, vocab] outlives its chunk, and no chunk's logits are computed twice.
+    const bool want_dh = grad_enabled() && h->requires_grad, want_dE = grad_enabled() && E->requires_grad;
+    Tensor dh1, dE1;
+    if (want_dh) dh1 = Tensor::make(N, d, h->data.dtype);
+    if (want_dE) dE1 = Tensor::make(V, d, PK_F32);
+    const Tensor& Ec = shadow_of(E);
+    Buffer nll(sizeof(float) * N);
+    const float g1 = 1.0f / static_cast<float>(N);
+    for (int64_t r0 = 0; r0 < N; r0 += chunk_rows) {
+        const int64_t rows = std::min(chunk_rows, N - r0);
+        const Tensor hview = h->data.row_range(r0, rows);
+        Tensor logits = Tensor::make(rows, V, PK_F32);
+        gemm(hview, false, Ec, true, logits.ptr(), PK_F32, rows, V, V, 0.0f);
+        float* nll_r = static_cast<float*>(nll.p) + r0;
+        const bool grads = want_dh || want_dE;
+        Tensor dl;
+        if (grads) dl = h->data.dtype == PK_F32 ? logits : Tensor::make(rows, V, h->data.dtype);
+        if (!k_ce_rows_once(logits, tg + r0, g1, nll_r, grads ? &dl : nullptr)) {
+            k_ce_rows(logits, tg + r0, g1, nll_r);
+            if (grads && h->data.dtype != PK_F32) k_cast(logits, dl);
         }
-        return k_sum_f32_to_host(static_cast<const float*>(nll.p), N);
-    };
-    const double total = pass(h, E, 0.0f, nullptr, nullptr);
+        if (want_dh)
+            gemm(dl, false, Ec, false, static_cast<char*>(dh1.ptr()) + r0 * d * hes, dh1.dtype, rows, d, d, 0.0f);
+        if (want_dE) gemm(dl, true, hview, false, dE1.ptr(), PK_F32, V, d, d, r0 == 0 ? 0.0f : 1.0f);
+    }
+    const double total = k_sum_f32_to_host(static_cast<const float*>(nll.p), N);
     Tensor out = Tensor::make(1, 1, PK_F32);
     k_fill(out, static_cast<float>(total / static_cast<double>(N)));
-    // Backward recomputes each chunk of logits: nothing of size [N, vocab] is kept.
-    return record(std::move(out), {h, E}, [pass, N](Variable* self) {
+    return record(std::move(out), {h, E}, [dh1, dE1](Variable* self) mutable {
         const Var& h = self->parents[0];
         const Var& E = self->parents[1];
-        const float g = scalar_to_host(self->grad) / static_cast<float>(N);
-        Tensor dh;
-        if (h->requires_grad) dh = Tensor::make(h->data.rows, h->data.cols, h->data.dtype);
-        Tensor* dE = E->requires_grad ? &E->ensure_grad() : nullptr;
-        pass(h, E, g, h->requires_grad ? &dh : nullptr, dE);
-        if (h->requires_grad) h->accumulate_owned(std::move(dh));
+        const float g = scalar_to_host(self->grad);  // upstream gradient of the scalar loss
+        if (h->requires_grad && !dh1.empty()) {
+            if (g == 1.0f)
+                h->accumulate_owned(std::move(dh1));
+            else
+                h->accumulate(dh1, g);
+        }
+        if (E->requires_grad && !dE1.empty()) {
+            if (g == 1.0f)
+                E->accumulate_owned(std::move(dE1));
+            else
+                E->accumulate(dE1, g);
+        }
+        dh1 = Tensor();
+        dE1 = Tensor();
     });
 }
 
