@@ -221,12 +221,13 @@ __global__ void colsum_parts(const float* part, float* dw, int nparts, int C) {
     __syncthreads();
     if (grp == 0 && col < C) dw[col] += (sh[0][threadIdx.x] + sh[1][threadIdx.x]) + (sh[2][threadIdx.x] + sh[3][threadIdx.x]);
 }
-// dst[i] += sum_s part[s][i], parts added in index order
-__global__ void add_parts(const float* part, float* dst, int nparts, int64_t n) {
+// dst[i] = beta * dst[i] + sum_s part[s][i], parts added in index order
+template <typename T>
+__global__ void add_parts(const float* part, T* dst, int nparts, int64_t n, float beta) {
     for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT) {
         float s = 0.0f;
         for (int p = 0; p < nparts; ++p) s += part[p * n + i];
-        dst[i] += s;
+        stf(dst, i, beta != 0.0f ? ldf(dst, i) + s : s);
     }
 }
 
@@ -612,27 +613,32 @@ void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dty
     const rocblas_datatype ct = c_dtype == PK_F32 ? rocblas_datatype_f32_r : rocblas_datatype_bf16_r;
     const float alpha = 1.0f;
     rocblas_set_stream(blas(), tape_stream());
-    // Weight gradients (X^T dY accumulated into an fp32 matrix): the contraction runs over every token while
-    // the output is a few hundred tiles at most, so one GEMM leaves most of the chip idle. The token axis is
-    // cut into slices that run as one strided-batched GEMM into separate partial products, which are then
-    // added in slice order: no atomics, so the sum is the same on every run.
-    if (tA && !tB && c_dtype == PK_F32 && beta == 1.0f && ldc == N && Ka >= 2048 && M * N <= (int64_t{1} << 21)) {
+    // Long contractions with a small output (weight gradients X^T dY over every token; dh = dlogits E over the
+    // vocabulary): one GEMM would be a few hundred tiles at most and leave most of the chip idle. The contraction
+    // axis is cut into slices that run as one strided-batched GEMM into separate fp32 partial products, which are
+    // then added in slice order: no atomics, so the sum is the same on every run.
+    if (!tB && ldc == N && Ka >= 2048 && M * N <= (int64_t{1} << 21) && (beta == 0.0f || beta == 1.0f)) {
         int S = 8;
         while (S > 1 && (Ka % S != 0 || Ka / S < 256)) S >>= 1;
         if (S > 1) {
             const int64_t Ks = Ka / S;
             Buffer part(sizeof(float) * static_cast<size_t>(S) * M * N);
             const float zero = 0.0f;
+            const int64_t stride_a = tA ? Ks * A.cols : Ks, stride_b = Ks * B.cols;
             const rocblas_status st = rocblas_gemm_strided_batched_ex(
-                blas(), rocblas_operation_none, rocblas_operation_transpose, static_cast<rocblas_int>(N),
-                static_cast<rocblas_int>(M), static_cast<rocblas_int>(Ks), &alpha, B.ptr(), ab,
-                static_cast<rocblas_int>(B.cols), Ks * B.cols, A.ptr(), ab, static_cast<rocblas_int>(A.cols), Ks * A.cols, &zero,
+                blas(), rocblas_operation_none, tA ? rocblas_operation_transpose : rocblas_operation_none,
+                static_cast<rocblas_int>(N), static_cast<rocblas_int>(M), static_cast<rocblas_int>(Ks), &alpha, B.ptr(), ab,
+                static_cast<rocblas_int>(B.cols), stride_b, A.ptr(), ab, static_cast<rocblas_int>(A.cols), stride_a, &zero,
                 part.p, rocblas_datatype_f32_r, static_cast<rocblas_int>(N), M * N, part.p, rocblas_datatype_f32_r,
                 static_cast<rocblas_int>(N), M * N, S, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
             if (st != rocblas_status_success)
                 throw std::runtime_error(std::string("rocblas_gemm_strided_batched_ex failed: ") + rocblas_status_to_string(st));
-            hipLaunchKernelGGL(add_parts, ew_grid(M * N), dim3(NT), 0, tape_stream(), static_cast<const float*>(part.p),
-                               static_cast<float*>(C), S, M * N);
+            if (c_dtype == PK_F32)
+                hipLaunchKernelGGL((add_parts<float>), ew_grid(M * N), dim3(NT), 0, tape_stream(),
+                                   static_cast<const float*>(part.p), static_cast<float*>(C), S, M * N, beta);
+            else
+                hipLaunchKernelGGL((add_parts<uint16_t>), ew_grid(M * N), dim3(NT), 0, tape_stream(),
+                                   static_cast<const float*>(part.p), static_cast<uint16_t*>(C), S, M * N, beta);
             post();
             return;
         }

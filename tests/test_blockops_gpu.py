@@ -187,6 +187,12 @@ def test_weight_gradient_gemm_long_contraction(bo):
         outs.append(host(g))
     assert np.abs(outs[0] - want).max() < 2e-4 * np.abs(want).max()  # fp32 accumulation over 4096 terms
     assert np.array_equal(outs[0], outs[1])
+    # the same slicing for a plain product with a long inner dimension and a bf16 result (dh = dlogits E)
+    a, b = synth.bf16_round(synth.randn(444, (130, 4096), 0.1)), synth.bf16_round(synth.randn(445, (4096, 72), 1.0))
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    got = bo.matmul(dev(a, torch.bfloat16), dev(b, torch.bfloat16))
+    close(got, synth.bf16_round(want.astype(np.float32)), 1e-2)
+    close(bo.matmul(dev(a, torch.bfloat16), dev(b, torch.bfloat16), out_dtype=torch.float32), want, 2e-4)
 
 
 def test_error_behaviour(bo):
