@@ -168,6 +168,11 @@ int pk_op_fill(void* y, float v, int64_t n, int dtype, void* stream);           
 /* ops::silu and its closure (src/ops.cpp:404-424). */
 int pk_op_silu_fwd(const void* x, void* y, int64_t n, int dtype, void* stream);
 int pk_op_silu_bwd(const void* x, const void* dy, void* dx, int64_t n, int dtype, void* stream);
+/* mul(silu(gate), up), LlamaBlock's SwiGLU (src/llama.cpp:55-58), as one pass each way instead of the two tape nodes
+ * ops::silu and ops::mul (src/ops.cpp:404-424, 76-83). */
+int pk_op_silu_mul_fwd(const void* gate, const void* up, void* y, int64_t n, int dtype, void* stream);
+int pk_op_silu_mul_bwd(const void* gate, const void* up, const void* dy, void* dgate, void* dup, int64_t n, int dtype,
+                       void* stream);
 /* ops::rmsnorm (src/ops.cpp:426-479; devops::rmsnorm_fwd / rmsnorm_bwd). w, rms_inv[rows] and dw are fp32;
  * dw and dx may be NULL (the reference's want_dw / want_dx) and are overwritten, not accumulated. */
 int pk_op_rmsnorm_fwd(const void* x, const float* w, float eps, void* y, float* rms_inv, int64_t rows, int64_t cols,

@@ -50,7 +50,7 @@ EXPORTS = ["pk_last_error", "pk_init", "pk_attn_fwd", "pk_attn_bwd_workspace_byt
            "pk_alloc", "pk_free", "pk_live_bytes", "pk_peak_bytes", "pk_reset_peak", "pk_trim",
            "pk_llama_create", "pk_llama_destroy", "pk_llama_num_params", "pk_llama_param_info", "pk_llama_set_param",
            "pk_llama_get_param", "pk_llama_get_grad", "pk_llama_loss_backward", "pk_llama_adamw_step",
-           "pk_op_add", "pk_op_mul", "pk_op_scale", "pk_op_axpy", "pk_op_fill", "pk_op_silu_fwd", "pk_op_silu_bwd",
+           "pk_op_add", "pk_op_mul", "pk_op_scale", "pk_op_axpy", "pk_op_fill", "pk_op_silu_fwd", "pk_op_silu_bwd", "pk_op_silu_mul_fwd", "pk_op_silu_mul_bwd",
            "pk_op_rmsnorm_fwd", "pk_op_rmsnorm_bwd", "pk_op_rope", "pk_op_embedding_fwd", "pk_op_embedding_bwd",
            "pk_op_cross_entropy", "pk_op_adamw", "pk_op_sumsq", "pk_op_gemm"]
 
@@ -98,6 +98,8 @@ def lib() -> C.CDLL:
         L.pk_op_fill.argtypes = [vp, cf, i64, ci, vp]
         L.pk_op_silu_fwd.argtypes = [vp, vp, i64, ci, vp]
         L.pk_op_silu_bwd.argtypes = [vp, vp, vp, i64, ci, vp]
+        L.pk_op_silu_mul_fwd.argtypes = [vp, vp, vp, i64, ci, vp]
+        L.pk_op_silu_mul_bwd.argtypes = [vp, vp, vp, vp, vp, i64, ci, vp]
         L.pk_op_rmsnorm_fwd.argtypes = [vp, vp, cf, vp, vp, i64, i64, ci, vp]
         L.pk_op_rmsnorm_bwd.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, ci, vp]
         L.pk_op_rope.argtypes = [vp, vp, cf, i64, i64, ci, ci, ci, vp, ci, vp]

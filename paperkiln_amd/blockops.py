@@ -84,6 +84,20 @@ def silu(x, dy=None):
     return y, dx
 
 
+def silu_mul(gate, up, dy=None):
+    """mul(silu(gate), up) in one pass; with dy also (dgate, dup)."""
+    _chk(gate, up)
+    y = torch.empty_like(gate)
+    L = _lib.lib()
+    check(L.pk_op_silu_mul_fwd(_p(gate), _p(up), _p(y), gate.numel(), _dt(gate), _s()))
+    if dy is None:
+        return y
+    _chk(gate, dy)
+    dg, du = torch.empty_like(gate), torch.empty_like(gate)
+    check(L.pk_op_silu_mul_bwd(_p(gate), _p(up), _p(dy), _p(dg), _p(du), gate.numel(), _dt(gate), _s()))
+    return y, dg, du
+
+
 def rmsnorm(x, w, dy=None, eps=1e-5):
     """ops::rmsnorm: y (and, with dy, dx and dw). w is fp32 [cols]."""
     _chk(x)

@@ -161,6 +161,25 @@ __global__ void ew_silu_bwd(const T* x, const T* dy, T* dx, int64_t n) {
     }
 }
 
+// silu(gate) .* up in one pass (the two tape nodes ops::silu, src/ops.cpp:404-424, and ops::mul, :76-83, of
+// LlamaBlock's SwiGLU, src/llama.cpp:55-58) and the pair of closures in one pass back.
+template <typename T>
+__global__ void ew_silu_mul_fwd(const T* gate, const T* up, T* y, int64_t n) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT) {
+        const float v = ldf(gate, i);
+        stf(y, i, (v / (1.0f + expf(-v))) * ldf(up, i));
+    }
+}
+template <typename T>
+__global__ void ew_silu_mul_bwd(const T* gate, const T* up, const T* dy, T* dgate, T* dup, int64_t n) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT) {
+        const float v = ldf(gate, i), g = ldf(dy, i);
+        const float s = 1.0f / (1.0f + expf(-v));
+        stf(dup, i, g * (v * s));
+        stf(dgate, i, (g * ldf(up, i)) * (s * (1.0f + v * (1.0f - s))));
+    }
+}
+
 __device__ inline float wave_sum(float x) {
 #pragma unroll
     for (int o = 32; o >= 1; o >>= 1) x += __shfl_xor(x, o, 64);
@@ -470,6 +489,26 @@ void k_silu_bwd(const Tensor& x, const Tensor& dy, const Tensor& dx) {
     PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((ew_silu_bwd<T>), ew_grid(x.numel()), dim3(NT), 0, tape_stream(),
                                                 static_cast<const T*>(x.ptr()), static_cast<const T*>(dy.ptr()),
                                                 static_cast<T*>(dx.ptr()), x.numel()));
+    post();
+}
+void k_silu_mul_fwd(const Tensor& gate, const Tensor& up, const Tensor& y) {
+    same_shape(gate, up, "mul");
+    same_shape(gate, y, "mul");
+    PK_DISPATCH1(T, gate.dtype, hipLaunchKernelGGL((ew_silu_mul_fwd<T>), ew_grid(gate.numel()), dim3(NT), 0, tape_stream(),
+                                                   static_cast<const T*>(gate.ptr()), static_cast<const T*>(up.ptr()),
+                                                   static_cast<T*>(y.ptr()), gate.numel()));
+    post();
+}
+void k_silu_mul_bwd(const Tensor& gate, const Tensor& up, const Tensor& dy, const Tensor& dgate, const Tensor& dup) {
+    same_shape(gate, up, "mul");
+    same_shape(gate, dy, "mul");
+    same_shape(gate, dgate, "mul");
+    same_shape(gate, dup, "mul");
+    PK_DISPATCH1(T, gate.dtype,
+                 hipLaunchKernelGGL((ew_silu_mul_bwd<T>), ew_grid(gate.numel()), dim3(NT), 0, tape_stream(),
+                                    static_cast<const T*>(gate.ptr()), static_cast<const T*>(up.ptr()),
+                                    static_cast<const T*>(dy.ptr()), static_cast<T*>(dgate.ptr()), static_cast<T*>(dup.ptr()),
+                                    gate.numel()));
     post();
 }
 void k_rmsnorm_fwd(const Tensor& x, const Tensor& w, float eps, const Tensor& y, float* rinv) {

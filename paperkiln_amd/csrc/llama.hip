@@ -130,7 +130,7 @@ struct Model {
         Var attn = ops::linear(ops::attention_qkv(qkv, cfg.n_heads, sc, seq_len, true, cfg.window, cfg.sinks), b.o);
         Var x1 = ops::add(x, attn);
         Var h2 = ops::rmsnorm(x1, b.ln2_w);
-        Var ffn = ops::linear(ops::mul(ops::silu(ops::linear(h2, b.gate)), ops::linear(h2, b.up)), b.down);
+        Var ffn = ops::linear(ops::silu_mul(ops::linear(h2, b.gate), ops::linear(h2, b.up)), b.down);
         return ops::add(x1, ffn);
     }
 

@@ -65,6 +65,15 @@ int pk_op_silu_fwd(const void* x, void* y, int64_t n, int dtype, void* stream) {
 int pk_op_silu_bwd(const void* x, const void* dy, void* dx, int64_t n, int dtype, void* stream) {
     return op_guard(stream, [&] { k_silu_bwd(vec(x, n, dtype), vec(dy, n, dtype), vec(dx, n, dtype)); });
 }
+int pk_op_silu_mul_fwd(const void* gate, const void* up, void* y, int64_t n, int dtype, void* stream) {
+    return op_guard(stream, [&] { k_silu_mul_fwd(vec(gate, n, dtype), vec(up, n, dtype), vec(y, n, dtype)); });
+}
+int pk_op_silu_mul_bwd(const void* gate, const void* up, const void* dy, void* dgate, void* dup, int64_t n, int dtype,
+                       void* stream) {
+    return op_guard(stream, [&] {
+        k_silu_mul_bwd(vec(gate, n, dtype), vec(up, n, dtype), vec(dy, n, dtype), vec(dgate, n, dtype), vec(dup, n, dtype));
+    });
+}
 int pk_op_rmsnorm_fwd(const void* x, const float* w, float eps, void* y, float* rms_inv, int64_t rows, int64_t cols,
                       int dtype, void* stream) {
     return op_guard(stream, [&] {

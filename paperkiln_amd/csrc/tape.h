@@ -85,6 +85,7 @@ Var add(const Var& a, const Var& b);                // ops.cpp:60-65
 Var mul(const Var& a, const Var& b);                // ops.cpp:76-83
 Var scale(const Var& x, float s);                   // ops.cpp:843-861
 Var silu(const Var& x);                             // ops.cpp:404-424
+Var silu_mul(const Var& gate, const Var& up);        // mul(silu(gate), up) as one node (llama.cpp:55-58)
 Var rmsnorm(const Var& x, const Var& w);            // ops.cpp:426-479, eps fixed at 1e-5 (:435)
 // ops::apply_rope on the fused [N, 3d] matrix (ops.cpp:481-537). rot_heads = 1 is the
 // reference as written (only the first head of q and of k is rotated, :498-499 with the

@@ -289,6 +289,22 @@ Var silu(const Var& x) {
     });
 }
 
+Var silu_mul(const Var& gate, const Var& up) {
+    if (gate->data.rows != up->data.rows || gate->data.cols != up->data.cols) throw std::runtime_error("mul: shape mismatch");
+    Tensor y = Tensor::make(gate->data.rows, gate->data.cols, gate->data.dtype);
+    k_silu_mul_fwd(gate->data, up->data, y);
+    return record(std::move(y), {gate, up}, [](Variable* self) {
+        const Var& gate = self->parents[0];
+        const Var& up = self->parents[1];
+        if (!gate->requires_grad && !up->requires_grad) return;
+        Tensor dg = Tensor::make(gate->data.rows, gate->data.cols, gate->data.dtype);
+        Tensor du = Tensor::make(gate->data.rows, gate->data.cols, gate->data.dtype);
+        k_silu_mul_bwd(gate->data, up->data, self->grad, dg, du);
+        if (gate->requires_grad) gate->accumulate_owned(std::move(dg));
+        if (up->requires_grad) up->accumulate_owned(std::move(du));
+    });
+}
+
 Var rmsnorm(const Var& x, const Var& w) {
     if (w->data.rows != 1 || w->data.cols != x->data.cols) throw std::runtime_error("rmsnorm: w must be [1, cols(x)]");
     auto rinv = std::make_shared<Buffer>(sizeof(float) * x->data.rows);

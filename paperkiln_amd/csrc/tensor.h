@@ -94,6 +94,8 @@ void k_scale(const Tensor& a, float s, const Tensor& y);                // y = a
 void k_axpy(const Tensor& y, float a, const Tensor& x);                 // y += a * x     (autograd.cpp:16-24)
 void k_silu_fwd(const Tensor& x, const Tensor& y);                      // ops.cpp:404-411
 void k_silu_bwd(const Tensor& x, const Tensor& dy, const Tensor& dx);   // ops.cpp:412-423
+void k_silu_mul_fwd(const Tensor& gate, const Tensor& up, const Tensor& y);  // silu(gate) .* up, llama.cpp:55-58
+void k_silu_mul_bwd(const Tensor& gate, const Tensor& up, const Tensor& dy, const Tensor& dgate, const Tensor& dup);
 void k_rmsnorm_fwd(const Tensor& x, const Tensor& w, float eps, const Tensor& y, float* rinv);  // ops.cpp:437-445
 void k_rmsnorm_bwd(const Tensor& dy, const Tensor& x, const float* rinv, const Tensor& w, const Tensor* dw_f32,
                    const Tensor* dx);                                   // ops.cpp:447-478

@@ -130,6 +130,11 @@ def test_block_ops_vs_oracle_larger(bo, oracle, dtype, tol):
     wy, wdx = oracle.silu(x, dy)
     y, dx = bo.silu(dev(x, td), dev(dy, td))
     close(y, wy, tol), close(dx, wdx, tol)
+    # silu(gate) .* up as one node: the product rule over the oracle's silu
+    up = rnd(synth.randn(412, (R, Cc), 1.0))
+    sy, sdx = oracle.silu(x, np.ones_like(x))  # sdx = silu'(x)
+    y, dgate, dup = bo.silu_mul(dev(x, td), dev(up, td), dev(dy, td))
+    close(y, sy * up, tol), close(dgate, dy * up * sdx, tol), close(dup, dy * sy, tol)
     a, b = rnd(synth.randn(404, (R, Cc), 1.0)), rnd(synth.randn(405, (R, Cc), 1.0))
     close(bo.add(dev(a, td), dev(b, td)), a + b, tol)
     close(bo.mul(dev(a, td), dev(b, td)), a * b, tol)
