@@ -281,6 +281,23 @@ __global__ void rope_k(const T* x, const int* pos, RopeFreq freq, int d, int hea
     }
 }
 
+// The same rotation applied where the data lies: only the rotated columns (q and k thirds, the first
+// rot_heads heads) are touched, everything else stays as it is.
+template <typename T>
+__global__ void rope_inplace_k(T* x, const int* pos, RopeFreq freq, int d, int head_dim, int rot_heads, float sign, int64_t N) {
+    const int ppr = rot_heads * head_dim;  // rotated pairs per row: 2 thirds x rot_heads x head_dim / 2
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < N * ppr; i += static_cast<int64_t>(gridDim.x) * NT) {
+        const int64_t row = i / ppr;
+        const int p = static_cast<int>(i % ppr), third = p / (ppr / 2), within = (p % (ppr / 2)) * 2;
+        const int64_t o = row * 3 * d + third * d + within;
+        const float th = sign * static_cast<float>(pos[row]) * freq.f[(within % head_dim) >> 1];
+        const float c_ = cosf(th), s_ = sinf(th);
+        const float x0 = ldf(x, o), x1 = ldf(x, o + 1);
+        stf(x, o, x0 * c_ - x1 * s_);
+        stf(x, o + 1, x0 * s_ + x1 * c_);
+    }
+}
+
 template <typename T>
 __global__ void emb_fwd(const float* table, const int* ids, T* y, int64_t n, int d) {
     for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n * d; i += static_cast<int64_t>(gridDim.x) * NT)
@@ -540,17 +557,31 @@ void k_rmsnorm_bwd(const Tensor& dy, const Tensor& x, const float* rinv, const T
         post();
     }
 }
-void k_rope(const Tensor& x, const int* pos, float theta, int d, int head_dim, int rot_heads, bool inverse,
-            const Tensor& y) {
+namespace {
+RopeFreq rope_freq(const Tensor& x, float theta, int d, int head_dim) {
     if (x.cols != 3 * d) throw std::runtime_error("apply_rope: cols must be divisible by 3");
     if (head_dim % 2 != 0 || head_dim > d) throw std::runtime_error("apply_rope: head_dim must be even and <= d");
     if (head_dim > 2 * ROPE_MAX_PAIRS) throw std::runtime_error("apply_rope: head_dim above 256 is not supported");
     RopeFreq freq;
     for (int dim = 0; dim < head_dim; dim += 2)  // ops.cpp:499-500
         freq.f[dim >> 1] = 1.0f / std::pow(theta, static_cast<float>(dim) / static_cast<float>(head_dim));
+    return freq;
+}
+}  // namespace
+void k_rope(const Tensor& x, const int* pos, float theta, int d, int head_dim, int rot_heads, bool inverse,
+            const Tensor& y) {
+    const RopeFreq freq = rope_freq(x, theta, d, head_dim);
     PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((rope_k<T>), ew_grid(x.numel() / 2), dim3(NT), 0, tape_stream(),
                                                 static_cast<const T*>(x.ptr()), pos, freq, d, head_dim, rot_heads,
                                                 inverse ? -1.0f : 1.0f, static_cast<T*>(y.ptr()), x.rows));
+    post();
+}
+void k_rope_inplace(const Tensor& x, const int* pos, float theta, int d, int head_dim, int rot_heads, bool inverse) {
+    const RopeFreq freq = rope_freq(x, theta, d, head_dim);
+    if (rot_heads < 1 || rot_heads * head_dim > d) throw std::runtime_error("apply_rope: head_dim must be even and <= d");
+    PK_DISPATCH1(T, x.dtype,
+                 hipLaunchKernelGGL((rope_inplace_k<T>), ew_grid(x.rows * rot_heads * head_dim), dim3(NT), 0, tape_stream(),
+                                    static_cast<T*>(x.ptr()), pos, freq, d, head_dim, rot_heads, inverse ? -1.0f : 1.0f, x.rows));
     post();
 }
 void k_embedding_fwd(const Tensor& table, const int* ids, const Tensor& y) {

@@ -125,7 +125,7 @@ struct Model {
         const int dk = cfg.d / cfg.n_heads;
         Var h = ops::rmsnorm(x, b.ln1_w);
         Var qkv = ops::linear3(h, b.q, b.k, b.v);
-        qkv = ops::apply_rope(qkv, pos, cfg.rope_theta, dk, cfg.rope_all_heads ? cfg.n_heads : 1);
+        qkv = ops::apply_rope(qkv, pos, cfg.rope_theta, dk, cfg.rope_all_heads ? cfg.n_heads : 1, /*in_place=*/true);
         const float sc = 1.0f / std::sqrt(static_cast<float>(dk));
         Var attn = ops::linear(ops::attention_qkv(qkv, cfg.n_heads, sc, seq_len, true, cfg.window, cfg.sinks), b.o);
         Var x1 = ops::add(x, attn);

@@ -90,7 +90,8 @@ Var rmsnorm(const Var& x, const Var& w);            // ops.cpp:426-479, eps fixe
 // ops::apply_rope on the fused [N, 3d] matrix (ops.cpp:481-537). rot_heads = 1 is the
 // reference as written (only the first head of q and of k is rotated, :498-499 with the
 // call at llama.cpp:36); rot_heads = n_heads rotates every head.
-Var apply_rope(const Var& qkv, const std::shared_ptr<Buffer>& pos_dev, float theta, int head_dim, int rot_heads);
+Var apply_rope(const Var& qkv, const std::shared_ptr<Buffer>& pos_dev, float theta, int head_dim, int rot_heads,
+               bool in_place = false);  // in_place: qkv is a projection nobody else reads; rotate it where it lies
 Var embedding(const Var& table, const std::shared_ptr<Buffer>& ids_dev, int64_t n);  // ops.cpp:329-348
 // All heads of llama.cpp:47-53 in one node: heads are read in place from the fused
 // [N, 3d] matrix (q | k | v thirds, head h at columns h*dk) and written side by side

@@ -167,9 +167,9 @@ Var checkpoint(const std::function<Var(const Var&)>& fn, const Var& x) {
     auto fn_copy = fn;
     out->backward_fn = [self, fn_copy]() {
         const Var& xin = self->parents[0];
-        // Re-run the segment on a detached leaf that shares the input's storage: nothing
-        // writes into an activation after it is produced, so the copy the reference makes
-        // (autograd.cpp:86) is not needed on a tape whose tensors are immutable.
+        // Re-run the segment on a detached leaf that shares the input's storage: no op writes
+        // into a tensor it did not produce itself, so the copy the reference makes
+        // (autograd.cpp:86) is not needed.
         Var x2 = make_var(xin->data, /*requires_grad=*/true);
         Var y2 = fn_copy(x2);
         if (y2->data.rows != self->grad.rows || y2->data.cols != self->grad.cols)
@@ -322,9 +322,22 @@ Var rmsnorm(const Var& x, const Var& w) {
     });
 }
 
-Var apply_rope(const Var& qkv, const std::shared_ptr<Buffer>& pos, float theta, int head_dim, int rot_heads) {
+Var apply_rope(const Var& qkv, const std::shared_ptr<Buffer>& pos, float theta, int head_dim, int rot_heads, bool in_place) {
     if (qkv->data.cols % 3 != 0) throw std::runtime_error("apply_rope: cols must be divisible by 3");
     const int d = static_cast<int>(qkv->data.cols / 3);
+    if (in_place) {
+        // The caller hands over a projection nobody else reads (a Linear's backward needs its input and weight, not
+        // its output): the rotation is applied where the data lies and the node shares the storage; the backward
+        // turns this node's gradient back in place and passes it on whole.
+        k_rope_inplace(qkv->data, static_cast<const int*>(pos->p), theta, d, head_dim, rot_heads, false);
+        return record(Tensor(qkv->data), {qkv}, [pos, theta, head_dim, rot_heads, d](Variable* self) {
+            const Var& x = self->parents[0];
+            if (!x->requires_grad) return;
+            k_rope_inplace(self->grad, static_cast<const int*>(pos->p), theta, d, head_dim, rot_heads, true);
+            x->accumulate_owned(std::move(self->grad));
+            self->grad = Tensor();
+        });
+    }
     Tensor y = Tensor::make(qkv->data.rows, qkv->data.cols, qkv->data.dtype);
     k_rope(qkv->data, static_cast<const int*>(pos->p), theta, d, head_dim, rot_heads, false, y);
     return record(std::move(y), {qkv}, [pos, theta, head_dim, rot_heads, d](Variable* self) {

@@ -103,6 +103,7 @@ void k_rmsnorm_bwd(const Tensor& dy, const Tensor& x, const float* rinv, const T
 // first `rot_heads` heads of the q third and of the k third; inverse = backward.
 void k_rope(const Tensor& x, const int* pos, float theta, int d, int head_dim, int rot_heads, bool inverse,
             const Tensor& y);
+void k_rope_inplace(const Tensor& x, const int* pos, float theta, int d, int head_dim, int rot_heads, bool inverse);
 void k_embedding_fwd(const Tensor& table_f32, const int* ids, const Tensor& y);       // ops.cpp:329-337
 void k_embedding_bwd(const Tensor& dy, const int* ids, const Tensor& dtable_f32);     // scatter-add, ops.cpp:338-347
 // Row-wise softmax cross-entropy on a block of logits (ops.cpp:350-376): writes
