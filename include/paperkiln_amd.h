@@ -103,7 +103,11 @@ int pk_attn_bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_ten
  * Caching allocator with a byte-level high-water mark: the HIP counterpart of
  * the per-call cudaMalloc/cudaFree in src/cuda_resident.cu:226-263 and
  * src/cuda_ops.cu:63-72, and the byte receipt that the reference's
- * live_variables() (include/microtorch/autograd.hpp:61-64) cannot give. */
+ * live_variables() (include/microtorch/autograd.hpp:61-64) cannot give.
+ * A freed block is handed out again at once, without waiting for the GPU: that
+ * is safe for work queued on ONE stream (later work on that stream runs after
+ * the earlier work that used the block), which is how one model's tape runs.
+ * Memory that several streams touch must come from elsewhere. */
 int pk_alloc(size_t bytes, void** out);
 int pk_free(void* p);
 size_t pk_live_bytes(void);

@@ -38,7 +38,7 @@ size_t round_up(size_t n) {
     if (n < (1u << 20)) return (n + 511) & ~size_t(511);
     return (n + ((1u << 20) - 1)) & ~size_t((1u << 20) - 1);  // 1 MiB granules above 1 MiB
 }
-hipStream_t g_stream = nullptr;
+thread_local hipStream_t g_stream = nullptr;  // per host thread: the block operators of the C ABI set it around each call
 }  // namespace
 
 hipStream_t tape_stream() { return g_stream; }
@@ -660,7 +660,7 @@ void k_adamw(const Tensor& p, const Tensor& g, const Tensor& m, const Tensor& v,
 // ---- GEMM -------------------------------------------------------------------
 namespace {
 rocblas_handle blas() {
-    static rocblas_handle h = [] {
+    static thread_local rocblas_handle h = [] {  // a rocBLAS handle serves one host thread at a time
         rocblas_handle x;
         if (rocblas_create_handle(&x) != rocblas_status_success) throw std::runtime_error("rocblas_create_handle failed");
         // no atomics-based split-K: a recomputed (checkpointed) block must reproduce its first forward bit for bit
