@@ -33,30 +33,32 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
 MEASURED_TRAFFIC_BYTES = {"dkdv": 5.11e8, "dq": 4.30e8, "fwd": 3.38e8}  # profiles/attn_*_pmc.txt, fetch x2.0 + write x1.0
 
 
-def cpu_baseline(B, T, H, dk, scale, seconds_budget=30.0):
-    """The reference's CPU attention (ops.cpp path) on ONE (batch, head) unit of
+def cpu_baseline(B, T, H, dk, scale):
+    """The reference's CPU attention (ops.cpp path) on two of the (batch, head) units of
     the same workload, single thread, timed with a wall clock; the rate is
     FLOPs-per-unit / time, so it compares with `value` directly."""
     import numpy as np
     from oracle.bindings import Oracle, load_reference
     from paperkiln_amd import synth
 
-    q = synth.bf16_round(synth.randn(11, (T, dk), 0.5))
-    k = synth.bf16_round(synth.randn(12, (T, dk), 0.5))
-    v = synth.bf16_round(synth.randn(13, (T, dk), 0.5))
-    g = synth.bf16_round(synth.randn(14, (T, dk), 1.0))
+    units = 2  # about 8 s each on one core
     flops_unit = 14.0 * dk * (T * (T + 1) // 2)
     ref = load_reference()
-    t0 = time.perf_counter()
-    if ref is not None:
-        ref.fused_attention(q, k, v, scale, 0, True, dy=g)
-        kind = "reference"
-    else:
-        orc = Oracle()
-        _, _, A = orc.head_fwd(q, k, v, scale, 0, True, 0, 0)
-        orc.head_bwd(q, k, v, A, g, scale, 0, True, 0, 0)
-        kind = "port"
-    dt = time.perf_counter() - t0
+    orc = None if ref is not None else Oracle()
+    kind = "reference" if ref is not None else "port"
+    dt = 0.0
+    for u in range(units):
+        q = synth.bf16_round(synth.randn(11 + 10 * u, (T, dk), 0.5))
+        k = synth.bf16_round(synth.randn(12 + 10 * u, (T, dk), 0.5))
+        v = synth.bf16_round(synth.randn(13 + 10 * u, (T, dk), 0.5))
+        g = synth.bf16_round(synth.randn(14 + 10 * u, (T, dk), 1.0))
+        t0 = time.perf_counter()
+        if ref is not None:
+            ref.fused_attention(q, k, v, scale, 0, True, dy=g)
+        else:
+            _, _, A = orc.head_fwd(q, k, v, scale, 0, True, 0, 0)
+            orc.head_bwd(q, k, v, A, g, scale, 0, True, 0, 0)
+        dt += time.perf_counter() - t0
     cpu = "unknown"
     try:
         for line in open("/proc/cpuinfo"):
@@ -65,9 +67,9 @@ def cpu_baseline(B, T, H, dk, scale, seconds_budget=30.0):
                 break
     except OSError:
         pass
-    return {"value": flops_unit / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": kind,
-            "sample": f"1 of {B * H} (batch, head) units of the same workload, fwd+bwd, {dt:.2f} s wall; "
-                      f"whole job would take ~{dt * B * H:.0f} s on one core",
+    return {"value": units * flops_unit / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": kind,
+            "sample": f"{units} of {B * H} (batch, head) units of the same workload, fwd+bwd, {dt:.2f} s wall; "
+                      f"whole job would take ~{dt / units * B * H:.0f} s on one core",
             "host_cpu": cpu, "host_nproc": os.cpu_count()}
 
 
