@@ -243,3 +243,28 @@ def test_full_size_cfg2_cfg3(oracle, name, B, T, Hq, Hkv, theta):
         sv = dv2.view(B, T, Hkv, rep, dk).sum(dim=3)
         assert float((sk - dk_).abs().max()) < 1e-3 * float(dk_.abs().max()) + 1e-4  # fp32 sums in another order
         assert float((sv - dv).abs().max()) < 1e-3 * float(dv.abs().max()) + 1e-4
+
+
+def test_long_sequence_prefix_property():
+    """T = 32768 (one head): by causality the first 4096 rows of every output equal the T = 4096 problem on the
+    prefix, bitwise for the forward; the backward of the prefix problem equals the long one when dO is zero past
+    the prefix. Exercises index arithmetic far beyond the sizes the oracle can reach."""
+    B, T, H, dk, P = 1, 32768, 1, 128, 4096
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
+    g = torch.Generator(device="cuda").manual_seed(9)
+    q, k, v = ((torch.randn((B, T, H, dk), generator=g, device="cuda") * 0.5).bfloat16() for _ in range(3))
+    d_o = torch.randn((B, T, H, dk), generator=g, device="cuda").bfloat16()
+    d_o[:, P:] = 0
+    o, lse = ops.attn_fwd(q, k, v, scale, True)
+    op, lsep = ops.attn_fwd(q[:, :P], k[:, :P], v[:, :P], scale, True)
+    assert torch.equal(o[:, :P], op) and torch.equal(lse[:, :, :P], lsep)
+    assert bool(torch.isfinite(o.float()).all()) and bool(torch.isfinite(lse).all())
+    # LSE of the last row against a direct evaluation of that one row
+    s_last = (k[0, :, 0].float() @ q[0, -1, 0].float()) * scale
+    assert abs(float(torch.logsumexp(s_last, 0)) - float(lse[0, 0, -1])) < BF16_LSE_TOL
+    dq, dk_, dv = ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, grad_dtype=torch.float32)
+    dqp, dkp, dvp = ops.attn_bwd(q[:, :P], k[:, :P], v[:, :P], op, lsep, d_o[:, :P], scale, True, grad_dtype=torch.float32)
+    assert torch.equal(dq[:, :P], dqp) and float(dq[:, P:].abs().max()) == 0.0
+    assert float(dk_[:, P:].abs().max()) == 0.0 and float(dv[:, P:].abs().max()) == 0.0
+    assert float((dk_[:, :P] - dkp).abs().max()) < 1e-4 * float(dkp.abs().max()) + 1e-5
+    assert float((dv[:, :P] - dvp).abs().max()) < 1e-4 * float(dvp.abs().max()) + 1e-5
