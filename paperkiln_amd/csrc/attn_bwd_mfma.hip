@@ -337,6 +337,8 @@ __global__ __launch_bounds__(256, 2) void mfma_dq(AttnArgs a) {
                 f32x16 s, dp;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.0f;
+                // matrix phases issue ahead of co-resident waves' exponent phases
+                __builtin_amdgcn_s_setprio(1);
 #pragma unroll
                 for (int kk = 0; kk < KK; ++kk) {
                     const bf16x8 kf = lds_read8(Ks + (nb * 32 + c32) * KT::S + kk * 16 + g * 8);
@@ -344,6 +346,7 @@ __global__ __launch_bounds__(256, 2) void mfma_dq(AttnArgs a) {
                     const bf16x8 vf = lds_read8(Vs + (nb * 32 + c32) * KT::S + kk * 16 + g * 8);
                     dp = mfma32(vf, greg[kk], dp);
                 }
+                __builtin_amdgcn_s_setprio(0);
                 // lane = query qi; element r = key n0 + nb*32 + (r/4)*8 + 4g + r%4
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
@@ -352,6 +355,7 @@ __global__ __launch_bounds__(256, 2) void mfma_dq(AttnArgs a) {
                     dp[r] = p * (dp[r] - dl);
                 }
                 const bf16x8 d0 = c_to_operand<0>(dp), d1 = c_to_operand<1>(dp);
+                __builtin_amdgcn_s_setprio(1);
                 // dQ^T += K^T dS^T, DB independent chains per k-chunk
 #pragma unroll
                 for (int db = 0; db < DB; ++db)
@@ -359,6 +363,7 @@ __global__ __launch_bounds__(256, 2) void mfma_dq(AttnArgs a) {
 #pragma unroll
                 for (int db = 0; db < DB; ++db)
                     dq_acc[db] = mfma32(lds_read_tr_operand_perm<D>(Ks, KT::S, nb * 32 + 16, db, lane), d1, dq_acc[db]);
+                __builtin_amdgcn_s_setprio(0);
             }
         }
         __syncthreads();

@@ -172,6 +172,9 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
             f32x16 s[2];
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[0][r] = s[1][r] = 0.0f;
+            // Waves in a matrix phase issue ahead of co-resident waves in the
+            // exponent phase: the matrix pipe is the scarcer resource.
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int kk = 0; kk < KK; ++kk) {
                 const bf16x8 k0f = lds_read8(Ks + c32 * C::KS + kk * 16 + g * 8);
@@ -179,6 +182,7 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
                 s[0] = mfma32(k0f, qreg[qb][kk], s[0]);
                 s[1] = mfma32(k1f, qreg[qb][kk], s[1]);
             }
+            __builtin_amdgcn_s_setprio(0);
             PK_TICK(0)
             const bool full = (n0 + BN - 1 < a.T) && (!a.causal || n0 + BN - 1 <= qlo) &&
                               (a.window == 0 || n0 + a.window > qhi || n0 + BN - 1 < a.sinks);
@@ -221,6 +225,7 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
             l[qb] += psum;  // per-lane partial; the two halves meet in the epilogue
             PK_TICK(1)
 
+            __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) {
                 const bf16x8 p0 = c_to_operand<0>(s[nb]);
@@ -232,6 +237,7 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
                 for (int db = 0; db < DB; ++db)
                     acc_o[qb][db] = mfma32(lds_read_tr_operand(Vs, C::VS, nb * 32 + 16, db * 32, lane), p1, acc_o[qb][db]);
             }
+            __builtin_amdgcn_s_setprio(0);
         }
 
         PK_TICK(2)
