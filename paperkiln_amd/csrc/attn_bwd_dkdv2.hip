@@ -55,7 +55,9 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
     __shared__ __attribute__((aligned(16))) float nlse_s[3][BMQ];            // -LSE * log2(e)
     __shared__ __attribute__((aligned(16))) float dl_s[3][BMQ];
 
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    // the wavefront index as a scalar: every test on it becomes a scalar branch
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int role = w >> 2, kbw = w & 3;
     const int g = lane >> 5, c32 = lane & 31;
     const int nkb = (a.T + BNK - 1) / BNK, rep = a.Hq / a.Hkv;
@@ -202,11 +204,13 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
                         for (int qd = 0; qd < 4; ++qd) {
                             const f32x4 nl = *reinterpret_cast<const f32x4*>(&nlse_s[s % 3][qb * 32 + qd * 8 + g * 4]);
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                float p = __builtin_amdgcn_exp2f(fmaf(sc[qd * 4 + e], cexp, nl[e]));
-                                if (!full) p = kvis(qlo + qd * 8 + g * 4 + e) ? p : 0.0f;
-                                sc[qd * 4 + e] = p;
-                            }
+                            for (int e = 0; e < 4; ++e)
+                                sc[qd * 4 + e] = __builtin_amdgcn_exp2f(fmaf(sc[qd * 4 + e], cexp, nl[e]));
+                        }
+                        if (!full) {  // off the common path: interior tiles carry no mask arithmetic at all
+#pragma unroll
+                            for (int r = 0; r < 16; ++r)
+                                sc[r] = kvis(qlo + (r >> 2) * 8 + g * 4 + (r & 3)) ? sc[r] : 0.0f;
                         }
                         const bf16x8 p0 = c_to_operand<0>(sc), p1 = c_to_operand<1>(sc);
                         // hand-over copy in fp16: P is in [0, 1], where fp16 carries 11 significant

@@ -129,7 +129,9 @@ __global__ __launch_bounds__(256, PK_DKDV_OCC) void mfma_dkdv(AttnArgs a) {
     __shared__ __attribute__((aligned(16))) float nlse_s[BMQ];  // -LSE * log2(e)
     __shared__ __attribute__((aligned(16))) float dl_s[BMQ];
 
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    // the wavefront index as a scalar: every test on it becomes a scalar branch
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = lane >> 5, c32 = lane & 31;
     const int nkb = (a.T + BNK - 1) / BNK, rep = a.Hq / a.Hkv;
     // Full-causal: key block i is seen by T - 128i queries; blocks i and nkb-1-i
@@ -222,10 +224,17 @@ __global__ __launch_bounds__(256, PK_DKDV_OCC) void mfma_dkdv(AttnArgs a) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int r = qd * 4 + e;
-                    float p = __builtin_amdgcn_exp2f(fmaf(s[r], cexp, nl[e]));
-                    if (!full) p = kvis(qlo + qd * 8 + g * 4 + e) ? p : 0.0f;
+                    const float p = __builtin_amdgcn_exp2f(fmaf(s[r], cexp, nl[e]));
                     s[r] = p;
                     dp[r] = p * (dp[r] - dl[e]);
+                }
+            }
+            if (!full) {  // off the common path: interior tiles carry no mask arithmetic at all
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const bool vis = kvis(qlo + (r >> 2) * 8 + g * 4 + (r & 3));
+                    s[r] = vis ? s[r] : 0.0f;
+                    dp[r] = vis ? dp[r] : 0.0f;
                 }
             }
             const bf16x8 p0 = c_to_operand<0>(s), p1 = c_to_operand<1>(s);
@@ -276,7 +285,9 @@ __global__ __launch_bounds__(256, 2) void mfma_dq(AttnArgs a) {
     __shared__ __attribute__((aligned(16))) uint16_t Ks[BN * KT::S];
     __shared__ __attribute__((aligned(16))) uint16_t Vs[BN * KT::S];
 
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    // the wavefront index as a scalar: every test on it becomes a scalar branch
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = lane >> 5, c32 = lane & 31;
     const int nqb = (a.T + BM - 1) / BM, rep = a.Hq / a.Hkv;
     const bool paired = a.causal && a.window == 0;  // as in the forward kernel
@@ -349,10 +360,11 @@ __global__ __launch_bounds__(256, 2) void mfma_dq(AttnArgs a) {
                 __builtin_amdgcn_s_setprio(0);
                 // lane = query qi; element r = key n0 + nb*32 + (r/4)*8 + 4g + r%4
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    float p = __builtin_amdgcn_exp2f(fmaf(s[r], cexp, nlse));
-                    if (!full) p = qvis(n0 + nb * 32 + (r >> 2) * 8 + g * 4 + (r & 3)) ? p : 0.0f;
-                    dp[r] = p * (dp[r] - dl);
+                for (int r = 0; r < 16; ++r) dp[r] = __builtin_amdgcn_exp2f(fmaf(s[r], cexp, nlse)) * (dp[r] - dl);
+                if (!full) {  // off the common path: interior tiles carry no mask arithmetic at all
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        dp[r] = qvis(n0 + nb * 32 + (r >> 2) * 8 + g * 4 + (r & 3)) ? dp[r] : 0.0f;
                 }
                 const bf16x8 d0 = c_to_operand<0>(dp), d1 = c_to_operand<1>(dp);
                 __builtin_amdgcn_s_setprio(1);

@@ -85,7 +85,9 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
     __shared__ __attribute__((aligned(16))) uint16_t Kbuf[2][BN * C::KS];
     __shared__ __attribute__((aligned(16))) uint16_t Vbuf[2][BN * C::VS];
 
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    // the wavefront index as a scalar: every test on it becomes a scalar branch
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = lane >> 5, c32 = lane & 31;
     const int nqb = (a.T + BM - 1) / BM, rep = a.Hq / a.Hkv;
     // Full-causal work per query block grows linearly with its index, so a
