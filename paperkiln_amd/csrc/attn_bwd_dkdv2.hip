@@ -49,8 +49,9 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
     constexpr int S = D + 8;            // tile row pitch (elements): 16-byte row reads conflict-free
     constexpr int NCH = D / 8;          // 16-byte chunks per row
     constexpr int CPT = BMQ * NCH / 512;  // chunks per thread per tensor per step
-    __shared__ __attribute__((aligned(16))) uint16_t Qs[3][BMQ * S];
-    __shared__ __attribute__((aligned(16))) uint16_t dOs[3][BMQ * S];
+    __shared__ __attribute__((aligned(16))) uint16_t tiles[2][3][BMQ * S];  // [Q | dO][ring slot]
+    uint16_t (*const Qs)[BMQ * S] = tiles[0];
+    uint16_t (*const dOs)[BMQ * S] = tiles[1];
     __shared__ __attribute__((aligned(16))) uint16_t Pbuf[2][2][4][64 * 16];  // [step parity][query block][key block][lane][16]
     __shared__ __attribute__((aligned(16))) float nlse_s[3][BMQ];            // -LSE * log2(e)
     __shared__ __attribute__((aligned(16))) float dl_s[3][BMQ];
@@ -60,6 +61,10 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int role = w >> 2, kbw = w & 3;
     const int g = lane >> 5, c32 = lane & 31;
+    // Lane parts of the two LDS operand addresses (elements): a 16-byte row read at
+    // (row c32, column 8g) and a transposing read as lds_read_tr_operand_perm lays it out.
+    const int row_lane = c32 * S + g * 8;
+    const int tr_lane = (4 * g + ((lane & 15) >> 2)) * S + TrMap<D>::src_col(0, (lane >> 4) & 1, lane & 3);
     const int nkb = (a.T + BNK - 1) / BNK, rep = a.Hq / a.Hkv;
     // Full-causal: key block i is seen by T - 128i queries; blocks i and nkb-1-i
     // are taken back to back so that every workgroup carries the same work.
@@ -101,7 +106,6 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
         for (int db = 0; db < DB; ++db)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[db][r] = 0.0f;
-        const KeyVis kvis(kj, a.T, a.causal, a.window, a.sinks);
 
         // Query tiles that can see keys [k0, k0+127] (paperkiln src/ops.cpp:960-965 inverted).
         const int khi = min(k0 + BNK, a.T) - 1;
@@ -132,16 +136,21 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
             }
         };
         auto commit = [&](int slot) {  // registers -> LDS ring slot
+            // The store addresses are rebuilt from the thread index at every call (the
+            // empty statement hides its value): a handful of shifts, where addresses
+            // kept live across the step were the ones the allocator sent to scratch.
+            int tid = threadIdx.x;
+            asm volatile("" : "+v"(tid));
 #pragma unroll
             for (int i = 0; i < CPT; ++i) {
-                const int c = threadIdx.x + 512 * i;
+                const int c = tid + 512 * i;
                 const int row = c / NCH, ch = c % NCH;
                 *reinterpret_cast<u32x4*>(Qs[slot] + row * S + ch * 8) = qr[i];
                 *reinterpret_cast<u32x4*>(dOs[slot] + row * S + ch * 8) = gr[i];
             }
-            if (threadIdx.x < BMQ) {
-                nlse_s[slot][threadIdx.x] = lse_r;
-                dl_s[slot][threadIdx.x] = dl_r;
+            if (tid < BMQ) {
+                nlse_s[slot][tid] = lse_r;
+                dl_s[slot][tid] = dl_r;
             }
         };
         // wavefront-uniform: is anything of (query block qb of step `step`) x (this key block) visible?
@@ -168,6 +177,15 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
 #else
 #define PK_TICK(i)
 #endif
+        // transposed operand (k-chunk = rows row0 + {4g..4g+3} u {8+4g..}) of column block db, from a
+        // pointer that already carries the lane part
+        auto tr_operand = [&](const uint16_t* p, int row0, int db) {
+            p += row0 * S + TrMap<D>::src_col(db, 0, 0);
+            const s16x4 lo = lds_read_tr4(p), hi = lds_read_tr4(p + 8 * S);
+            typedef short s16x8 __attribute__((ext_vector_type(8)));
+            const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            return *reinterpret_cast<const bf16x8*>(&v);
+        };
         // iteration s: role 0 works on step s, role 1 on step s-1
         for (int s = 0; s <= steps; ++s) {
             PK_TICK(3)
@@ -178,24 +196,26 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
             PK_TICK(0)
             if (role == 0) {
                 if (s < steps) {
-                    const uint16_t* Qt = Qs[s % 3];
-                    const uint16_t* Gt = dOs[s % 3];
+                    // One register each for the row-read and the transposing-read address of
+                        // this step; every fragment is then an immediate offset away. Left to
+                        // itself the compiler keeps a dozen pre-offset copies and spills.
+                    int xrow = (s % 3) * (BMQ * S) + row_lane;                  // Q rows
+                    int ytr = (3 + s % 3) * (BMQ * S) + tr_lane;                // dO transposed
+                    asm volatile("" : "+v"(xrow), "+v"(ytr));
+                    const uint16_t* flat = &tiles[0][0][0];
 #pragma unroll
                     for (int qb = 0; qb < 2; ++qb) {
                         int qlo;
                         if (!block_live(s, qb, qlo)) continue;
-                        // two accumulator chains (even / odd k-chunks): a dependent MFMA pair
-                        // costs 52 cycles, an independent one 32
-                        f32x16 sc, sc2;
+                        // One accumulator chain: the other role's wavefront on this SIMD issues
+                        // into the gaps a dependent MFMA pair leaves, and the registers of a
+                        // second chain would push the kernel into scratch.
+                        f32x16 sc;
 #pragma unroll
-                        for (int r = 0; r < 16; ++r) sc[r] = sc2[r] = 0.0f;
+                        for (int r = 0; r < 16; ++r) sc[r] = 0.0f;
 #pragma unroll
-                        for (int kk = 0; kk < KK; kk += 2) {
-                            sc = mfma32(lds_read8(Qt + (qb * 32 + c32) * S + kk * 16 + g * 8), kv[kk], sc);
-                            sc2 = mfma32(lds_read8(Qt + (qb * 32 + c32) * S + (kk + 1) * 16 + g * 8), kv[kk + 1], sc2);
-                        }
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) sc[r] += sc2[r];
+                        for (int kk = 0; kk < KK; ++kk)
+                            sc = mfma32(lds_read8(flat + xrow + qb * 32 * S + kk * 16), kv[kk], sc);
                         const int qhi = qlo + 31;
                         const bool full = qhi < a.T && kw0 + 31 < a.T && (!a.causal || kw0 + 31 <= qlo) &&
                                           (a.window == 0 || kw0 + a.window > qhi || kw0 + 31 < a.sinks);
@@ -208,6 +228,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
                                 sc[qd * 4 + e] = __builtin_amdgcn_exp2f(fmaf(sc[qd * 4 + e], cexp, nl[e]));
                         }
                         if (!full) {  // off the common path: interior tiles carry no mask arithmetic at all
+                            const KeyVis kvis(kj, a.T, a.causal, a.window, a.sinks);
 #pragma unroll
                             for (int r = 0; r < 16; ++r)
                                 sc[r] = kvis(qlo + (r >> 2) * 8 + g * 4 + (r & 3)) ? sc[r] : 0.0f;
@@ -227,31 +248,29 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
                         // dV^T += dO^T P
 #pragma unroll
                         for (int db = 0; db < DB; ++db)
-                            acc[db] = mfma32(lds_read_tr_operand_perm<D>(Gt, S, qb * 32, db, lane), p0, acc[db]);
+                            acc[db] = mfma32(tr_operand(flat + ytr, qb * 32, db), p0, acc[db]);
 #pragma unroll
                         for (int db = 0; db < DB; ++db)
-                            acc[db] = mfma32(lds_read_tr_operand_perm<D>(Gt, S, qb * 32 + 16, db, lane), p1, acc[db]);
+                            acc[db] = mfma32(tr_operand(flat + ytr, qb * 32 + 16, db), p1, acc[db]);
                     }
                 }
             } else {
                 if (s >= 1) {
                     const int sp = s - 1;
-                    const uint16_t* Qt = Qs[sp % 3];
-                    const uint16_t* Gt = dOs[sp % 3];
+                    int xrow = (3 + sp % 3) * (BMQ * S) + row_lane;             // dO rows
+                    int ytr = (sp % 3) * (BMQ * S) + tr_lane;                   // Q transposed
+                    asm volatile("" : "+v"(xrow), "+v"(ytr));
+                    const uint16_t* flat = &tiles[0][0][0];
 #pragma unroll
                     for (int qb = 0; qb < 2; ++qb) {
                         int qlo;
                         if (!block_live(sp, qb, qlo)) continue;
-                        f32x16 dp, dp2;
+                        f32x16 dp;
 #pragma unroll
-                        for (int r = 0; r < 16; ++r) dp[r] = dp2[r] = 0.0f;
+                        for (int r = 0; r < 16; ++r) dp[r] = 0.0f;
 #pragma unroll
-                        for (int kk = 0; kk < KK; kk += 2) {
-                            dp = mfma32(lds_read8(Gt + (qb * 32 + c32) * S + kk * 16 + g * 8), kv[kk], dp);
-                            dp2 = mfma32(lds_read8(Gt + (qb * 32 + c32) * S + (kk + 1) * 16 + g * 8), kv[kk + 1], dp2);
-                        }
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) dp[r] += dp2[r];
+                        for (int kk = 0; kk < KK; ++kk)
+                            dp = mfma32(lds_read8(flat + xrow + qb * 32 * S + kk * 16), kv[kk], dp);
                         const uint16_t* pb = Pbuf[sp & 1][qb][kbw] + lane * 16;
                         u32x4 praw[2];
                         praw[0] = *reinterpret_cast<const u32x4*>(pb);
@@ -270,10 +289,10 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
                         // dK^T += Q^T dS
 #pragma unroll
                         for (int db = 0; db < DB; ++db)
-                            acc[db] = mfma32(lds_read_tr_operand_perm<D>(Qt, S, qb * 32, db, lane), d0, acc[db]);
+                            acc[db] = mfma32(tr_operand(flat + ytr, qb * 32, db), d0, acc[db]);
 #pragma unroll
                         for (int db = 0; db < DB; ++db)
-                            acc[db] = mfma32(lds_read_tr_operand_perm<D>(Qt, S, qb * 32 + 16, db, lane), d1, acc[db]);
+                            acc[db] = mfma32(tr_operand(flat + ytr, qb * 32 + 16, db), d1, acc[db]);
                     }
                 }
             }
