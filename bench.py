@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
 # HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs
 # (FETCH_SIZE, WRITE_SIZE) scaled by a copy kernel of known size; see
 # profiles/. None until measured for the current kernel.
-MEASURED_TRAFFIC_BYTES = {"dkdv": 5.11e8, "dq": 4.30e8, "fwd": 3.38e8}  # profiles/attn_*_pmc.txt, fetch x2.0 + write x1.0
+MEASURED_TRAFFIC_BYTES = {"dkdv": 4.05e8, "dq": 4.15e8, "fwd": 3.66e8}  # profiles/attn_*_pmc.txt, fetch x2.0 + write x1.0
 
 
 def cpu_baseline(B, T, H, dk, scale):
@@ -141,8 +141,9 @@ def llama_step():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=200)
+    # the card leaves its idle clock state only under sustained load: a short warm-up would time the ramp
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--sections", default="window,llama",
                     help="extra measurements beside the headline: any of window,llama (empty = headline only, "

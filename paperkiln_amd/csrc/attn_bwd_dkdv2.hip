@@ -52,7 +52,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
     __shared__ __attribute__((aligned(16))) uint16_t tiles[2][3][BMQ * S];  // [Q | dO][ring slot]
     uint16_t (*const Qs)[BMQ * S] = tiles[0];
     uint16_t (*const dOs)[BMQ * S] = tiles[1];
-    __shared__ __attribute__((aligned(16))) uint16_t Pbuf[2][2][4][64 * 16];  // [step parity][query block][key block][lane][16]
+    __shared__ __attribute__((aligned(16))) uint16_t Pbuf[2][2][4][2 * 64 * 8];  // [step parity][query block][key block][half][lane][8]
     __shared__ __attribute__((aligned(16))) float nlse_s[3][BMQ];            // -LSE * log2(e)
     __shared__ __attribute__((aligned(16))) float dl_s[3][BMQ];
 
@@ -236,7 +236,9 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
                         const bf16x8 p0 = c_to_operand<0>(sc), p1 = c_to_operand<1>(sc);
                         // hand-over copy in fp16: P is in [0, 1], where fp16 carries 11 significant
                         // bits against bf16's 8, so dS is built from a P as good as the old fp32 one
-                        uint16_t* pb = Pbuf[s & 1][qb][kbw] + lane * 16;
+                        // the two 16-byte halves of a lane sit 1 KB apart: consecutive lanes then
+                        // write consecutive 16-byte chunks and no two lanes share a bank
+                        uint16_t* pb = Pbuf[s & 1][qb][kbw] + lane * 8;
                         h16x2 ph[8];
 #pragma unroll
                         for (int i = 0; i < 8; ++i) {
@@ -244,7 +246,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
                             ph[i] = __builtin_convertvector(pr, h16x2);  // round to nearest even
                         }
                         *reinterpret_cast<u32x4*>(pb) = *reinterpret_cast<u32x4*>(&ph[0]);
-                        *reinterpret_cast<u32x4*>(pb + 8) = *reinterpret_cast<u32x4*>(&ph[4]);
+                        *reinterpret_cast<u32x4*>(pb + 512) = *reinterpret_cast<u32x4*>(&ph[4]);
                         // dV^T += dO^T P
 #pragma unroll
                         for (int db = 0; db < DB; ++db)
@@ -271,10 +273,10 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
 #pragma unroll
                         for (int kk = 0; kk < KK; ++kk)
                             dp = mfma32(lds_read8(flat + xrow + qb * 32 * S + kk * 16), kv[kk], dp);
-                        const uint16_t* pb = Pbuf[sp & 1][qb][kbw] + lane * 16;
+                        const uint16_t* pb = Pbuf[sp & 1][qb][kbw] + lane * 8;
                         u32x4 praw[2];
                         praw[0] = *reinterpret_cast<const u32x4*>(pb);
-                        praw[1] = *reinterpret_cast<const u32x4*>(pb + 8);
+                        praw[1] = *reinterpret_cast<const u32x4*>(pb + 512);
                         const h16x2* ph = reinterpret_cast<const h16x2*>(praw);
                         // dS = P .* (dP - delta); P arrives as fp16 pairs of elements (2i, 2i+1)
 #pragma unroll
