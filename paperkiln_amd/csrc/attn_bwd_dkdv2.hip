@@ -170,13 +170,6 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
         }
         __syncthreads();
 
-#ifdef PK_TIMING
-        long long tacc[4] = {0, 0, 0, 0};
-        long long tprev = __builtin_readcyclecounter();
-#define PK_TICK(i) { long long now = __builtin_readcyclecounter(); tacc[i] += now - tprev; tprev = now; }
-#else
-#define PK_TICK(i)
-#endif
         // transposed operand (k-chunk = rows row0 + {4g..4g+3} u {8+4g..}) of column block db, from a
         // pointer that already carries the lane part
         auto tr_operand = [&](const uint16_t* p, int row0, int db) {
@@ -188,12 +181,10 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
         };
         // iteration s: role 0 works on step s, role 1 on step s-1
         for (int s = 0; s <= steps; ++s) {
-            PK_TICK(3)
             if (s + 1 < steps) {
                 commit((s + 1) % 3);  // slot last read (by role 1) before the previous barrier
                 if (s + 2 < steps) fetch(s + 2);
             }
-            PK_TICK(0)
             if (role == 0) {
                 if (s < steps) {
                     // One register each for the row-read and the transposing-read address of
@@ -298,17 +289,8 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
                     }
                 }
             }
-            PK_TICK(1)
             __syncthreads();
-            PK_TICK(2)
         }
-#ifdef PK_TIMING
-        if (a.lazy_t != 0.0f && lane == 0) {
-            long long* dbg = reinterpret_cast<long long*>(a.dq) + (static_cast<long long>(blockIdx.x) * 8 + w) * 8;
-            for (int q = 0; q < 4; ++q) dbg[q] += tacc[q];
-            dbg[4] += steps;
-        }
-#endif
 
         if (kj < a.T) {
             void* dst = role == 0 ? a.dv : a.dk;
@@ -338,16 +320,7 @@ int launch(const AttnArgs& a, hipStream_t st) {
 
 }  // namespace
 
-int launch_mfma_dkdv2(const AttnArgs& a0, hipStream_t st) {
-    AttnArgs a = a0;
-    a.lazy_t = 0.0f;
-#ifdef PK_TIMING
-    // timing build only: the dq pointer (unused by this kernel) carries the debug buffer
-    if (getenv("PK_DBG_PTR")) {
-        a.dq = reinterpret_cast<void*>(strtoull(getenv("PK_DBG_PTR"), nullptr, 0));
-        a.lazy_t = 1.0f;
-    }
-#endif
+int launch_mfma_dkdv2(const AttnArgs& a, hipStream_t st) {
     if (a.dk_dim == 128) return a.grad_f32 ? launch<128, true>(a, st) : launch<128, false>(a, st);
     return a.grad_f32 ? launch<64, true>(a, st) : launch<64, false>(a, st);
 }

@@ -11,13 +11,9 @@
 //
 // Three launches, no atomics, deterministic:
 //   mfma_delta    one pass over O and dO.
-//   mfma_dkdv     a workgroup owns 128 keys of one KV head (32 per wavefront,
-//                 K and V held in registers), loops over the query heads of
-//                 its GQA group and over the query tiles that can see it.
-//                 S = Q K^T and dP = dO V^T come out with lane = key, so
-//                 P and dS feed dV^T += dO^T P and dK^T += Q^T dS straight
-//                 from registers; Q^T / dO^T are transposing LDS reads of the
-//                 same row-major tiles.
+//   mfma_dkdv2    (attn_bwd_dkdv2.hip) a workgroup owns 128 keys of one KV
+//                 head and loops over the query heads of its GQA group and
+//                 over the query tiles that can see it.
 //   mfma_dq       a workgroup owns 128 queries of one head (32 per
 //                 wavefront, Q and dO in registers), loops over the visible
 //                 key tiles: S^T = K Q^T, dP^T = V dO^T (lane = query, so LSE
@@ -31,9 +27,6 @@ namespace pk {
 namespace {
 
 constexpr float LOG2E = 1.4426950408889634f;
-#ifndef PK_DKDV_OCC
-#define PK_DKDV_OCC 1
-#endif
 
 // ---- delta --------------------------------------------------------------
 template <int D>
@@ -115,165 +108,6 @@ __device__ inline void store4(void* base, int64_t idx, float x0, float x1, float
         u32x2 v = {pack_bf16(x0, x1), pack_bf16(x2, x3)};
         *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(base) + idx) = v;
     }
-}
-
-// ---- dK, dV ---------------------------------------------------------------
-template <int D, bool GF32>
-__global__ __launch_bounds__(256, PK_DKDV_OCC) void mfma_dkdv(AttnArgs a) {
-    constexpr int BMQ = 64;   // queries per step
-    constexpr int BNK = 128;  // keys per workgroup
-    constexpr int KK = D / 16, DB = D / 32;
-    using QT = Tile<D, BMQ>;
-    __shared__ __attribute__((aligned(16))) uint16_t Qs[BMQ * QT::S];
-    __shared__ __attribute__((aligned(16))) uint16_t dOs[BMQ * QT::S];
-    __shared__ __attribute__((aligned(16))) float nlse_s[BMQ];  // -LSE * log2(e)
-    __shared__ __attribute__((aligned(16))) float dl_s[BMQ];
-
-    const int lane = threadIdx.x & 63;
-    // the wavefront index as a scalar: every test on it becomes a scalar branch
-    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int g = lane >> 5, c32 = lane & 31;
-    const int nkb = (a.T + BNK - 1) / BNK, rep = a.Hq / a.Hkv;
-    // Full-causal: key block i is seen by T - 128i queries; blocks i and nkb-1-i
-    // are taken back to back so that every workgroup carries the same work.
-    const bool paired = a.causal && a.window == 0;
-    int blk, rr, kvu;
-    if (!xcd_map(paired ? (nkb + 1) / 2 : nkb, 1, a.Hkv * a.B, blk, rr, kvu)) return;
-    const int hk = kvu % a.Hkv, b = kvu / a.Hkv;
-    const int npass = (paired && blk != nkb - 1 - blk) ? 2 : 1;
-  for (int pass = 0; pass < npass; ++pass) {
-    const int kblk = pass == 0 ? blk : nkb - 1 - blk;  // heavy block first
-    const int k0 = kblk * BNK;
-    const int kw0 = k0 + w * 32;  // this wavefront's keys
-    const float cexp = a.scale * LOG2E;
-
-    bf16x8 kreg[KK], vreg[KK];
-    load_row_operand<D>(a.k, b * a.k_sb + hk * a.k_sh, a.k_st, kw0 + c32, a.T, g, kreg);
-    load_row_operand<D>(a.v, b * a.v_sb + hk * a.v_sh, a.v_st, kw0 + c32, a.T, g, vreg);
-
-    f32x16 dk_acc[DB], dv_acc[DB];
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) dk_acc[db][r] = dv_acc[db][r] = 0.0f;
-
-    // Query tiles that can see keys [k0, k0+127] (src/ops.cpp:960-965 inverted).
-    const int khi = min(k0 + BNK, a.T) - 1;
-    const int qt_lo = a.causal ? k0 / BMQ : 0;
-    const int qt_hi = (a.window > 0 && k0 >= a.sinks) ? min(a.T - 1, khi + a.window - 1) / BMQ
-                                                       : (a.T - 1) / BMQ;
-    const int nqt = qt_hi - qt_lo + 1;
-    const int steps = nqt * rep;
-
-    u32x4 qr[QT::CPT], gr[QT::CPT];
-    float lse_r = 0.0f, dl_r = 0.0f;
-    auto fetch = [&](int step) {
-        const int h = hk * rep + step / nqt, q0 = (qt_lo + step % nqt) * BMQ;
-        QT::load(a.q, b * a.q_sb + h * a.q_sh, a.q_st, q0, a.T, qr);
-        QT::load(a.d_o, b * a.do_sb + h * a.do_sh, a.do_st, q0, a.T, gr);
-        if (threadIdx.x < BMQ) {
-            const int t = q0 + threadIdx.x;
-            const int64_t lrow = (static_cast<int64_t>(b) * a.Hq + h) * a.T + t;
-            lse_r = t < a.T ? -a.lse[lrow] * LOG2E : 0.0f;
-            dl_r = t < a.T ? a.delta[lrow] : 0.0f;
-        }
-    };
-    auto commit = [&]() {
-        QT::store(Qs, qr);
-        QT::store(dOs, gr);
-        if (threadIdx.x < BMQ) {
-            nlse_s[threadIdx.x] = lse_r;
-            dl_s[threadIdx.x] = dl_r;
-        }
-    };
-    if (steps > 0) {
-        fetch(0);
-        commit();
-    }
-    __syncthreads();
-
-    for (int step = 0; step < steps; ++step) {
-        const int q0 = (qt_lo + step % nqt) * BMQ;
-        if (step + 1 < steps) fetch(step + 1);
-
-#pragma unroll
-        for (int qb = 0; qb < BMQ / 32; ++qb) {
-            const int qlo = q0 + qb * 32, qhi = qlo + 31;
-            if (qlo >= a.T || kw0 >= a.T) continue;
-            if (a.causal && kw0 > qhi) continue;
-            if (a.window > 0 && kw0 + 31 + a.window <= qlo && kw0 >= a.sinks) continue;
-
-            f32x16 s, dp;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.0f;
-#pragma unroll
-            for (int kk = 0; kk < KK; ++kk) {
-                const bf16x8 qf = lds_read8(Qs + (qb * 32 + c32) * QT::S + kk * 16 + g * 8);
-                s = mfma32(qf, kreg[kk], s);
-                const bf16x8 gf = lds_read8(dOs + (qb * 32 + c32) * QT::S + kk * 16 + g * 8);
-                dp = mfma32(gf, vreg[kk], dp);
-            }
-            const bool full = qhi < a.T && kw0 + 31 < a.T && (!a.causal || kw0 + 31 <= qlo) &&
-                              (a.window == 0 || kw0 + a.window > qhi || kw0 + 31 < a.sinks);
-            const KeyVis kvis(kw0 + c32, a.T, a.causal, a.window, a.sinks);
-            // lane = key kw0+c32; element r = query qlo + (r/4)*8 + 4g + r%4
-#pragma unroll
-            for (int qd = 0; qd < 4; ++qd) {
-                const f32x4 nl = *reinterpret_cast<const f32x4*>(nlse_s + qb * 32 + qd * 8 + g * 4);
-                const f32x4 dl = *reinterpret_cast<const f32x4*>(dl_s + qb * 32 + qd * 8 + g * 4);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int r = qd * 4 + e;
-                    const float p = __builtin_amdgcn_exp2f(fmaf(s[r], cexp, nl[e]));
-                    s[r] = p;
-                    dp[r] = p * (dp[r] - dl[e]);
-                }
-            }
-            if (!full) {  // off the common path: interior tiles carry no mask arithmetic at all
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const bool vis = kvis(qlo + (r >> 2) * 8 + g * 4 + (r & 3));
-                    s[r] = vis ? s[r] : 0.0f;
-                    dp[r] = vis ? dp[r] : 0.0f;
-                }
-            }
-            const bf16x8 p0 = c_to_operand<0>(s), p1 = c_to_operand<1>(s);
-            const bf16x8 d0 = c_to_operand<0>(dp), d1 = c_to_operand<1>(dp);
-            // dV^T += dO^T P ; dK^T += Q^T dS (A = transposed LDS tiles). Consecutive
-            // MFMAs go to different accumulators (a dependent pair costs 52 cycles, not 32).
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                dv_acc[db] = mfma32(lds_read_tr_operand_perm<D>(dOs, QT::S, qb * 32, db, lane), p0, dv_acc[db]);
-                dk_acc[db] = mfma32(lds_read_tr_operand_perm<D>(Qs, QT::S, qb * 32, db, lane), d0, dk_acc[db]);
-            }
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                dv_acc[db] = mfma32(lds_read_tr_operand_perm<D>(dOs, QT::S, qb * 32 + 16, db, lane), p1, dv_acc[db]);
-                dk_acc[db] = mfma32(lds_read_tr_operand_perm<D>(Qs, QT::S, qb * 32 + 16, db, lane), d1, dk_acc[db]);
-            }
-        }
-        __syncthreads();
-        if (step + 1 < steps) commit();
-        __syncthreads();
-    }
-
-    const int kj = kw0 + c32;
-    if (kj < a.T) {
-        const int64_t kb = b * a.dk_sb + hk * a.dk_sh + kj * a.dk_st;
-        const int64_t vb = b * a.dv_sb + hk * a.dv_sh + kj * a.dv_st;
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int qd = 0; qd < 4; ++qd) {
-                const int d0 = TrMap<D>::col0(db, qd, g);
-                store4<GF32>(a.dk, kb + d0, dk_acc[db][qd * 4] * a.scale, dk_acc[db][qd * 4 + 1] * a.scale,
-                             dk_acc[db][qd * 4 + 2] * a.scale, dk_acc[db][qd * 4 + 3] * a.scale);
-                store4<GF32>(a.dv, vb + d0, dv_acc[db][qd * 4], dv_acc[db][qd * 4 + 1],
-                             dv_acc[db][qd * 4 + 2], dv_acc[db][qd * 4 + 3]);
-            }
-    }
-    __syncthreads();  // the next pass refills the tile buffers
-  }
 }
 
 // ---- dQ -------------------------------------------------------------------
@@ -411,13 +245,8 @@ int launch(const AttnArgs& a, int stages, hipStream_t st) {
         hipLaunchKernelGGL((mfma_delta<D>), dim3((rows + RPB - 1) / RPB), dim3(256), 0, st, a);
         PK_HIP(hipGetLastError());
     }
-    static const bool old_dkdv = getenv("PK_DKDV_OLD") != nullptr;
-    if ((stages & PK_BWD_DKDV) && !old_dkdv) {
+    if (stages & PK_BWD_DKDV) {
         if (int rc = launch_mfma_dkdv2(a, st)) return rc;
-    } else if (stages & PK_BWD_DKDV) {
-        hipLaunchKernelGGL((mfma_dkdv<D, GF32>), dim3(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, 1, a.Hkv * a.B)), dim3(256),
-                           0, st, a);
-        PK_HIP(hipGetLastError());
     }
     if (stages & PK_BWD_DQ) {
         hipLaunchKernelGGL((mfma_dq<D, GF32>), dim3(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, a.Hq / a.Hkv, a.Hkv * a.B)),

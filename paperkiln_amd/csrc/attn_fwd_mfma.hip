@@ -147,13 +147,6 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
     __syncthreads();
     int cur = 0;
 
-#ifdef PK_TIMING
-    long long tacc[5] = {0, 0, 0, 0, 0};
-    long long tprev = __builtin_readcyclecounter();
-#define PK_TICK(i) { long long now = __builtin_readcyclecounter(); tacc[i] += now - tprev; tprev = now; }
-#else
-#define PK_TICK(i)
-#endif
     while (t <= hi) {
         const int n0 = t * BN;
         const int tn = (t + 1 == ns) ? lo : t + 1;
@@ -185,7 +178,6 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
                 s[1] = mfma32(k1f, qreg[qb][kk], s[1]);
             }
             __builtin_amdgcn_s_setprio(0);
-            PK_TICK(0)
             const bool full = (n0 + BN - 1 < a.T) && (!a.causal || n0 + BN - 1 <= qlo) &&
                               (a.window == 0 || n0 + a.window > qhi || n0 + BN - 1 < a.sinks);
             if (!full) {
@@ -204,7 +196,7 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[nb][r]);
             mx = xhalf_max(mx);
-            if (__any((mx - m[qb]) * cexp > a.lazy_t)) {  // wavefront-uniform, rare after the first tiles
+            if (__any((mx - m[qb]) * cexp > LAZY_T)) {  // wavefront-uniform, rare after the first tiles
                 const float mn = fmaxf(m[qb], mx);
                 const float alpha = __builtin_amdgcn_exp2f((m[qb] - mn) * cexp);
                 l[qb] *= alpha;
@@ -225,7 +217,6 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
                     psum += p;
                 }
             l[qb] += psum;  // per-lane partial; the two halves meet in the epilogue
-            PK_TICK(1)
 
             __builtin_amdgcn_s_setprio(1);
 #pragma unroll
@@ -242,23 +233,13 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
             __builtin_amdgcn_s_setprio(0);
         }
 
-        PK_TICK(2)
         // The other buffer was last read one iteration ago, before the previous barrier.
         if (tn <= hi) store_kv_lds<D>(Kbuf[cur ^ 1], Vbuf[cur ^ 1], kr, vr);
-        PK_TICK(3)
         __syncthreads();
-        PK_TICK(4)
         cur ^= 1;
         t = tn;
     }
 
-#ifdef PK_TIMING
-    if (a.delta && lane == 0) {
-        long long* dbg = reinterpret_cast<long long*>(a.delta) + (static_cast<long long>(blockIdx.x) * 4 + w) * 8;
-        for (int i = 0; i < 5; ++i) dbg[i] = tacc[i];
-        dbg[5] = hi + 1;
-    }
-#endif
     // Epilogue: O = acc / l, LSE = m*scale + ln(l) (natural log, scaled units).
 #pragma unroll
     for (int qb = 0; qb < NQ; ++qb) {
@@ -316,24 +297,9 @@ bool mfma_supported(const AttnArgs& a) {
     return true;
 }
 
-int launch_mfma_fwd(const AttnArgs& a0, hipStream_t st) {
-    AttnArgs a = a0;
-    a.lazy_t = getenv("PK_LAZY_T") ? atof(getenv("PK_LAZY_T")) : LAZY_T;
-#ifdef PK_TIMING
-    if (getenv("PK_DBG_PTR")) a.delta = reinterpret_cast<float*>(strtoull(getenv("PK_DBG_PTR"), nullptr, 0));
-#endif
-    // Two 32-query blocks per wavefront halve the LDS traffic per MFMA; short
-    // sequences keep one so that the grid still covers the chip.
-    static const int variant = getenv("PK_FWD_VARIANT") ? atoi(getenv("PK_FWD_VARIANT")) : 0;
-    const bool big = static_cast<int64_t>(a.T) * a.Hq * a.B >= 256 * 256 * 2;
-    if (a.dk_dim == 128) {
-        if (variant == 1) return launch<128, 1, 2>(a, st);
-        if (variant == 2) return launch<128, 1, 1>(a, st);
-        if (variant == 3) return launch<128, 2, 1>(a, st);
-        return launch<128, 1, 2>(a, st);
-    }
-    if (variant == 1) return launch<64, 1, 2>(a, st);
-    if (variant == 3) return launch<64, 2, 1>(a, st);
+int launch_mfma_fwd(const AttnArgs& a, hipStream_t st) {
+    // One 32-query block per wavefront, two workgroups per CU.
+    if (a.dk_dim == 128) return launch<128, 1, 2>(a, st);
     return launch<64, 1, 2>(a, st);
 }
 

@@ -45,7 +45,6 @@ struct AttnArgs {
     int causal, window, sinks;
     int grad_f32; // dq/dk/dv element type: 1 = fp32, 0 = bf16
     float scale;
-    float lazy_t; // debug
 };
 
 // Visible-set test shared by every kernel: the reference's two ranges
