@@ -87,11 +87,13 @@ int pk_attn_bwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k
                 const pk_tensor4* d_o, const pk_tensor4* dq, const pk_tensor4* dk,
                 const pk_tensor4* dv, void* workspace, size_t workspace_bytes, void* stream);
 
-/* The same backward, one launch at a time, so that a caller can bracket each
- * kernel with events: PK_BWD_DELTA (row sums D_i = sum_d O*dO into the
- * workspace), PK_BWD_DKDV (needs DELTA done), PK_BWD_DQ (needs DELTA done).
- * pk_attn_bwd == all three in that order. The reference has no counterpart:
- * its closure is a single host function (src/ops.cpp:902-933). */
+/* The same backward by parts, so that a caller can bracket kernels with
+ * events: PK_BWD_DELTA (row sums D_i = sum_d O*dO into the workspace),
+ * PK_BWD_DKDV (needs DELTA done), PK_BWD_DQ (needs DELTA done). On the bf16
+ * path DELTA | DQ in one call is a single kernel (dQ forms D_i for its own
+ * rows and writes them), and pk_attn_bwd == that kernel followed by DKDV.
+ * The reference has no counterpart: its closure is a single host function
+ * (src/ops.cpp:902-933). */
 enum { PK_BWD_DELTA = 1, PK_BWD_DKDV = 2, PK_BWD_DQ = 4, PK_BWD_ALL = 7 };
 int pk_attn_bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k,
                        const pk_tensor4* v, const pk_tensor4* o, const float* lse,

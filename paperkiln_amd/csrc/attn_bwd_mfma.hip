@@ -111,7 +111,10 @@ __device__ inline void store4(void* base, int64_t idx, float x0, float x1, float
 }
 
 // ---- dQ -------------------------------------------------------------------
-template <int D, bool GF32>
+// FUSE_DELTA: the workgroup also forms delta for its own 128 rows (it holds their dO
+// already; O costs one more row read), uses it and writes it for the dK/dV kernel,
+// which then has to run after this one. Saves the separate pass over O and dO.
+template <int D, bool GF32, bool FUSE_DELTA>
 __global__ __launch_bounds__(256, 2) void mfma_dq(AttnArgs a) {
     constexpr int BM = 128, BN = 64;
     constexpr int KK = D / 16, DB = D / 32;
@@ -140,9 +143,25 @@ __global__ __launch_bounds__(256, 2) void mfma_dq(AttnArgs a) {
     load_row_operand<D>(a.q, b * a.q_sb + h * a.q_sh, a.q_st, qi, a.T, g, qreg);
     load_row_operand<D>(a.d_o, b * a.do_sb + h * a.do_sh, a.do_st, qi, a.T, g, greg);
     float nlse = 0.0f, dl = 0.0f;
-    if (qi < a.T) {
-        const int64_t lrow = (static_cast<int64_t>(b) * a.Hq + h) * a.T + qi;
-        nlse = -a.lse[lrow] * LOG2E;
+    const int64_t lrow = (static_cast<int64_t>(b) * a.Hq + h) * a.T + qi;
+    if (qi < a.T) nlse = -a.lse[lrow] * LOG2E;
+    if (FUSE_DELTA) {
+        bf16x8 oreg[KK];  // zero rows past the end, as dO
+        load_row_operand<D>(a.o, b * a.o_sb + h * a.o_sh, a.o_st, qi, a.T, g, oreg);
+        float part = 0.0f;  // this lane's half of the row: d = 16kk + 8g .. +7
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const u32x4 ov = *reinterpret_cast<const u32x4*>(&oreg[kk]);
+            const u32x4 gv = *reinterpret_cast<const u32x4*>(&greg[kk]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                part = fmaf(__uint_as_float(ov[i] << 16), __uint_as_float(gv[i] << 16), part);
+                part = fmaf(__uint_as_float(ov[i] & 0xFFFF0000u), __uint_as_float(gv[i] & 0xFFFF0000u), part);
+            }
+        }
+        dl = xhalf_sum(part);
+        if (qi < a.T && g == 0) a.delta[lrow] = dl;
+    } else if (qi < a.T) {
         dl = a.delta[lrow];
     }
     const QueryVis qvis(qi, a.T, a.causal, a.window, a.sinks);
@@ -241,16 +260,21 @@ int launch(const AttnArgs& a, int stages, hipStream_t st) {
     constexpr int RPB = 256 / (D / 8);
     const int nb128 = (a.T + 127) / 128;
     const bool paired = a.causal && a.window == 0;
-    if (stages & PK_BWD_DELTA) {
+    const dim3 dq_grid(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, a.Hq / a.Hkv, a.Hkv * a.B));
+    // delta and dQ asked for together: dQ forms delta itself and runs first, dK/dV reads what it wrote
+    const bool fused = (stages & PK_BWD_DELTA) && (stages & PK_BWD_DQ);
+    if (fused) {
+        hipLaunchKernelGGL((mfma_dq<D, GF32, true>), dq_grid, dim3(256), 0, st, a);
+        PK_HIP(hipGetLastError());
+    } else if (stages & PK_BWD_DELTA) {
         hipLaunchKernelGGL((mfma_delta<D>), dim3((rows + RPB - 1) / RPB), dim3(256), 0, st, a);
         PK_HIP(hipGetLastError());
     }
     if (stages & PK_BWD_DKDV) {
         if (int rc = launch_mfma_dkdv2(a, st)) return rc;
     }
-    if (stages & PK_BWD_DQ) {
-        hipLaunchKernelGGL((mfma_dq<D, GF32>), dim3(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, a.Hq / a.Hkv, a.Hkv * a.B)),
-                           dim3(256), 0, st, a);
+    if (!fused && (stages & PK_BWD_DQ)) {
+        hipLaunchKernelGGL((mfma_dq<D, GF32, false>), dq_grid, dim3(256), 0, st, a);
         PK_HIP(hipGetLastError());
     }
     return PK_OK;
