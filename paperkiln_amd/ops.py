@@ -58,6 +58,12 @@ def attn_fwd(q, k, v, scale, causal=True, window=0, sinks=0):
 BWD_DELTA, BWD_DKDV, BWD_DQ, BWD_ALL = 1, 2, 4, 7
 
 
+def bwd_workspace_bytes(q, k, grad_dtype=None):
+    """Bytes of scratch pk_attn_bwd needs for these shapes (pk_attn_bwd_workspace_bytes)."""
+    sh = _shape(q, k, 1.0, True, 0, 0, grad_dtype or q.dtype)
+    return max(int(_lib.lib().pk_attn_bwd_workspace_bytes(C.byref(sh))), 16)
+
+
 def attn_bwd(q, k, v, o, lse, d_o, scale, causal=True, window=0, sinks=0, grad_dtype=None, out=None,
              stages=BWD_ALL):
     """Recompute backward from (Q, K, V, O, LSE, dO). Returns (dq, dk, dv);

@@ -115,6 +115,32 @@ def test_fp32_path_on_bf16_shapes_agrees(oracle):
     assert max(errs) < FP32_TOL
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+@pytest.mark.parametrize("window,sinks", [(0, 0), (48, 3)])
+def test_backward_by_parts_equals_one_call(dtype, window, sinks):
+    """pk_attn_bwd_stages: DELTA, DKDV, DQ one at a time (the separate delta kernel and the dQ kernel that reads
+    it) against the single call (dQ forms delta itself). The two sum delta in a different order, so the bar is
+    a few units in the last place of the gradient's storage type, not bitwise."""
+    B, T, Hq, Hkv, dk = 2, 300, 4, 2, 128
+    rng = np.random.default_rng(17)
+    q, k, v, d_o = (dev(rng.standard_normal((B, T, h, dk), dtype=np.float32), dtype) for h in (Hq, Hkv, Hkv, Hq))
+    scale = float(1 / np.sqrt(dk))
+    o, lse = ops.attn_fwd(q, k, v, scale, True, window, sinks)
+    one = ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, window, sinks)
+    out = tuple(torch.full_like(x, float("nan")) for x in (q, k, v))
+    ws = torch.empty(ops.bwd_workspace_bytes(q, k), dtype=torch.uint8, device="cuda")
+    for st in (ops.BWD_DELTA, ops.BWD_DKDV, ops.BWD_DQ):
+        ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, window, sinks, out=out + (ws,), stages=st)
+    torch.cuda.synchronize()
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -20
+    for name, a, b in zip(("dQ", "dK", "dV"), one, out):
+        a, b = host(a), host(b)
+        assert np.isfinite(b).all(), name
+        err, ref = maxabs(a, b), float(np.abs(a).max())
+        print(f"\n  {name}: max|one - parts| {err:.2e} (max |grad| {ref:.2e})", flush=True)
+        assert err <= 4 * ulp * ref, name
+
+
 def test_strided_qkv_views():
     """Heads read in place from a fused [N, 3d] projection (no repack)."""
     B, T, H, dk = 2, 256, 4, 64
