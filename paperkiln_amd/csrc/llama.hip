@@ -69,8 +69,10 @@ struct Model {
     std::vector<Block> blocks;
     std::vector<std::pair<std::string, Var>> named;
     bool checkpoint_blocks = false;
-    // AdamW state (nn.cpp:293-299)
-    std::vector<Tensor> m, v;
+    // Master weights, gradients and the two AdamW moments (nn.cpp:293-299) each live in ONE
+    // allocation, [1, slab_len] fp32, with every parameter's tensors as views at the same offset:
+    // zero_grad, the clip norm and the optimiser step are then one launch each, not one per parameter.
+    Tensor pslab, gslab, mslab, vslab;
     long t = 0;
 
     void reg(const std::string& name, const Var& p) { named.emplace_back(name, p); }
@@ -111,6 +113,35 @@ struct Model {
         norm_w = make_param(1, d, ones);
         reg("norm.weight", norm_w);
         if (!c.tie_embeddings) throw std::runtime_error("llama: only the tied head (lm_head = embed_tokens) is built");
+        build_slabs();
+    }
+
+    void build_slabs() {
+        std::vector<int64_t> off;
+        int64_t total = 0;
+        for (const auto& kv : named) {  // 256-byte granules keep every view aligned for the GEMMs
+            off.push_back(total);
+            total += (kv.second->data.numel() + 63) / 64 * 64;
+        }
+        pslab = Tensor::make(1, total, PK_F32);
+        gslab = Tensor::make(1, total, PK_F32);
+        k_fill(pslab, 0.0f);
+        k_fill(gslab, 0.0f);
+        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+        for (size_t i = 0; i < named.size(); ++i) {
+            Variable& p = *named[i].second;
+            auto view = [&](const Tensor& slab) {
+                Tensor t = slab;
+                t.rows = p.data.rows;
+                t.cols = p.data.cols;
+                t.off_bytes = off[i] * static_cast<int64_t>(sizeof(float));
+                return t;
+            };
+            Tensor w = view(pslab);
+            hip_check(hipMemcpy(w.ptr(), p.data.ptr(), sizeof(float) * p.data.numel(), hipMemcpyDeviceToDevice), "hipMemcpy");
+            p.data = w;
+            p.grad = view(gslab);
+        }
     }
 
     std::vector<Var> parameters() const {
@@ -246,9 +277,7 @@ int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets
             if (host_targets[i] < 0 || host_targets[i] >= m->cfg.vocab)
                 throw std::runtime_error("cross_entropy: target out of range");
         m->checkpoint_blocks = checkpoint_blocks != 0;
-        auto params = m->parameters();
-        zero_grad(params);
-        for (const auto& p : params) p->ensure_grad();  // persistent state, kept out of the activation receipt
+        k_fill(m->gslab, 0.0f);  // zero_grad: every parameter's gradient is a view of this slab
         auto ids = ints_to_dev(host_ids, n);
         auto tg = ints_to_dev(host_targets, n);
         // Everything allocated from here on, until backward returns, is activation memory.
@@ -293,25 +322,28 @@ int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets
 int pk_llama_adamw_step(void* h, float lr, float b1, float b2, float eps, float wd, float max_norm, float* total_norm) {
     return guarded([&] {
         Model* m = static_cast<Model*>(h);
-        auto params = m->parameters();
-        if (m->m.empty()) {
-            for (const auto& p : params) {
-                m->m.push_back(Tensor::make(p->data.rows, p->data.cols, PK_F32));
-                m->v.push_back(Tensor::make(p->data.rows, p->data.cols, PK_F32));
-                k_fill(m->m.back(), 0.0f);
-                k_fill(m->v.back(), 0.0f);
-            }
+        if (m->mslab.empty()) {
+            m->mslab = Tensor::make(1, m->pslab.cols, PK_F32);
+            m->vslab = Tensor::make(1, m->pslab.cols, PK_F32);
+            k_fill(m->mslab, 0.0f);
+            k_fill(m->vslab, 0.0f);
         }
+        // ops::clip_grad_norm over the slab (the padding between parameters is zero): double
+        // accumulation as the reference (ops.cpp:1047-1053), one host round trip.
         double tn = 0.0;
-        if (max_norm > 0.0f) tn = ops::clip_grad_norm(params, max_norm);
+        if (max_norm > 0.0f) {
+            Buffer parts(sizeof(double) * SUMSQ_MAX_PARTS);
+            const int nb = k_sumsq_parts(m->gslab, static_cast<double*>(parts.p));
+            tn = std::sqrt(k_sum_f64_to_host(static_cast<const double*>(parts.p), nb));
+            if (tn > max_norm && tn > 0.0) k_scale(m->gslab, static_cast<float>(max_norm / tn), m->gslab);
+        }
         if (total_norm) *total_norm = static_cast<float>(tn);
         ++m->t;
         const float c1 = 1.0f - std::pow(b1, static_cast<float>(m->t));
         const float c2 = 1.0f - std::pow(b2, static_cast<float>(m->t));
-        for (size_t k = 0; k < params.size(); ++k) {
-            if (params[k]->grad.empty()) continue;  // never accumulated (nn.cpp:309)
-            k_adamw(params[k]->data, params[k]->grad, m->m[k], m->v[k], lr, b1, b2, eps, wd, c1, c2);
-        }
+        // every parameter of this model receives a gradient each step, so the reference's "skip a
+        // parameter that never accumulated" (nn.cpp:309) never applies; padding stays at zero
+        k_adamw(m->pslab, m->gslab, m->mslab, m->vslab, lr, b1, b2, eps, wd, c1, c2);
         invalidate_shadows();
         hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
     });
