@@ -163,20 +163,25 @@ __global__ void ew_silu_bwd(const T* x, const T* dy, T* dx, int64_t n) {
 
 // silu(gate) .* up in one pass (the two tape nodes ops::silu, src/ops.cpp:404-424, and ops::mul, :76-83, of
 // LlamaBlock's SwiGLU, src/llama.cpp:55-58) and the pair of closures in one pass back.
+// gate, up (and dgate, dup) are [rows, cols] matrices with row pitch ld: ld == cols for separate
+// contiguous matrices, ld == 2*cols for the two halves of one [rows, 2*cols] projection.
 template <typename T>
-__global__ void ew_silu_mul_fwd(const T* gate, const T* up, T* y, int64_t n) {
+__global__ void ew_silu_mul_fwd(const T* gate, const T* up, T* y, int64_t n, int64_t cols, int64_t ld) {
     for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT) {
-        const float v = ldf(gate, i);
-        stf(y, i, (v / (1.0f + expf(-v))) * ldf(up, i));
+        const int64_t j = (i / cols) * ld + i % cols;
+        const float v = ldf(gate, j);
+        stf(y, i, (v / (1.0f + expf(-v))) * ldf(up, j));
     }
 }
 template <typename T>
-__global__ void ew_silu_mul_bwd(const T* gate, const T* up, const T* dy, T* dgate, T* dup, int64_t n) {
+__global__ void ew_silu_mul_bwd(const T* gate, const T* up, const T* dy, T* dgate, T* dup, int64_t n, int64_t cols,
+                                int64_t ld) {
     for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT) {
-        const float v = ldf(gate, i), g = ldf(dy, i);
+        const int64_t j = (i / cols) * ld + i % cols;
+        const float v = ldf(gate, j), g = ldf(dy, i);
         const float s = 1.0f / (1.0f + expf(-v));
-        stf(dup, i, g * (v * s));
-        stf(dgate, i, (g * ldf(up, i)) * (s * (1.0f + v * (1.0f - s))));
+        stf(dup, j, g * (v * s));
+        stf(dgate, j, (g * ldf(up, j)) * (s * (1.0f + v * (1.0f - s))));
     }
 }
 
@@ -248,6 +253,30 @@ __global__ void add_parts(const float* part, T* dst, int nparts, int64_t n, floa
         for (int p = 0; p < nparts; ++p) s += part[p * n + i];
         stf(dst, i, beta != 0.0f ? ldf(dst, i) + s : s);
     }
+}
+
+// The same sum, scattered: the [M, nsplit*N] result is cut into nsplit column blocks and block k
+// goes to its own contiguous [M, N] destination (the gradients of weights that were multiplied as
+// one concatenated matrix).
+struct SplitDst {
+    float* p[4];
+};
+__global__ void add_parts_split(const float* part, SplitDst dst, int nparts, int64_t M, int64_t N, int nsplit, float beta) {
+    const int64_t W = N * nsplit, n = M * W;
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT) {
+        float s = 0.0f;
+        for (int p = 0; p < nparts; ++p) s += part[p * n + i];
+        const int64_t r = i / W, c = i % W;
+        float* d = dst.p[c / N] + r * N + c % N;
+        *d = beta != 0.0f ? *d + s : s;
+    }
+}
+// dst[r][off + c] = src[r][c]: one column block of a concatenated matrix with row pitch ld
+template <typename TA, typename TY>
+__global__ void cast_cols_k(const TA* src, TY* dst, int64_t rows, int64_t cols, int64_t ld, int64_t off) {
+    const int64_t n = rows * cols;
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT)
+        stf(dst, (i / cols) * ld + off + i % cols, ldf(src, i));
 }
 
 // apply_rope (ops.cpp:497-509 forward, :519-533 backward = rotation by -theta).
@@ -469,6 +498,14 @@ void k_cast(const Tensor& src, const Tensor& dst) {
                                     static_cast<const TA*>(src.ptr()), 1.0f, static_cast<TY*>(dst.ptr()), src.numel())));
     post();
 }
+void k_cast_cols(const Tensor& src, const Tensor& dst, int64_t col_off) {
+    if (src.rows != dst.rows || col_off < 0 || col_off + src.cols > dst.cols) throw std::runtime_error("cast_cols: shape mismatch");
+    PK_DISPATCH1(TA, src.dtype, PK_DISPATCH1(TY, dst.dtype,
+                 hipLaunchKernelGGL((cast_cols_k<TA, TY>), ew_grid(src.numel()), dim3(NT), 0, tape_stream(),
+                                    static_cast<const TA*>(src.ptr()), static_cast<TY*>(dst.ptr()), src.rows, src.cols,
+                                    dst.cols, col_off)));
+    post();
+}
 template <int OP>
 static void binary(const Tensor& a, const Tensor& b, const Tensor& y, const char* who) {
     same_shape(a, b, who);
@@ -513,7 +550,7 @@ void k_silu_mul_fwd(const Tensor& gate, const Tensor& up, const Tensor& y) {
     same_shape(gate, y, "mul");
     PK_DISPATCH1(T, gate.dtype, hipLaunchKernelGGL((ew_silu_mul_fwd<T>), ew_grid(gate.numel()), dim3(NT), 0, tape_stream(),
                                                    static_cast<const T*>(gate.ptr()), static_cast<const T*>(up.ptr()),
-                                                   static_cast<T*>(y.ptr()), gate.numel()));
+                                                   static_cast<T*>(y.ptr()), gate.numel(), gate.cols, gate.cols));
     post();
 }
 void k_silu_mul_bwd(const Tensor& gate, const Tensor& up, const Tensor& dy, const Tensor& dgate, const Tensor& dup) {
@@ -525,7 +562,24 @@ void k_silu_mul_bwd(const Tensor& gate, const Tensor& up, const Tensor& dy, cons
                  hipLaunchKernelGGL((ew_silu_mul_bwd<T>), ew_grid(gate.numel()), dim3(NT), 0, tape_stream(),
                                     static_cast<const T*>(gate.ptr()), static_cast<const T*>(up.ptr()),
                                     static_cast<const T*>(dy.ptr()), static_cast<T*>(dgate.ptr()), static_cast<T*>(dup.ptr()),
-                                    gate.numel()));
+                                    gate.numel(), gate.cols, gate.cols));
+    post();
+}
+void k_silu_mul_cat_fwd(const Tensor& gu, const Tensor& y) {
+    if (gu.cols != 2 * y.cols || gu.rows != y.rows || gu.dtype != y.dtype) throw std::runtime_error("silu_mul: shape mismatch");
+    PK_DISPATCH1(T, gu.dtype, hipLaunchKernelGGL((ew_silu_mul_fwd<T>), ew_grid(y.numel()), dim3(NT), 0, tape_stream(),
+                                                 static_cast<const T*>(gu.ptr()), static_cast<const T*>(gu.ptr()) + y.cols,
+                                                 static_cast<T*>(y.ptr()), y.numel(), y.cols, gu.cols));
+    post();
+}
+void k_silu_mul_cat_bwd(const Tensor& gu, const Tensor& dy, const Tensor& dgu) {
+    if (gu.cols != 2 * dy.cols || gu.rows != dy.rows || gu.dtype != dy.dtype) throw std::runtime_error("silu_mul: shape mismatch");
+    same_shape(gu, dgu, "mul");
+    PK_DISPATCH1(T, gu.dtype,
+                 hipLaunchKernelGGL((ew_silu_mul_bwd<T>), ew_grid(dy.numel()), dim3(NT), 0, tape_stream(),
+                                    static_cast<const T*>(gu.ptr()), static_cast<const T*>(gu.ptr()) + dy.cols,
+                                    static_cast<const T*>(dy.ptr()), static_cast<T*>(dgu.ptr()),
+                                    static_cast<T*>(dgu.ptr()) + dy.cols, dy.numel(), dy.cols, gu.cols));
     post();
 }
 void k_rmsnorm_fwd(const Tensor& x, const Tensor& w, float eps, const Tensor& y, float* rinv) {
@@ -721,6 +775,37 @@ void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dty
         static_cast<rocblas_int>(ldc), rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
     if (st != rocblas_status_success)
         throw std::runtime_error(std::string("rocblas_gemm_ex failed: ") + rocblas_status_to_string(st));
+}
+
+void gemm_tn_split(const Tensor& A, const Tensor& B, float* const* dst, int nsplit, float beta) {
+    const int64_t K = A.rows, M = A.cols, W = B.cols;
+    if (B.rows != K) throw std::runtime_error("gemm: inner dimensions disagree");
+    if (nsplit < 1 || nsplit > 4 || W % nsplit != 0) throw std::runtime_error("gemm_tn_split: bad column split");
+    if (A.dtype != B.dtype) throw std::runtime_error("gemm: operand dtypes differ");
+    const rocblas_datatype ab = A.dtype == PK_F32 ? rocblas_datatype_f32_r : rocblas_datatype_bf16_r;
+    const float alpha = 1.0f, zero = 0.0f;
+    rocblas_set_stream(blas(), tape_stream());
+    // the contraction axis in slices, as in gemm(); short contractions run as one slice
+    int S = 1;
+    if (K >= 2048 && M * W <= (int64_t{1} << 21)) {
+        S = 8;
+        while (S > 1 && (K % S != 0 || K / S < 256)) S >>= 1;
+    }
+    const int64_t Ks = K / S;
+    Buffer part(sizeof(float) * static_cast<size_t>(S) * M * W);
+    const rocblas_status st = rocblas_gemm_strided_batched_ex(
+        blas(), rocblas_operation_none, rocblas_operation_transpose, static_cast<rocblas_int>(W),
+        static_cast<rocblas_int>(M), static_cast<rocblas_int>(Ks), &alpha, B.ptr(), ab, static_cast<rocblas_int>(W), Ks * W,
+        A.ptr(), ab, static_cast<rocblas_int>(M), Ks * M, &zero, part.p, rocblas_datatype_f32_r,
+        static_cast<rocblas_int>(W), M * W, part.p, rocblas_datatype_f32_r, static_cast<rocblas_int>(W), M * W, S,
+        rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
+    if (st != rocblas_status_success)
+        throw std::runtime_error(std::string("rocblas_gemm_strided_batched_ex failed: ") + rocblas_status_to_string(st));
+    SplitDst d{};
+    for (int k = 0; k < nsplit; ++k) d.p[k] = dst[k];
+    hipLaunchKernelGGL(add_parts_split, ew_grid(M * W), dim3(NT), 0, tape_stream(), static_cast<const float*>(part.p), d, S,
+                       M, W / nsplit, nsplit, beta);
+    post();
 }
 
 }  // namespace pk

@@ -161,7 +161,7 @@ struct Model {
         Var attn = ops::linear(ops::attention_qkv(qkv, cfg.n_heads, sc, seq_len, true, cfg.window, cfg.sinks), b.o);
         Var x1 = ops::add(x, attn);
         Var h2 = ops::rmsnorm(x1, b.ln2_w);
-        Var ffn = ops::linear(ops::silu_mul(ops::linear(h2, b.gate), ops::linear(h2, b.up)), b.down);
+        Var ffn = ops::linear(ops::silu_mul_cat(ops::linear_cat(h2, {b.gate, b.up})), b.down);
         return ops::add(x1, ffn);
     }
 
@@ -289,8 +289,7 @@ int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets
                 Var x = make_var(probe);
                 (void)ops::linear3(x, b.q, b.k, b.v);
                 (void)ops::linear(x, b.o);
-                (void)ops::linear(x, b.gate);
-                (void)ops::linear(x, b.up);
+                (void)ops::linear_cat(x, {b.gate, b.up});
                 Tensor pf = Tensor::make(1, m->cfg.d_ff, compute_dtype());
                 k_fill(pf, 0.0f);
                 (void)ops::linear(make_var(pf), b.down);

@@ -81,11 +81,13 @@ Var linear(const Var& x, const Var& W);
 // Three projections of the same input written side by side into one [N, 3*out]
 // matrix: the concat_cols({q, k, v}) of llama.cpp:30-36 without the copies.
 Var linear3(const Var& x, const Var& Wq, const Var& Wk, const Var& Wv);
+Var linear_cat(const Var& x, const std::vector<Var>& Ws);  // y = x [W_0 | W_1 | ...], equal widths, 1..4 weights
 Var add(const Var& a, const Var& b);                // ops.cpp:60-65
 Var mul(const Var& a, const Var& b);                // ops.cpp:76-83
 Var scale(const Var& x, float s);                   // ops.cpp:843-861
 Var silu(const Var& x);                             // ops.cpp:404-424
 Var silu_mul(const Var& gate, const Var& up);        // mul(silu(gate), up) as one node (llama.cpp:55-58)
+Var silu_mul_cat(const Var& gate_up);                // the same on the halves of one [N, 2*d_ff] projection [gate | up]
 Var rmsnorm(const Var& x, const Var& w);            // ops.cpp:426-479, eps fixed at 1e-5 (:435)
 // ops::apply_rope on the fused [N, 3d] matrix (ops.cpp:481-537). rot_heads = 1 is the
 // reference as written (only the first head of q and of k is rotated, :498-499 with the

@@ -32,6 +32,19 @@ const Tensor& shadow_of(const Var& W) {
     return it->second;
 }
 
+// [W_0 | W_1 | ...] in the compute dtype, keyed by the first weight; rebuilt after every optimizer step
+std::unordered_map<const Variable*, Tensor> g_shadow_cat;
+const Tensor& shadow_cat(const std::vector<Var>& Ws) {
+    auto it = g_shadow_cat.find(Ws[0].get());
+    if (it == g_shadow_cat.end()) {
+        const int64_t d = Ws[0]->data.cols;
+        Tensor t = Tensor::make(Ws[0]->data.rows, d * static_cast<int64_t>(Ws.size()), g_compute);
+        for (size_t k = 0; k < Ws.size(); ++k) k_cast_cols(Ws[k]->data, t, static_cast<int64_t>(k) * d);
+        it = g_shadow_cat.emplace(Ws[0].get(), std::move(t)).first;
+    }
+    return it->second;
+}
+
 // Post-order DFS over parents, iterative (autograd.cpp:31-45).
 void topo(const Var& root, std::vector<Variable*>& order) {
     std::unordered_set<Variable*> seen;
@@ -90,9 +103,13 @@ void set_compute_dtype(int dtype) {
     if (dtype != PK_F32 && dtype != PK_BF16) throw std::runtime_error("compute dtype must be PK_F32 or PK_BF16");
     g_compute = dtype;
     g_shadow.clear();
+    g_shadow_cat.clear();
 }
 int compute_dtype() { return g_compute; }
-void invalidate_shadows() { g_shadow.clear(); }
+void invalidate_shadows() {
+    g_shadow.clear();
+    g_shadow_cat.clear();
+}
 
 Tensor& Variable::ensure_grad() {
     if (grad.empty()) {
@@ -203,43 +220,49 @@ Var linear(const Var& x, const Var& W) {
     });
 }
 
-Var linear3(const Var& x, const Var& Wq, const Var& Wk, const Var& Wv) {
-    const int64_t N = x->data.rows, d = Wq->data.cols;
-    if (Wk->data.cols != d || Wv->data.cols != d || Wq->data.rows != x->data.cols || Wk->data.rows != x->data.cols ||
-        Wv->data.rows != x->data.cols)
-        throw std::runtime_error("matmul: inner dimensions disagree");
-    Tensor y = Tensor::make(N, 3 * d, x->data.dtype);
-    const size_t es = y.esize();
-    const Var Ws[3] = {Wq, Wk, Wv};
-    for (int i = 0; i < 3; ++i)
-        gemm(x->data, false, shadow_of(Ws[i]), false, static_cast<char*>(y.ptr()) + i * d * es, y.dtype, N, d, 3 * d, 0.0f);
-    return record(std::move(y), {x, Wq, Wk, Wv}, [d](Variable* self) {
+// y = x [W_0 | W_1 | ...]: several Linear layers that read the same input (q/k/v projections,
+// gate/up projections) as ONE GEMM against the column-wise concatenation of their weights, which
+// is kept as a compute-dtype copy like any other shadow. Backward is one GEMM for dX and one for
+// all the weight gradients, whose column blocks are scattered to the separate gradient tensors.
+Var linear_cat(const Var& x, const std::vector<Var>& Ws) {
+    if (Ws.empty() || Ws.size() > 4) throw std::runtime_error("linear_cat: 1 to 4 weights");
+    const int64_t N = x->data.rows, d = Ws[0]->data.cols;
+    for (const Var& W : Ws)
+        if (W->data.cols != d || W->data.rows != x->data.cols) throw std::runtime_error("matmul: inner dimensions disagree");
+    const int n = static_cast<int>(Ws.size());
+    Tensor y = Tensor::make(N, n * d, x->data.dtype);
+    gemm(x->data, false, shadow_cat(Ws), false, y.ptr(), y.dtype, N, n * d, n * d, 0.0f);
+    std::vector<Var> parents{x};
+    parents.insert(parents.end(), Ws.begin(), Ws.end());
+    return record(std::move(y), std::move(parents), [n](Variable* self) {
         const Var& x = self->parents[0];
-        const int64_t N = x->data.rows;
-        // the three column slices of dY, viewed as [N, d] matrices with row pitch 3d
-        Tensor dx;
-        if (x->requires_grad) dx = Tensor::make(N, x->data.cols, x->data.dtype);
-        for (int i = 0; i < 3; ++i) {
-            const Var& W = self->parents[1 + i];
-            Tensor slice = Tensor::make(N, d, self->grad.dtype);  // contiguous copy of the slice
-            {
-                // strided copy via GEMM-free path: cast kernel works on contiguous data only, so
-                // use a 2-D memcpy
-                const size_t es = slice.esize();
-                hip_check(hipMemcpy2DAsync(slice.ptr(), d * es, static_cast<const char*>(self->grad.ptr()) + i * d * es,
-                                           3 * d * es, d * es, N, hipMemcpyDeviceToDevice, tape_stream()),
-                          "hipMemcpy2DAsync");
-            }
-            if (x->requires_grad)
-                gemm(slice, false, shadow_of(W), true, dx.ptr(), dx.dtype, N, x->data.cols, x->data.cols, i == 0 ? 0.0f : 1.0f);
-            if (W->requires_grad) {
-                Tensor& g = W->ensure_grad();
-                gemm(x->data, true, slice, false, g.ptr(), g.dtype, g.rows, g.cols, g.cols, 1.0f);
-            }
+        const std::vector<Var> Ws(self->parents.begin() + 1, self->parents.end());
+        if (x->requires_grad) {  // dX = dY [W_0 | W_1 | ...]^T
+            Tensor dx = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
+            gemm(self->grad, false, shadow_cat(Ws), true, dx.ptr(), dx.dtype, dx.rows, dx.cols, dx.cols, 0.0f);
+            x->accumulate_owned(std::move(dx));
         }
-        if (x->requires_grad) x->accumulate_owned(std::move(dx));
+        bool any = false;
+        for (const Var& W : Ws) any = any || W->requires_grad;
+        if (any) {  // dW_k += X^T dY[:, block k]
+            float* dst[4] = {nullptr, nullptr, nullptr, nullptr};
+            std::vector<Tensor> unused;
+            for (int k = 0; k < n; ++k) {
+                if (Ws[k]->requires_grad) {
+                    Tensor& g = Ws[k]->ensure_grad();
+                    if (g.dtype != PK_F32) throw std::runtime_error("linear_cat: weight gradients must be fp32");
+                    dst[k] = static_cast<float*>(g.ptr());
+                } else {
+                    unused.push_back(Tensor::make(Ws[k]->data.rows, Ws[k]->data.cols, PK_F32));
+                    dst[k] = static_cast<float*>(unused.back().ptr());
+                }
+            }
+            gemm_tn_split(x->data, self->grad, dst, n, 1.0f);
+        }
     });
 }
+
+Var linear3(const Var& x, const Var& Wq, const Var& Wk, const Var& Wv) { return linear_cat(x, {Wq, Wk, Wv}); }
 
 Var add(const Var& a, const Var& b) {
     Tensor y = Tensor::make(a->data.rows, a->data.cols, a->data.dtype);
@@ -302,6 +325,19 @@ Var silu_mul(const Var& gate, const Var& up) {
         k_silu_mul_bwd(gate->data, up->data, self->grad, dg, du);
         if (gate->requires_grad) gate->accumulate_owned(std::move(dg));
         if (up->requires_grad) up->accumulate_owned(std::move(du));
+    });
+}
+
+Var silu_mul_cat(const Var& gu) {
+    if (gu->data.cols % 2 != 0) throw std::runtime_error("mul: shape mismatch");
+    Tensor y = Tensor::make(gu->data.rows, gu->data.cols / 2, gu->data.dtype);
+    k_silu_mul_cat_fwd(gu->data, y);
+    return record(std::move(y), {gu}, [](Variable* self) {
+        const Var& gu = self->parents[0];
+        if (!gu->requires_grad) return;
+        Tensor dgu = Tensor::make(gu->data.rows, gu->data.cols, gu->data.dtype);
+        k_silu_mul_cat_bwd(gu->data, self->grad, dgu);
+        gu->accumulate_owned(std::move(dgu));
     });
 }
 

@@ -88,6 +88,7 @@ void set_tape_stream(hipStream_t s);
 // All take row-major contiguous tensors; T = fp32 or bf16 storage, fp32 math.
 void k_fill(const Tensor& y, float v);
 void k_cast(const Tensor& src, const Tensor& dst);                      // dtype conversion / copy
+void k_cast_cols(const Tensor& src, const Tensor& dst, int64_t col_off);  // dst[:, off:off+src.cols] = src
 void k_add(const Tensor& a, const Tensor& b, const Tensor& y);          // y = a + b      (ops.cpp:60-65)
 void k_mul(const Tensor& a, const Tensor& b, const Tensor& y);          // y = a .* b     (ops.cpp:76-83)
 void k_scale(const Tensor& a, float s, const Tensor& y);                // y = a * s
@@ -96,6 +97,9 @@ void k_silu_fwd(const Tensor& x, const Tensor& y);                      // ops.c
 void k_silu_bwd(const Tensor& x, const Tensor& dy, const Tensor& dx);   // ops.cpp:412-423
 void k_silu_mul_fwd(const Tensor& gate, const Tensor& up, const Tensor& y);  // silu(gate) .* up, llama.cpp:55-58
 void k_silu_mul_bwd(const Tensor& gate, const Tensor& up, const Tensor& dy, const Tensor& dgate, const Tensor& dup);
+// the same on the two halves of one [rows, 2*cols] matrix [gate | up]
+void k_silu_mul_cat_fwd(const Tensor& gu, const Tensor& y);
+void k_silu_mul_cat_bwd(const Tensor& gu, const Tensor& dy, const Tensor& dgu);
 void k_rmsnorm_fwd(const Tensor& x, const Tensor& w, float eps, const Tensor& y, float* rinv);  // ops.cpp:437-445
 void k_rmsnorm_bwd(const Tensor& dy, const Tensor& x, const float* rinv, const Tensor& w, const Tensor* dw_f32,
                    const Tensor* dx);                                   // ops.cpp:447-478
@@ -128,5 +132,7 @@ void k_adamw(const Tensor& p, const Tensor& g, const Tensor& m, const Tensor& v,
 // matrix (ldc). beta is 0 or 1.
 void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dtype, int64_t M, int64_t N, int64_t ldc,
           float beta);
+// dst[k] ([A.cols, B.cols/nsplit] fp32, contiguous) = beta * dst[k] + A^T B[:, k-th column block], k < nsplit <= 4
+void gemm_tn_split(const Tensor& A, const Tensor& B, float* const* dst, int nsplit, float beta);
 
 }  // namespace pk
