@@ -145,6 +145,90 @@ __global__ void ew_fill(TY* y, float v, int64_t n) {
     for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT)
         stf(y, i, v);
 }
+// ---- 8-wide bf16 forms -------------------------------------------------------
+// The streaming kernels of the bf16 compute path move 16 bytes per lane and instruction when the
+// element count (and any row pitch) is a multiple of 8 and the pointers are 16-byte aligned; the
+// one-element kernels above and below remain for everything else. Same arithmetic, same rounding
+// (nearest even; v_cvt_pk_bf16_f32 here, the integer form in stf).
+struct F8 {
+    float v[8];
+};
+__device__ inline F8 ld8(const uint16_t* p, int64_t e) {
+    const u32x4 r = *reinterpret_cast<const u32x4*>(p + e);
+    F8 o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        o.v[2 * k] = __uint_as_float(r[k] << 16);
+        o.v[2 * k + 1] = __uint_as_float(r[k] & 0xFFFF0000u);
+    }
+    return o;
+}
+__device__ inline F8 ld8(const float* p, int64_t e) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p + e), b = *reinterpret_cast<const f32x4*>(p + e + 4);
+    return F8{{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]}};
+}
+__device__ inline void st8(uint16_t* p, int64_t e, const F8& x) {
+    const u32x4 r = {pack_bf16(x.v[0], x.v[1]), pack_bf16(x.v[2], x.v[3]), pack_bf16(x.v[4], x.v[5]), pack_bf16(x.v[6], x.v[7])};
+    *reinterpret_cast<u32x4*>(p + e) = r;
+}
+#define PK_EW8_LOOP(i, n8) \
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < (n8); i += static_cast<int64_t>(gridDim.x) * NT)
+template <int OP>
+__global__ void ew_binary8(const uint16_t* a, const uint16_t* b, uint16_t* y, int64_t n8) {
+    PK_EW8_LOOP(i, n8) {
+        const F8 x = ld8(a, i * 8), z = ld8(b, i * 8);
+        F8 o;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) o.v[k] = OP == 0 ? x.v[k] + z.v[k] : x.v[k] * z.v[k];
+        st8(y, i * 8, o);
+    }
+}
+__global__ void ew_scale8(const uint16_t* a, float s, uint16_t* y, int64_t n8) {
+    PK_EW8_LOOP(i, n8) {
+        F8 x = ld8(a, i * 8);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) x.v[k] *= s;
+        st8(y, i * 8, x);
+    }
+}
+__global__ void ew_axpy8(uint16_t* y, float a, const uint16_t* x, int64_t n8) {
+    PK_EW8_LOOP(i, n8) {
+        F8 o = ld8(y, i * 8);
+        const F8 z = ld8(x, i * 8);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) o.v[k] = o.v[k] + a * z.v[k];
+        st8(y, i * 8, o);
+    }
+}
+// cols8, ld8: row length and row pitch of gate / up (and dgate / dup) in units of 8 elements
+__global__ void ew_silu_mul_fwd8(const uint16_t* gate, const uint16_t* up, uint16_t* y, int64_t n8, int64_t cols8, int64_t ld8_) {
+    PK_EW8_LOOP(i, n8) {
+        const int64_t j = ((i / cols8) * ld8_ + i % cols8) * 8;
+        const F8 g = ld8(gate, j), u = ld8(up, j);
+        F8 o;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) o.v[k] = (g.v[k] / (1.0f + expf(-g.v[k]))) * u.v[k];
+        st8(y, i * 8, o);
+    }
+}
+__global__ void ew_silu_mul_bwd8(const uint16_t* gate, const uint16_t* up, const uint16_t* dy, uint16_t* dgate, uint16_t* dup,
+                                 int64_t n8, int64_t cols8, int64_t ld8_) {
+    PK_EW8_LOOP(i, n8) {
+        const int64_t j = ((i / cols8) * ld8_ + i % cols8) * 8;
+        const F8 v = ld8(gate, j), u = ld8(up, j), g = ld8(dy, i * 8);
+        F8 du, dg;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float sg = 1.0f / (1.0f + expf(-v.v[k]));
+            du.v[k] = g.v[k] * (v.v[k] * sg);
+            dg.v[k] = (g.v[k] * u.v[k]) * (sg * (1.0f + v.v[k] * (1.0f - sg)));
+        }
+        st8(dup, j, du);
+        st8(dgate, j, dg);
+    }
+}
+inline bool aligned16p(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
 template <typename T>
 __global__ void ew_silu_fwd(const T* x, T* y, int64_t n) {
     for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT) {
@@ -222,6 +306,53 @@ __global__ void rms_bwd_dx(const T* dy, const T* x, const float* rinv, const flo
     const float ri = rinv[row], k = ri * ri * term / static_cast<float>(C);
     for (int j = lane; j < C; j += 64) stf(dx + row * C, j, ri * (ldf(gr, j) * w[j] - ldf(xr, j) * k));
 }
+// 8-wide bf16 forms of the two row kernels above (C a multiple of 8): one 16-byte load per lane
+// covers a 512-column row in a single step.
+__global__ void rms_fwd8(const uint16_t* x, const float* w, float eps, uint16_t* y, float* rinv, int64_t R, int C) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= R) return;
+    const uint16_t* xr = x + row * C;
+    float ss = 0.0f;
+    for (int j = lane * 8; j < C; j += 512) {
+        const F8 v = ld8(xr, j);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) ss = fmaf(v.v[k], v.v[k], ss);
+    }
+    ss = wave_sum(ss) / static_cast<float>(C);
+    const float ri = 1.0f / sqrtf(ss + eps);
+    if (lane == 0) rinv[row] = ri;
+    for (int j = lane * 8; j < C; j += 512) {
+        F8 v = ld8(xr, j);
+        const F8 g = ld8(w, j);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v.v[k] = v.v[k] * ri * g.v[k];
+        st8(y + row * C, j, v);
+    }
+}
+__global__ void rms_bwd_dx8(const uint16_t* dy, const uint16_t* x, const float* rinv, const float* w, uint16_t* dx, int64_t R,
+                            int C) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= R) return;
+    const uint16_t* xr = x + row * C;
+    const uint16_t* gr = dy + row * C;
+    float term = 0.0f;
+    for (int j = lane * 8; j < C; j += 512) {
+        const F8 g = ld8(gr, j), v = ld8(xr, j), ww = ld8(w, j);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) term = fmaf(g.v[k] * ww.v[k], v.v[k], term);
+    }
+    term = wave_sum(term);
+    const float ri = rinv[row], kk = ri * ri * term / static_cast<float>(C);
+    for (int j = lane * 8; j < C; j += 512) {
+        const F8 g = ld8(gr, j), v = ld8(xr, j), ww = ld8(w, j);
+        F8 o;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) o.v[k] = ri * (g.v[k] * ww.v[k] - v.v[k] * kk);
+        st8(dx + row * C, j, o);
+    }
+}
 // dw_j = sum_i dY_ij x_ij rinv_i, in two deterministic stages: each block sums
 // ROWS_PB rows into part[block][C], then one block per column chunk adds the parts.
 constexpr int ROWS_PB = 32;  // 8192 rows -> 256 blocks, one per CU
@@ -234,16 +365,43 @@ __global__ void rms_bwd_dw_part(const T* dy, const T* x, const float* rinv, floa
         part[static_cast<int64_t>(blockIdx.x) * C + j] = s;
     }
 }
+// 8-wide bf16 form: C/8 threads cover a row, the block's NT / (C/8) row groups meet in LDS in a fixed order.
+// Needs C % 8 == 0 and C/8 a divisor of NT.
+__global__ void rms_bwd_dw_part8(const uint16_t* dy, const uint16_t* x, const float* rinv, float* part, int64_t R, int C) {
+    extern __shared__ float sh_dw[];  // [NT / (C/8)][C]
+    const int c8 = C / 8, col = (threadIdx.x % c8) * 8, rg = threadIdx.x / c8, nrg = NT / c8;
+    const int64_t r0 = static_cast<int64_t>(blockIdx.x) * ROWS_PB, r1 = min(r0 + ROWS_PB, R);
+    F8 acc{};
+    for (int64_t i = r0 + rg; i < r1; i += nrg) {
+        const F8 g = ld8(dy, i * C + col), v = ld8(x, i * C + col);
+        const float ri = rinv[i];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) acc.v[k] = fmaf(g.v[k] * v.v[k], ri, acc.v[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) sh_dw[rg * C + col + k] = acc.v[k];
+    __syncthreads();
+    for (int j = threadIdx.x; j < C; j += NT) {
+        float t = 0.0f;
+        for (int q = 0; q < nrg; ++q) t += sh_dw[q * C + j];
+        part[static_cast<int64_t>(blockIdx.x) * C + j] = t;
+    }
+}
 __global__ void colsum_parts(const float* part, float* dw, int nparts, int C) {
-    // 64 columns x 4 groups of parts per block; the groups meet in a fixed order
-    __shared__ float sh[4][64];
+    // 64 columns x 16 groups of parts per block (1024 threads: each walks a sixteenth of the
+    // parts, the walk being a chain of dependent loads); the groups meet in a fixed order
+    __shared__ float sh[16][64];
     const int col = blockIdx.x * 64 + (threadIdx.x & 63), grp = threadIdx.x >> 6;
     float s = 0.0f;
     if (col < C)
-        for (int p = grp; p < nparts; p += 4) s += part[static_cast<int64_t>(p) * C + col];
+        for (int p = grp; p < nparts; p += 16) s += part[static_cast<int64_t>(p) * C + col];
     sh[grp][threadIdx.x & 63] = s;
     __syncthreads();
-    if (grp == 0 && col < C) dw[col] += (sh[0][threadIdx.x] + sh[1][threadIdx.x]) + (sh[2][threadIdx.x] + sh[3][threadIdx.x]);
+    if (grp == 0 && col < C) {
+        float t = 0.0f;
+        for (int q = 0; q < 16; ++q) t += sh[q][threadIdx.x];
+        dw[col] += t;
+    }
 }
 // dst[i] = beta * dst[i] + sum_s part[s][i], parts added in index order
 template <typename T>
@@ -510,6 +668,14 @@ template <int OP>
 static void binary(const Tensor& a, const Tensor& b, const Tensor& y, const char* who) {
     same_shape(a, b, who);
     same_shape(a, y, who);
+    if (a.dtype == PK_BF16 && b.dtype == PK_BF16 && y.dtype == PK_BF16 && a.numel() % 8 == 0 && aligned16p(a.ptr()) &&
+        aligned16p(b.ptr()) && aligned16p(y.ptr())) {
+        hipLaunchKernelGGL((ew_binary8<OP>), ew_grid(a.numel() / 8), dim3(NT), 0, tape_stream(),
+                           static_cast<const uint16_t*>(a.ptr()), static_cast<const uint16_t*>(b.ptr()),
+                           static_cast<uint16_t*>(y.ptr()), a.numel() / 8);
+        post();
+        return;
+    }
     PK_DISPATCH1(TA, a.dtype, PK_DISPATCH1(TB, b.dtype, PK_DISPATCH1(TY, y.dtype,
                  hipLaunchKernelGGL((ew_binary<TA, TB, TY, OP>), ew_grid(a.numel()), dim3(NT), 0, tape_stream(),
                                     static_cast<const TA*>(a.ptr()), static_cast<const TB*>(b.ptr()),
@@ -520,6 +686,12 @@ void k_add(const Tensor& a, const Tensor& b, const Tensor& y) { binary<0>(a, b, 
 void k_mul(const Tensor& a, const Tensor& b, const Tensor& y) { binary<1>(a, b, y, "mul"); }
 void k_scale(const Tensor& a, float s, const Tensor& y) {
     same_shape(a, y, "scale");
+    if (a.dtype == PK_BF16 && y.dtype == PK_BF16 && a.numel() % 8 == 0 && aligned16p(a.ptr()) && aligned16p(y.ptr())) {
+        hipLaunchKernelGGL(ew_scale8, ew_grid(a.numel() / 8), dim3(NT), 0, tape_stream(), static_cast<const uint16_t*>(a.ptr()),
+                           s, static_cast<uint16_t*>(y.ptr()), a.numel() / 8);
+        post();
+        return;
+    }
     PK_DISPATCH1(TA, a.dtype, PK_DISPATCH1(TY, y.dtype,
                  hipLaunchKernelGGL((ew_scale<TA, TY>), ew_grid(a.numel()), dim3(NT), 0, tape_stream(),
                                     static_cast<const TA*>(a.ptr()), s, static_cast<TY*>(y.ptr()), a.numel())));
@@ -527,6 +699,12 @@ void k_scale(const Tensor& a, float s, const Tensor& y) {
 }
 void k_axpy(const Tensor& y, float a, const Tensor& x) {
     if (x.rows != y.rows || x.cols != y.cols) throw std::runtime_error("accumulate: gradient shape mismatch");  // autograd.cpp:20-22
+    if (x.dtype == PK_BF16 && y.dtype == PK_BF16 && y.numel() % 8 == 0 && aligned16p(x.ptr()) && aligned16p(y.ptr())) {
+        hipLaunchKernelGGL(ew_axpy8, ew_grid(y.numel() / 8), dim3(NT), 0, tape_stream(), static_cast<uint16_t*>(y.ptr()), a,
+                           static_cast<const uint16_t*>(x.ptr()), y.numel() / 8);
+        post();
+        return;
+    }
     PK_DISPATCH1(TY, y.dtype, PK_DISPATCH1(TX, x.dtype,
                  hipLaunchKernelGGL((ew_axpy<TY, TX>), ew_grid(y.numel()), dim3(NT), 0, tape_stream(),
                                     static_cast<TY*>(y.ptr()), a, static_cast<const TX*>(x.ptr()), y.numel())));
@@ -545,45 +723,70 @@ void k_silu_bwd(const Tensor& x, const Tensor& dy, const Tensor& dx) {
                                                 static_cast<T*>(dx.ptr()), x.numel()));
     post();
 }
+namespace {
+// gate, up: [rows, cols] with row pitch ld; y, dy contiguous; dgate, dup with pitch ld
+void silu_mul_fwd_launch(const void* gate, const void* up, void* y, int dtype, int64_t rows, int64_t cols, int64_t ld) {
+    const int64_t n = rows * cols;
+    if (dtype == PK_BF16 && cols % 8 == 0 && ld % 8 == 0 && aligned16p(gate) && aligned16p(up) && aligned16p(y)) {
+        hipLaunchKernelGGL(ew_silu_mul_fwd8, ew_grid(n / 8), dim3(NT), 0, tape_stream(), static_cast<const uint16_t*>(gate),
+                           static_cast<const uint16_t*>(up), static_cast<uint16_t*>(y), n / 8, cols / 8, ld / 8);
+    } else {
+        PK_DISPATCH1(T, dtype, hipLaunchKernelGGL((ew_silu_mul_fwd<T>), ew_grid(n), dim3(NT), 0, tape_stream(),
+                                                  static_cast<const T*>(gate), static_cast<const T*>(up),
+                                                  static_cast<T*>(y), n, cols, ld));
+    }
+    post();
+}
+void silu_mul_bwd_launch(const void* gate, const void* up, const void* dy, void* dgate, void* dup, int dtype, int64_t rows,
+                         int64_t cols, int64_t ld) {
+    const int64_t n = rows * cols;
+    if (dtype == PK_BF16 && cols % 8 == 0 && ld % 8 == 0 && aligned16p(gate) && aligned16p(up) && aligned16p(dy) &&
+        aligned16p(dgate) && aligned16p(dup)) {
+        hipLaunchKernelGGL(ew_silu_mul_bwd8, ew_grid(n / 8), dim3(NT), 0, tape_stream(), static_cast<const uint16_t*>(gate),
+                           static_cast<const uint16_t*>(up), static_cast<const uint16_t*>(dy), static_cast<uint16_t*>(dgate),
+                           static_cast<uint16_t*>(dup), n / 8, cols / 8, ld / 8);
+    } else {
+        PK_DISPATCH1(T, dtype, hipLaunchKernelGGL((ew_silu_mul_bwd<T>), ew_grid(n), dim3(NT), 0, tape_stream(),
+                                                  static_cast<const T*>(gate), static_cast<const T*>(up),
+                                                  static_cast<const T*>(dy), static_cast<T*>(dgate), static_cast<T*>(dup), n,
+                                                  cols, ld));
+    }
+    post();
+}
+}  // namespace
 void k_silu_mul_fwd(const Tensor& gate, const Tensor& up, const Tensor& y) {
     same_shape(gate, up, "mul");
     same_shape(gate, y, "mul");
-    PK_DISPATCH1(T, gate.dtype, hipLaunchKernelGGL((ew_silu_mul_fwd<T>), ew_grid(gate.numel()), dim3(NT), 0, tape_stream(),
-                                                   static_cast<const T*>(gate.ptr()), static_cast<const T*>(up.ptr()),
-                                                   static_cast<T*>(y.ptr()), gate.numel(), gate.cols, gate.cols));
-    post();
+    silu_mul_fwd_launch(gate.ptr(), up.ptr(), y.ptr(), gate.dtype, gate.rows, gate.cols, gate.cols);
 }
 void k_silu_mul_bwd(const Tensor& gate, const Tensor& up, const Tensor& dy, const Tensor& dgate, const Tensor& dup) {
     same_shape(gate, up, "mul");
     same_shape(gate, dy, "mul");
     same_shape(gate, dgate, "mul");
     same_shape(gate, dup, "mul");
-    PK_DISPATCH1(T, gate.dtype,
-                 hipLaunchKernelGGL((ew_silu_mul_bwd<T>), ew_grid(gate.numel()), dim3(NT), 0, tape_stream(),
-                                    static_cast<const T*>(gate.ptr()), static_cast<const T*>(up.ptr()),
-                                    static_cast<const T*>(dy.ptr()), static_cast<T*>(dgate.ptr()), static_cast<T*>(dup.ptr()),
-                                    gate.numel(), gate.cols, gate.cols));
-    post();
+    silu_mul_bwd_launch(gate.ptr(), up.ptr(), dy.ptr(), dgate.ptr(), dup.ptr(), gate.dtype, gate.rows, gate.cols, gate.cols);
 }
 void k_silu_mul_cat_fwd(const Tensor& gu, const Tensor& y) {
     if (gu.cols != 2 * y.cols || gu.rows != y.rows || gu.dtype != y.dtype) throw std::runtime_error("silu_mul: shape mismatch");
-    PK_DISPATCH1(T, gu.dtype, hipLaunchKernelGGL((ew_silu_mul_fwd<T>), ew_grid(y.numel()), dim3(NT), 0, tape_stream(),
-                                                 static_cast<const T*>(gu.ptr()), static_cast<const T*>(gu.ptr()) + y.cols,
-                                                 static_cast<T*>(y.ptr()), y.numel(), y.cols, gu.cols));
-    post();
+    const char* g = static_cast<const char*>(gu.ptr());
+    silu_mul_fwd_launch(g, g + y.cols * gu.esize(), y.ptr(), gu.dtype, y.rows, y.cols, gu.cols);
 }
 void k_silu_mul_cat_bwd(const Tensor& gu, const Tensor& dy, const Tensor& dgu) {
     if (gu.cols != 2 * dy.cols || gu.rows != dy.rows || gu.dtype != dy.dtype) throw std::runtime_error("silu_mul: shape mismatch");
     same_shape(gu, dgu, "mul");
-    PK_DISPATCH1(T, gu.dtype,
-                 hipLaunchKernelGGL((ew_silu_mul_bwd<T>), ew_grid(dy.numel()), dim3(NT), 0, tape_stream(),
-                                    static_cast<const T*>(gu.ptr()), static_cast<const T*>(gu.ptr()) + dy.cols,
-                                    static_cast<const T*>(dy.ptr()), static_cast<T*>(dgu.ptr()),
-                                    static_cast<T*>(dgu.ptr()) + dy.cols, dy.numel(), dy.cols, gu.cols));
-    post();
+    const char* g = static_cast<const char*>(gu.ptr());
+    char* d = static_cast<char*>(dgu.ptr());
+    silu_mul_bwd_launch(g, g + dy.cols * gu.esize(), dy.ptr(), d, d + dy.cols * gu.esize(), gu.dtype, dy.rows, dy.cols, gu.cols);
 }
 void k_rmsnorm_fwd(const Tensor& x, const Tensor& w, float eps, const Tensor& y, float* rinv) {
     if (w.rows != 1 || w.cols != x.cols || w.dtype != PK_F32) throw std::runtime_error("rmsnorm: w must be [1, cols(x)]");
+    if (x.dtype == PK_BF16 && x.cols % 8 == 0 && aligned16p(x.ptr()) && aligned16p(y.ptr()) && aligned16p(w.ptr())) {
+        hipLaunchKernelGGL(rms_fwd8, dim3((x.rows + 3) / 4), dim3(NT), 0, tape_stream(), static_cast<const uint16_t*>(x.ptr()),
+                           static_cast<const float*>(w.ptr()), eps, static_cast<uint16_t*>(y.ptr()), rinv, x.rows,
+                           static_cast<int>(x.cols));
+        post();
+        return;
+    }
     PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((rms_fwd<T>), dim3((x.rows + 3) / 4), dim3(NT), 0, tape_stream(),
                                                 static_cast<const T*>(x.ptr()), static_cast<const float*>(w.ptr()), eps,
                                                 static_cast<T*>(y.ptr()), rinv, x.rows, static_cast<int>(x.cols)));
@@ -593,20 +796,33 @@ void k_rmsnorm_bwd(const Tensor& dy, const Tensor& x, const float* rinv, const T
                    const Tensor* dx) {
     const int C = static_cast<int>(x.cols);
     if (dx) {
-        PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((rms_bwd_dx<T>), dim3((x.rows + 3) / 4), dim3(NT), 0, tape_stream(),
-                                                    static_cast<const T*>(dy.ptr()), static_cast<const T*>(x.ptr()), rinv,
-                                                    static_cast<const float*>(w.ptr()), static_cast<T*>(dx->ptr()),
-                                                    x.rows, C));
+        if (x.dtype == PK_BF16 && C % 8 == 0 && aligned16p(x.ptr()) && aligned16p(dy.ptr()) && aligned16p(dx->ptr()) &&
+            aligned16p(w.ptr())) {
+            hipLaunchKernelGGL(rms_bwd_dx8, dim3((x.rows + 3) / 4), dim3(NT), 0, tape_stream(),
+                               static_cast<const uint16_t*>(dy.ptr()), static_cast<const uint16_t*>(x.ptr()), rinv,
+                               static_cast<const float*>(w.ptr()), static_cast<uint16_t*>(dx->ptr()), x.rows, C);
+        } else {
+            PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((rms_bwd_dx<T>), dim3((x.rows + 3) / 4), dim3(NT), 0, tape_stream(),
+                                                        static_cast<const T*>(dy.ptr()), static_cast<const T*>(x.ptr()), rinv,
+                                                        static_cast<const float*>(w.ptr()), static_cast<T*>(dx->ptr()),
+                                                        x.rows, C));
+        }
         post();
     }
     if (dw) {
         const int nparts = static_cast<int>((x.rows + ROWS_PB - 1) / ROWS_PB);
         Buffer part(sizeof(float) * static_cast<size_t>(nparts) * C);
-        PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((rms_bwd_dw_part<T>), dim3(nparts), dim3(NT), 0, tape_stream(),
-                                                    static_cast<const T*>(dy.ptr()), static_cast<const T*>(x.ptr()), rinv,
-                                                    static_cast<float*>(part.p), x.rows, C));
+        if (x.dtype == PK_BF16 && C % 8 == 0 && NT % (C / 8) == 0 && aligned16p(x.ptr()) && aligned16p(dy.ptr())) {
+            hipLaunchKernelGGL(rms_bwd_dw_part8, dim3(nparts), dim3(NT), sizeof(float) * (NT / (C / 8)) * C, tape_stream(),
+                               static_cast<const uint16_t*>(dy.ptr()), static_cast<const uint16_t*>(x.ptr()), rinv,
+                               static_cast<float*>(part.p), x.rows, C);
+        } else {
+            PK_DISPATCH1(T, x.dtype, hipLaunchKernelGGL((rms_bwd_dw_part<T>), dim3(nparts), dim3(NT), 0, tape_stream(),
+                                                        static_cast<const T*>(dy.ptr()), static_cast<const T*>(x.ptr()), rinv,
+                                                        static_cast<float*>(part.p), x.rows, C));
+        }
         post();
-        hipLaunchKernelGGL(colsum_parts, dim3((C + 63) / 64), dim3(NT), 0, tape_stream(),
+        hipLaunchKernelGGL(colsum_parts, dim3((C + 63) / 64), dim3(1024), 0, tape_stream(),
                            static_cast<const float*>(part.p), static_cast<float*>(dw->ptr()), nparts, C);
         post();
     }

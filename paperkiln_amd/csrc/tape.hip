@@ -191,9 +191,9 @@ Var checkpoint(const std::function<Var(const Var&)>& fn, const Var& x) {
         Var y2 = fn_copy(x2);
         if (y2->data.rows != self->grad.rows || y2->data.cols != self->grad.cols)
             throw std::runtime_error("checkpoint: recomputed output shape mismatch");
-        y2->accumulate(self->grad);
+        y2->accumulate_owned(std::move(self->grad));  // this node's gradient has no other reader
         run_backward(y2);  // parameters inside fn are the model's own, their grads land in place
-        if (xin->requires_grad && !x2->grad.empty()) xin->accumulate(x2->grad);
+        if (xin->requires_grad && !x2->grad.empty()) xin->accumulate_owned(std::move(x2->grad));
     };
     return out;
 }
@@ -268,8 +268,9 @@ Var add(const Var& a, const Var& b) {
     Tensor y = Tensor::make(a->data.rows, a->data.cols, a->data.dtype);
     k_add(a->data, b->data, y);
     return record(std::move(y), {a, b}, [](Variable* self) {
+        // one parent gets a copy (or an axpy), the other takes the tensor itself
         if (self->parents[0]->requires_grad) self->parents[0]->accumulate(self->grad);
-        if (self->parents[1]->requires_grad) self->parents[1]->accumulate(self->grad);
+        if (self->parents[1]->requires_grad) self->parents[1]->accumulate_owned(std::move(self->grad));
     });
 }
 
