@@ -127,7 +127,7 @@ __global__ __launch_bounds__(256, 2) void mfma_dq(AttnArgs a) {
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = lane >> 5, c32 = lane & 31;
     const int nqb = (a.T + BM - 1) / BM, rep = a.Hq / a.Hkv;
-    const bool paired = a.causal && a.window == 0;  // as in the forward kernel
+    const bool paired = pair_causal_blocks(nqb, a.Hq * a.B, a.causal, a.window);
     int blk, rr, kvu;
     if (!xcd_map(paired ? (nqb + 1) / 2 : nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv, h = hk * rep + rr;
@@ -259,7 +259,7 @@ int launch(const AttnArgs& a, int stages, hipStream_t st) {
     const int64_t rows = static_cast<int64_t>(a.B) * a.Hq * a.T;
     constexpr int RPB = 256 / (D / 8);
     const int nb128 = (a.T + 127) / 128;
-    const bool paired = a.causal && a.window == 0;
+    const bool paired = pair_causal_blocks(nb128, a.Hq * a.B, a.causal, a.window);
     const dim3 dq_grid(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, a.Hq / a.Hkv, a.Hkv * a.B));
     // delta and dQ asked for together: dQ forms delta itself and runs first, dK/dV reads what it wrote
     const bool fused = (stages & PK_BWD_DELTA) && (stages & PK_BWD_DQ);

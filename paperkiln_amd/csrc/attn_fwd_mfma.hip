@@ -94,7 +94,7 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
     // workgroup takes blocks i and nqb-1-i back to back: every workgroup then
     // carries the same number of key tiles and the last wave of workgroups
     // does not idle three quarters of the chip.
-    const bool paired = a.causal && a.window == 0;
+    const bool paired = pair_causal_blocks(nqb, a.Hq * a.B, a.causal, a.window);
     int blk, rr, kvu;
     if (!xcd_map(paired ? (nqb + 1) / 2 : nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv, h = hk * rep + rr;
@@ -267,7 +267,7 @@ template <int D, int NQ, int OCC>
 int launch(const AttnArgs& a, hipStream_t st) {
     constexpr int BM = 128 * NQ;
     const int nqb = (a.T + BM - 1) / BM;
-    const bool paired = a.causal && a.window == 0;
+    const bool paired = pair_causal_blocks(nqb, a.Hq * a.B, a.causal, a.window);
     dim3 grid(xcd_grid(paired ? (nqb + 1) / 2 : nqb, a.Hq / a.Hkv, a.Hkv * a.B));
     hipLaunchKernelGGL((mfma_fwd<D, NQ, OCC>), grid, dim3(256), 0, st, a);
     PK_HIP(hipGetLastError());
