@@ -9,8 +9,9 @@
 //   dV = P^T dO          dP = dO V^T      dS = P .* (dP - delta)
 //   dQ = scale * dS K    dK = scale * dS^T Q
 //
-// Three launches, no atomics, deterministic:
-//   mfma_delta    one pass over O and dO.
+// No atomics, deterministic. The full backward is two launches, mfma_dq (which
+// also forms delta) then mfma_dkdv2; asked for by parts it is three:
+//   mfma_delta    one pass over O and dO (only when delta is wanted without dQ).
 //   mfma_dkdv2    (attn_bwd_dkdv2.hip) a workgroup owns 128 keys of one KV
 //                 head and loops over the query heads of its GQA group and
 //                 over the query tiles that can see it.
