@@ -142,3 +142,38 @@ def swa_attention(q, k, v, scale, window, sinks, seq_len=0):
 def attention(q, k, v, scale, causal=True, window=0, sinks=0):
     """All heads at once on [B,T,H,dk] tensors (GQA when k/v have fewer heads). Differentiable."""
     return _AttnFn.apply(q, k, v, scale, causal, window, sinks)
+
+
+class _CheckpointFn(torch.autograd.Function):
+    """checkpoint(fn, x) of the reference (src/autograd.cpp:68-102): the forward runs fn with the
+    tape off and keeps only its input and output; the backward re-runs fn on a detached copy of the
+    input with the tape on, seeds the recomputed output with the incoming gradient and runs the inner
+    tape, so parameters used inside fn receive their gradients in place and x receives the inner
+    input's gradient."""
+
+    @staticmethod
+    def forward(ctx, fn, x):
+        ctx.fn = fn
+        ctx.save_for_backward(x)
+        with torch.no_grad():
+            return fn(x)
+
+    @staticmethod
+    def backward(ctx, dy):
+        (x,) = ctx.saved_tensors
+        x2 = x.detach().requires_grad_(True)
+        with torch.enable_grad():
+            y2 = ctx.fn(x2)
+        if y2.shape != dy.shape:
+            raise RuntimeError("checkpoint: recomputed output shape mismatch")
+        torch.autograd.backward(y2, dy)
+        return None, x2.grad
+
+
+def checkpoint(fn, x):
+    """y = fn(x) without keeping fn's intermediate activations; they are rebuilt in the backward.
+    As in the reference, the node is only recorded when x requires a gradient (the closure hangs
+    off x, src/autograd.cpp:80-83); with the tape off it is a plain call."""
+    if not torch.is_grad_enabled() or not x.requires_grad:
+        return fn(x)
+    return _CheckpointFn.apply(fn, x)

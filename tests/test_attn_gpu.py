@@ -141,6 +141,47 @@ def test_backward_by_parts_equals_one_call(dtype, window, sinks):
         assert err <= 4 * ulp * ref, name
 
 
+def test_python_checkpoint_matches_plain():
+    """ops.checkpoint around a block that contains the attention node: loss, input gradient and the
+    gradients of parameters used inside the block equal the plain run bit for bit (same kernels, same
+    order), and the block's intermediates are not kept between forward and backward."""
+    B, T, H, dk = 2, 256, 4, 64
+    d = H * dk
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    x0 = torch.randn((B * T, d), generator=gen, device="cuda")
+    wq, wk, wv = (torch.randn((d, d), generator=gen, device="cuda") * 0.05 for _ in range(3))
+    scale = float(1 / np.sqrt(dk))
+
+    def run(use_ckpt):
+        x = x0.clone().requires_grad_(True)
+        ws = [w.clone().requires_grad_(True) for w in (wq, wk, wv)]
+
+        def block(h):
+            q, k, v = ((h @ w).bfloat16().view(B, T, H, dk) for w in ws)
+            return h + ops.attention(q, k, v, scale).float().view(B * T, d)
+
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        h = x
+        for _ in range(3):
+            h = ops.checkpoint(block, h) if use_ckpt else block(h)
+        held = torch.cuda.memory_allocated() - base
+        loss = (h * h).mean()
+        loss.backward()
+        torch.cuda.synchronize()
+        return float(loss.detach()), host(x.grad), [host(w.grad) for w in ws], held
+
+    l0, gx0, gw0, held0 = run(False)
+    l1, gx1, gw1, held1 = run(True)
+    print(f"\n  bytes held after forward: plain {held0}, checkpointed {held1}", flush=True)
+    assert l0 == l1
+    assert np.array_equal(gx0, gx1)
+    for a, b in zip(gw0, gw1):
+        assert np.array_equal(a, b)
+    assert held1 * 2 < held0
+
+
 def test_strided_qkv_views():
     """Heads read in place from a fused [N, 3d] projection (no repack)."""
     B, T, H, dk = 2, 256, 4, 64
