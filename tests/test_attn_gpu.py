@@ -105,6 +105,49 @@ def test_bf16_against_oracle(oracle, case):
             assert maxabs(a, w) < BF16_TOL
 
 
+def _sweep_cases(n=28, seed=2024):
+    """Seeded draw over the corners the tiles care about: lengths around multiples of 32 / 64 / 128, windows of
+    1, just under / at / over a tile and past the sequence, sink counts across tile edges, GQA ratios."""
+    rng = np.random.default_rng(seed)
+    lens = [1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 191, 257, 300, 449, 512, 640, 700]
+    wins = [0, 0, 1, 5, 31, 64, 65, 200, 10_000]
+    sinks = [0, 0, 1, 4, 63, 64, 65, 130]
+    out = []
+    for i in range(n):
+        T = int(rng.choice(lens))
+        w = int(rng.choice(wins))
+        out.append((f"sweep{i}", int(rng.integers(1, 3)), T, int(rng.integers(1, 4)), int(rng.integers(1, 3)),
+                    int(rng.choice([64, 128])), bool(w > 0 or rng.integers(0, 4) > 0), w, int(rng.choice(sinks)) if w else 0))
+    return out
+
+
+@pytest.mark.parametrize("case", _sweep_cases(), ids=lambda c: f"{c[0]}_B{c[1]}_T{c[2]}_r{c[3]}_kv{c[4]}_d{c[5]}_c{int(c[6])}_w{c[7]}_s{c[8]}")
+def test_bf16_sweep_against_oracle(oracle, case):
+    name, B, T, rep, Hkv, dk, causal, window, sinks = case
+    q, k, v, d_o = make(B, T, rep * Hkv, Hkv, dk, 1.0, 7000 + T)
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
+    want_o, want_lse = oracle.attn_fwd(q, k, v, scale, causal, window, sinks)
+    want = (want_o, want_lse) + oracle.attn_bwd(q, k, v, d_o, scale, causal, window, sinks)
+    got = run_gpu(q, k, v, d_o, scale, causal, window, sinks, torch.bfloat16, torch.float32)
+    errs = report(name, got, want)
+    assert max(errs[0], errs[2], errs[3], errs[4]) < BF16_TOL and errs[1] < BF16_LSE_TOL
+
+
+@pytest.mark.parametrize("case", _sweep_cases(14, 77), ids=lambda c: f"{c[0]}_T{c[2]}_r{c[3]}_kv{c[4]}_c{int(c[6])}_w{c[7]}_s{c[8]}")
+def test_fp32_sweep_against_oracle(oracle, case):
+    """The fp32 path (any head_dim up to 256) on the same kind of draw, at its own bar of 1e-5; head_dim is taken
+    from a list that includes sizes no MFMA kernel serves."""
+    name, B, T, rep, Hkv, _, causal, window, sinks = case
+    dk = [8, 24, 32, 48, 64, 80, 128, 200][T % 8]
+    rng = np.random.default_rng(9000 + T)
+    q, k, v, d_o = (rng.standard_normal((B, T, h, dk)).astype(np.float32) for h in (rep * Hkv, Hkv, Hkv, rep * Hkv))
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
+    want_o, want_lse = oracle.attn_fwd(q, k, v, scale, causal, window, sinks)
+    want = (want_o, want_lse) + oracle.attn_bwd(q, k, v, d_o, scale, causal, window, sinks)
+    errs = report(f"{name} d{dk}", run_gpu(q, k, v, d_o, scale, causal, window, sinks, torch.float32), want)
+    assert max(errs) < FP32_TOL
+
+
 def test_fp32_path_on_bf16_shapes_agrees(oracle):
     """The generic fp32 kernels at an MFMA-eligible shape: 1e-5."""
     q, k, v, d_o = make(1, 200, 2, 1, 64, 1.0, 900)
