@@ -225,6 +225,49 @@ def test_python_checkpoint_matches_plain():
     assert held1 * 2 < held0
 
 
+def test_two_host_threads_two_streams():
+    """The attention entry points hold no shared mutable state: two host threads, each on its own stream and its
+    own tensors, get exactly the results a single thread gets (ctypes drops the GIL for the duration of a call)."""
+    import threading
+    B, T, H, dk = 2, 512, 4, 128
+    scale = float(1 / np.sqrt(dk))
+
+    def inputs(seed):
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        return tuple(torch.randn((B, T, H, dk), generator=g, device="cuda").bfloat16() for _ in range(4))
+
+    def work(q, k, v, d_o, reps):
+        out = None
+        for _ in range(reps):
+            o, lse = ops.attn_fwd(q, k, v, scale, True)
+            out = (o, lse) + tuple(ops.attn_bwd(q, k, v, o, lse, d_o, scale, True))
+        return out
+
+    data = [inputs(100), inputs(200)]
+    want = [work(*d, 1) for d in data]
+    torch.cuda.synchronize()
+    got, errs = [None, None], []
+
+    def runner(i):
+        try:
+            st = torch.cuda.Stream()
+            with torch.cuda.stream(st):
+                got[i] = work(*data[i], 20)
+            st.synchronize()
+        except Exception as e:  # surfaced in the main thread below
+            errs.append(e)
+
+    th = [threading.Thread(target=runner, args=(i,)) for i in range(2)]
+    for t in th:
+        t.start()
+    for t in th:
+        t.join()
+    assert not errs, errs
+    for w, g in zip(want, got):
+        for a, b in zip(w, g):
+            assert torch.equal(a, b)
+
+
 def test_strided_qkv_views():
     """Heads read in place from a fused [N, 3d] projection (no repack)."""
     B, T, H, dk = 2, 256, 4, 64
