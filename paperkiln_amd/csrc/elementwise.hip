@@ -413,6 +413,15 @@ __global__ void add_parts(const float* part, T* dst, int nparts, int64_t n, floa
     }
 }
 
+__global__ void add_parts4(const float* part, float* dst, int nparts, int64_t n4, float beta) {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n4; i += static_cast<int64_t>(gridDim.x) * NT) {
+        f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int p = 0; p < nparts; ++p) s += *reinterpret_cast<const f32x4*>(part + (p * n4 + i) * 4);
+        f32x4* d = reinterpret_cast<f32x4*>(dst) + i;
+        *d = beta != 0.0f ? *d + s : s;
+    }
+}
+
 // The same sum, scattered: the [M, nsplit*N] result is cut into nsplit column blocks and block k
 // goes to its own contiguous [M, N] destination (the gradients of weights that were multiplied as
 // one concatenated matrix).
@@ -426,6 +435,17 @@ __global__ void add_parts_split(const float* part, SplitDst dst, int nparts, int
         for (int p = 0; p < nparts; ++p) s += part[p * n + i];
         const int64_t r = i / W, c = i % W;
         float* d = dst.p[c / N] + r * N + c % N;
+        *d = beta != 0.0f ? *d + s : s;
+    }
+}
+// four columns per thread (N a multiple of 4, so a group of four never straddles two destinations)
+__global__ void add_parts_split4(const float* part, SplitDst dst, int nparts, int64_t M, int64_t N, int nsplit, float beta) {
+    const int64_t W = N * nsplit, n4 = M * W / 4;
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n4; i += static_cast<int64_t>(gridDim.x) * NT) {
+        f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int p = 0; p < nparts; ++p) s += *reinterpret_cast<const f32x4*>(part + p * (n4 * 4) + i * 4);
+        const int64_t r = (i * 4) / W, c = (i * 4) % W;
+        f32x4* d = reinterpret_cast<f32x4*>(dst.p[c / N] + r * N + c % N);
         *d = beta != 0.0f ? *d + s : s;
     }
 }
@@ -973,7 +993,10 @@ void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dty
                 static_cast<rocblas_int>(N), M * N, S, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
             if (st != rocblas_status_success)
                 throw std::runtime_error(std::string("rocblas_gemm_strided_batched_ex failed: ") + rocblas_status_to_string(st));
-            if (c_dtype == PK_F32)
+            if (c_dtype == PK_F32 && (M * N) % 4 == 0 && aligned16p(C))
+                hipLaunchKernelGGL(add_parts4, ew_grid(M * N / 4), dim3(NT), 0, tape_stream(),
+                                   static_cast<const float*>(part.p), static_cast<float*>(C), S, M * N / 4, beta);
+            else if (c_dtype == PK_F32)
                 hipLaunchKernelGGL((add_parts<float>), ew_grid(M * N), dim3(NT), 0, tape_stream(),
                                    static_cast<const float*>(part.p), static_cast<float*>(C), S, M * N, beta);
             else
@@ -1019,8 +1042,14 @@ void gemm_tn_split(const Tensor& A, const Tensor& B, float* const* dst, int nspl
         throw std::runtime_error(std::string("rocblas_gemm_strided_batched_ex failed: ") + rocblas_status_to_string(st));
     SplitDst d{};
     for (int k = 0; k < nsplit; ++k) d.p[k] = dst[k];
-    hipLaunchKernelGGL(add_parts_split, ew_grid(M * W), dim3(NT), 0, tape_stream(), static_cast<const float*>(part.p), d, S,
-                       M, W / nsplit, nsplit, beta);
+    bool vec = (W / nsplit) % 4 == 0;
+    for (int k = 0; k < nsplit; ++k) vec = vec && aligned16p(dst[k]);
+    if (vec)
+        hipLaunchKernelGGL(add_parts_split4, ew_grid(M * W / 4), dim3(NT), 0, tape_stream(), static_cast<const float*>(part.p),
+                           d, S, M, W / nsplit, nsplit, beta);
+    else
+        hipLaunchKernelGGL(add_parts_split, ew_grid(M * W), dim3(NT), 0, tape_stream(), static_cast<const float*>(part.p), d,
+                           S, M, W / nsplit, nsplit, beta);
     post();
 }
 
