@@ -148,6 +148,32 @@ def test_fp32_sweep_against_oracle(oracle, case):
     assert max(errs) < FP32_TOL
 
 
+@pytest.mark.parametrize("dk", [64, 128])
+def test_bf16_large_scores(oracle, dk):
+    """Scores spread over +-60 natural-log units (softmax close to one-hot, running max moving by far more than the
+    lazy-rescale threshold between tiles, keys ordered so that the maximum keeps growing along the sequence): nothing
+    overflows, LSE holds its absolute bar, O and the gradients hold 2e-2 relative to their own scale."""
+    B, T, H = 1, 320, 2
+    rng = np.random.default_rng(123)
+    q = rng.standard_normal((B, T, H, dk)).astype(np.float32) * 4.0
+    k = rng.standard_normal((B, T, H, dk)).astype(np.float32) * 4.0
+    k *= np.linspace(0.25, 1.5, T, dtype=np.float32)[None, :, None, None]  # later keys reach larger scores
+    v = rng.standard_normal((B, T, H, dk)).astype(np.float32)
+    d_o = rng.standard_normal((B, T, H, dk)).astype(np.float32)
+    q, k, v, d_o = (synth.bf16_round(x) for x in (q, k, v, d_o))
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
+    want_o, want_lse = oracle.attn_fwd(q, k, v, scale, True, 0, 0)
+    want = (want_o, want_lse) + oracle.attn_bwd(q, k, v, d_o, scale, True, 0, 0)
+    got = run_gpu(q, k, v, d_o, scale, True, 0, 0, torch.bfloat16, torch.float32)
+    assert all(np.isfinite(x).all() for x in got)
+    errs = report(f"large scores d{dk} (max |LSE| {np.abs(want_lse).max():.1f})", got, want)
+    assert np.abs(want_lse).max() > 40.0
+    # LSE of magnitude ~100 is held to fp32 relative accuracy, not to 1e-3 absolute
+    assert errs[1] < 1e-5 * float(np.abs(want_lse).max()) + BF16_LSE_TOL
+    for e, w in zip((errs[0], errs[2], errs[3], errs[4]), (want[0], want[2], want[3], want[4])):
+        assert e < BF16_TOL * max(1.0, float(np.abs(w).max()))
+
+
 def test_fp32_path_on_bf16_shapes_agrees(oracle):
     """The generic fp32 kernels at an MFMA-eligible shape: 1e-5."""
     q, k, v, d_o = make(1, 200, 2, 1, 64, 1.0, 900)
