@@ -43,9 +43,37 @@ def cpu_baseline(B, T, H, dk, scale):
 
     units = 2  # about 8 s each on one core
     flops_unit = 14.0 * dk * (T * (T + 1) // 2)
-    ref = load_reference()
-    orc = None if ref is not None else Oracle()
-    kind = "reference" if ref is not None else "port"
+    # The reference's GEMM announces its SIMD level on stdout when the library is loaded; this script's
+    # stdout carries exactly one JSON line, so file descriptor 1 points at stderr while the CPU leg runs.
+    sys.stdout.flush()
+    saved_stdout = os.dup(1)
+    os.dup2(2, 1)
+    try:
+        ref = load_reference()
+        orc = None if ref is not None else Oracle()
+        kind = "reference" if ref is not None else "port"
+        dt = _cpu_units(units, ref, orc, T, dk, scale, synth)
+    finally:
+        import ctypes
+        ctypes.CDLL(None).fflush(None)  # the C library's own stdout buffer, before descriptor 1 goes back
+        sys.stdout.flush()
+        os.dup2(saved_stdout, 1)
+        os.close(saved_stdout)
+    cpu = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                cpu = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {"value": units * flops_unit / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": kind,
+            "sample": f"{units} of {B * H} (batch, head) units of the same workload, fwd+bwd, {dt:.2f} s wall; "
+                      f"whole job would take ~{dt / units * B * H:.0f} s on one core",
+            "host_cpu": cpu, "host_nproc": os.cpu_count()}
+
+
+def _cpu_units(units, ref, orc, T, dk, scale, synth):
     dt = 0.0
     for u in range(units):
         q = synth.bf16_round(synth.randn(11 + 10 * u, (T, dk), 0.5))
@@ -59,18 +87,7 @@ def cpu_baseline(B, T, H, dk, scale):
             _, _, A = orc.head_fwd(q, k, v, scale, 0, True, 0, 0)
             orc.head_bwd(q, k, v, A, g, scale, 0, True, 0, 0)
         dt += time.perf_counter() - t0
-    cpu = "unknown"
-    try:
-        for line in open("/proc/cpuinfo"):
-            if line.startswith("model name"):
-                cpu = line.split(":", 1)[1].strip()
-                break
-    except OSError:
-        pass
-    return {"value": units * flops_unit / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": kind,
-            "sample": f"{units} of {B * H} (batch, head) units of the same workload, fwd+bwd, {dt:.2f} s wall; "
-                      f"whole job would take ~{dt / units * B * H:.0f} s on one core",
-            "host_cpu": cpu, "host_nproc": os.cpu_count()}
+    return dt
 
 
 def window_variant(ops, q, k, v, d_o, out, scale, B, H, T, dk, warmup, steps):
