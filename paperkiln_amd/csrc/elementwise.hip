@@ -556,7 +556,7 @@ __global__ void ce_rows(T* logits, const int* targets, float gscale, float* nll,
 constexpr int CE_NT = 1024, CE_V4 = 8;  // 8 float4 per thread
 template <typename TOut, bool WRITE>
 __global__ __launch_bounds__(CE_NT) void ce_rows_reg(const float* logits, TOut* dl, const int* targets, float gscale,
-                                                     float* nll, int C) {
+                                                     float* nll, int C, int64_t dl_ld) {
     __shared__ float sh[CE_NT / 64];
     const float* row = logits + static_cast<int64_t>(blockIdx.x) * C;
     const int t = targets[blockIdx.x];
@@ -606,7 +606,9 @@ __global__ __launch_bounds__(CE_NT) void ce_rows_reg(const float* logits, TOut* 
                 float o[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) o[e] = (v[i][e] * inv - (j + e == t ? 1.0f : 0.0f)) * gscale;
-                TOut* dst = dl + static_cast<int64_t>(blockIdx.x) * C + j;
+                // dl may be the logits buffer itself (bf16 rows written over the fp32 row they came from):
+                // every thread of the row has its logits in registers since before the first reduction
+                TOut* dst = dl + static_cast<int64_t>(blockIdx.x) * dl_ld + j;
                 if (sizeof(TOut) == 4) {
                     f32x4 w = {o[0], o[1], o[2], o[3]};
                     *reinterpret_cast<f32x4*>(dst) = w;
@@ -892,19 +894,20 @@ void k_ce_rows(const Tensor& logits, const int* targets, float gscale, float* nl
                                                      static_cast<int>(logits.cols)));
     post();
 }
-bool k_ce_rows_once(const Tensor& logits, const int* targets, float gscale, float* nll_rows, const Tensor* dl) {
+bool k_ce_rows_once(const Tensor& logits, const int* targets, float gscale, float* nll_rows, const Tensor* dl, int64_t dl_ld) {
     const int C = static_cast<int>(logits.cols);
+    if (dl_ld == 0) dl_ld = C;
     if (logits.dtype != PK_F32 || C % 4 != 0 || C > CE_NT * CE_V4 * 4) return false;  // caller takes the generic kernel
     const float* src = static_cast<const float*>(logits.ptr());
     if (!dl) {
         hipLaunchKernelGGL((ce_rows_reg<float, false>), dim3(logits.rows), dim3(CE_NT), 0, tape_stream(), src,
-                           static_cast<float*>(nullptr), targets, gscale, nll_rows, C);
+                           static_cast<float*>(nullptr), targets, gscale, nll_rows, C, dl_ld);
     } else if (dl->dtype == PK_F32) {
         hipLaunchKernelGGL((ce_rows_reg<float, true>), dim3(logits.rows), dim3(CE_NT), 0, tape_stream(), src,
-                           static_cast<float*>(dl->ptr()), targets, gscale, nll_rows, C);
+                           static_cast<float*>(dl->ptr()), targets, gscale, nll_rows, C, dl_ld);
     } else {
         hipLaunchKernelGGL((ce_rows_reg<uint16_t, true>), dim3(logits.rows), dim3(CE_NT), 0, tape_stream(), src,
-                           static_cast<uint16_t*>(dl->ptr()), targets, gscale, nll_rows, C);
+                           static_cast<uint16_t*>(dl->ptr()), targets, gscale, nll_rows, C, dl_ld);
     }
     post();
     return true;
@@ -962,7 +965,8 @@ rocblas_handle blas() {
 }  // namespace
 
 void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dtype, int64_t M, int64_t N, int64_t ldc,
-          float beta) {
+          float beta, int64_t lda) {
+    if (lda == 0) lda = A.cols;
     const int64_t Ka = tA ? A.rows : A.cols, Kb = tB ? B.cols : B.rows;
     const int64_t Ma = tA ? A.cols : A.rows, Nb = tB ? B.rows : B.cols;
     if (Ka != Kb) throw std::runtime_error("gemm: inner dimensions disagree");  // device.cpp:97
@@ -984,11 +988,11 @@ void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dty
             const int64_t Ks = Ka / S;
             Buffer part(sizeof(float) * static_cast<size_t>(S) * M * N);
             const float zero = 0.0f;
-            const int64_t stride_a = tA ? Ks * A.cols : Ks, stride_b = Ks * B.cols;
+            const int64_t stride_a = tA ? Ks * lda : Ks, stride_b = Ks * B.cols;
             const rocblas_status st = rocblas_gemm_strided_batched_ex(
                 blas(), rocblas_operation_none, tA ? rocblas_operation_transpose : rocblas_operation_none,
                 static_cast<rocblas_int>(N), static_cast<rocblas_int>(M), static_cast<rocblas_int>(Ks), &alpha, B.ptr(), ab,
-                static_cast<rocblas_int>(B.cols), stride_b, A.ptr(), ab, static_cast<rocblas_int>(A.cols), stride_a, &zero,
+                static_cast<rocblas_int>(B.cols), stride_b, A.ptr(), ab, static_cast<rocblas_int>(lda), stride_a, &zero,
                 part.p, rocblas_datatype_f32_r, static_cast<rocblas_int>(N), M * N, part.p, rocblas_datatype_f32_r,
                 static_cast<rocblas_int>(N), M * N, S, rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
             if (st != rocblas_status_success)
@@ -1010,7 +1014,7 @@ void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dty
         blas(), tB ? rocblas_operation_transpose : rocblas_operation_none,
         tA ? rocblas_operation_transpose : rocblas_operation_none, static_cast<rocblas_int>(N),
         static_cast<rocblas_int>(M), static_cast<rocblas_int>(Ka), &alpha, B.ptr(), ab, static_cast<rocblas_int>(B.cols),
-        A.ptr(), ab, static_cast<rocblas_int>(A.cols), &beta, C, ct, static_cast<rocblas_int>(ldc), C, ct,
+        A.ptr(), ab, static_cast<rocblas_int>(lda), &beta, C, ct, static_cast<rocblas_int>(ldc), C, ct,
         static_cast<rocblas_int>(ldc), rocblas_datatype_f32_r, rocblas_gemm_algo_standard, 0, 0);
     if (st != rocblas_status_success)
         throw std::runtime_error(std::string("rocblas_gemm_ex failed: ") + rocblas_status_to_string(st));

@@ -301,7 +301,7 @@ int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets
         dev_reset_peak();
         const size_t live0 = live_variables();
         Var hid = m->hidden(ids, n, seq_len);
-        Var l = fused_head ? ops::linear_cross_entropy(hid, m->embed, tg, 1024)
+        Var l = fused_head ? ops::linear_cross_entropy(hid, m->embed, tg, 2048)
                            : ops::cross_entropy(ops::matmul_nt(hid, m->embed), tg);
         hid.reset();
         hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");

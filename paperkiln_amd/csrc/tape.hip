@@ -571,15 +571,28 @@ Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffe
         gemm(hview, false, Ec, true, logits.ptr(), PK_F32, rows, V, V, 0.0f);
         float* nll_r = static_cast<float*>(nll.p) + r0;
         const bool grads = want_dh || want_dE;
+        // dlogits takes the place of the logits it came from: in fp32 the same matrix, in bf16 the first half of
+        // every fp32 row (row pitch 2V bf16 elements), so a chunk holds one [rows, V] fp32 buffer and nothing else.
         Tensor dl;
-        if (grads) dl = h->data.dtype == PK_F32 ? logits : Tensor::make(rows, V, h->data.dtype);
-        if (!k_ce_rows_once(logits, tg + r0, g1, nll_r, grads ? &dl : nullptr)) {
-            k_ce_rows(logits, tg + r0, g1, nll_r);
-            if (grads && h->data.dtype != PK_F32) k_cast(logits, dl);
+        int64_t dl_ld = V;
+        if (grads) {
+            dl = logits;
+            if (h->data.dtype != PK_F32) {
+                dl.dtype = h->data.dtype;
+                dl_ld = 2 * V;
+            }
+        }
+        if (!k_ce_rows_once(logits, tg + r0, g1, nll_r, grads ? &dl : nullptr, dl_ld)) {
+            k_ce_rows(logits, tg + r0, g1, nll_r);  // generic row kernel: dlogits in place as fp32
+            if (grads && h->data.dtype != PK_F32) {
+                dl = Tensor::make(rows, V, h->data.dtype);
+                dl_ld = V;
+                k_cast(logits, dl);
+            }
         }
         if (want_dh)
-            gemm(dl, false, Ec, false, static_cast<char*>(dh1.ptr()) + r0 * d * hes, dh1.dtype, rows, d, d, 0.0f);
-        if (want_dE) gemm(dl, true, hview, false, dE1.ptr(), PK_F32, V, d, d, r0 == 0 ? 0.0f : 1.0f);
+            gemm(dl, false, Ec, false, static_cast<char*>(dh1.ptr()) + r0 * d * hes, dh1.dtype, rows, d, d, 0.0f, dl_ld);
+        if (want_dE) gemm(dl, true, hview, false, dE1.ptr(), PK_F32, V, d, d, r0 == 0 ? 0.0f : 1.0f, dl_ld);
     }
     const double total = k_sum_f32_to_host(static_cast<const float*>(nll.p), N);
     Tensor out = Tensor::make(1, 1, PK_F32);

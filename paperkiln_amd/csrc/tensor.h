@@ -116,7 +116,8 @@ void k_embedding_bwd(const Tensor& dy, const int* ids, const Tensor& dtable_f32)
 void k_ce_rows(const Tensor& logits, const int* targets, float gscale, float* nll_rows);
 // The same on fp32 logits that are read once and left untouched: dl == nullptr computes only the nll, otherwise
 // dlogits go to *dl (fp32 or bf16). Returns false when the shape does not fit (the caller then uses k_ce_rows).
-bool k_ce_rows_once(const Tensor& logits, const int* targets, float gscale, float* nll_rows, const Tensor* dl);
+bool k_ce_rows_once(const Tensor& logits, const int* targets, float gscale, float* nll_rows, const Tensor* dl,
+                    int64_t dl_ld = 0);  // dl_ld: row pitch of dl in its own elements (0 = cols)
 double k_sum_f32_to_host(const float* x, int64_t n);                   // double accumulation, ops.cpp:360-367
 double k_sumsq_to_host(const Tensor& g);                               // clip_grad_norm's sum, ops.cpp:1046-1052
 // The same in two halves, so that many gradients cost one host round trip: per-block partial sums (at most
@@ -131,7 +132,7 @@ void k_adamw(const Tensor& p, const Tensor& g, const Tensor& m, const Tensor& v,
 // (device::gemm, src/device.cpp:91-125). C may be a column slice of a wider
 // matrix (ldc). beta is 0 or 1.
 void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dtype, int64_t M, int64_t N, int64_t ldc,
-          float beta);
+          float beta, int64_t lda = 0);
 // dst[k] ([A.cols, B.cols/nsplit] fp32, contiguous) = beta * dst[k] + A^T B[:, k-th column block], k < nsplit <= 4
 void gemm_tn_split(const Tensor& A, const Tensor& B, float* const* dst, int nsplit, float beta);
 
