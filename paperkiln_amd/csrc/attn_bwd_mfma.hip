@@ -63,17 +63,19 @@ struct Tile {
     static constexpr int S = D + 8;             // row pitch (elements)
     static constexpr int NCH = D / 8;           // 16-byte chunks per row
     static constexpr int CPT = ROWS * NCH / 256;
-    __device__ static void load(const void* base, int64_t off, int64_t st_t, int r0, int T, u32x4* r) {
+    // this thread's byte offsets inside a tile whose rows are st_t elements apart
+    __device__ static void offsets(int64_t st_t, int* boff) {
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
             const int c = threadIdx.x + 256 * i;
-            const int row = c / NCH, ch = c % NCH;
-            u32x4 z = {0, 0, 0, 0};
-            if (r0 + row < T)
-                z = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(base) + off +
-                                                    (r0 + row) * st_t + ch * 8);
-            r[i] = z;
+            boff[i] = static_cast<int>((c / NCH) * st_t + (c % NCH) * 8) * 2;
         }
+    }
+    // rows r0 .. r0+ROWS-1 of the matrix at base + off; rows past T read as zero
+    __device__ static void load(const void* base, int64_t off, int64_t st_t, int r0, int T, const int* boff, u32x4* r) {
+        const __amdgpu_buffer_rsrc_t rs = tile_rsrc(base, off, st_t, r0, T, D);
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) r[i] = tile_load16(rs, boff[i]);
     }
     __device__ static void store(uint16_t* lds, const u32x4* r) {
 #pragma unroll
@@ -179,8 +181,11 @@ __global__ __launch_bounds__(256, 2) void mfma_dq(AttnArgs a) {
     int t = ns > 0 ? 0 : lo;
 
     u32x4 kr[KT::CPT], vr[KT::CPT];
-    KT::load(a.k, kb, a.k_st, t * BN, a.T, kr);
-    KT::load(a.v, vb, a.v_st, t * BN, a.T, vr);
+    int koff[KT::CPT], voff[KT::CPT];
+    KT::offsets(a.k_st, koff);
+    KT::offsets(a.v_st, voff);
+    KT::load(a.k, kb, a.k_st, t * BN, a.T, koff, kr);
+    KT::load(a.v, vb, a.v_st, t * BN, a.T, voff, vr);
     KT::store(Ks, kr);
     KT::store(Vs, vr);
     __syncthreads();
@@ -189,8 +194,8 @@ __global__ __launch_bounds__(256, 2) void mfma_dq(AttnArgs a) {
         const int n0 = t * BN;
         const int tn = (t + 1 == ns) ? lo : t + 1;
         if (tn <= hi) {
-            KT::load(a.k, kb, a.k_st, tn * BN, a.T, kr);
-            KT::load(a.v, vb, a.v_st, tn * BN, a.T, vr);
+            KT::load(a.k, kb, a.k_st, tn * BN, a.T, koff, kr);
+            KT::load(a.v, vb, a.v_st, tn * BN, a.T, voff, vr);
         }
         const bool skip = qlo >= a.T || (a.causal && n0 > qhi) ||
                           (a.window > 0 && n0 + BN - 1 + a.window <= qlo && n0 >= a.sinks);

@@ -36,22 +36,17 @@ struct FwdCfg {
     static constexpr int CPT = BN * NCH / 256;  // chunks per thread per tile
 };
 
+// koff / voff: this thread's byte offsets inside a tile (fixed for the whole kernel); keys past the end read as zero
 template <int D>
-__device__ inline void load_kv_regs(const AttnArgs& a, int64_t kb, int64_t vb, int n0, u32x4* kr,
-                                    u32x4* vr) {
+__device__ inline void load_kv_regs(const AttnArgs& a, int64_t kb, int64_t vb, int n0, const int* koff, const int* voff,
+                                    u32x4* kr, u32x4* vr) {
     using C = FwdCfg<D>;
+    const __amdgpu_buffer_rsrc_t krs = tile_rsrc(a.k, kb, a.k_st, n0, a.T, D);
+    const __amdgpu_buffer_rsrc_t vrs = tile_rsrc(a.v, vb, a.v_st, n0, a.T, D);
 #pragma unroll
     for (int i = 0; i < C::CPT; ++i) {
-        const int c = threadIdx.x + 256 * i;
-        const int row = c / C::NCH, ch = c % C::NCH;
-        const int t = n0 + row;
-        u32x4 z = {0, 0, 0, 0};
-        kr[i] = z;
-        vr[i] = z;
-        if (t < a.T) {
-            kr[i] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.k) + kb + t * a.k_st + ch * 8);
-            vr[i] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.v) + vb + t * a.v_st + ch * 8);
-        }
+        kr[i] = tile_load16(krs, koff[i]);
+        vr[i] = tile_load16(vrs, voff[i]);
     }
 }
 
@@ -142,7 +137,14 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
     int t = ns > 0 ? 0 : lo;
 
     u32x4 kr[C::CPT], vr[C::CPT];
-    load_kv_regs<D>(a, kb, vb, t * BN, kr, vr);
+    int koff[C::CPT], voff[C::CPT];
+#pragma unroll
+    for (int i = 0; i < C::CPT; ++i) {
+        const int c = threadIdx.x + 256 * i;
+        koff[i] = static_cast<int>((c / C::NCH) * a.k_st + (c % C::NCH) * 8) * 2;
+        voff[i] = static_cast<int>((c / C::NCH) * a.v_st + (c % C::NCH) * 8) * 2;
+    }
+    load_kv_regs<D>(a, kb, vb, t * BN, koff, voff, kr, vr);
     store_kv_lds<D>(Kbuf[0], Vbuf[0], kr, vr);
     __syncthreads();
     int cur = 0;
@@ -150,7 +152,7 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
     while (t <= hi) {
         const int n0 = t * BN;
         const int tn = (t + 1 == ns) ? lo : t + 1;
-        if (tn <= hi) load_kv_regs<D>(a, kb, vb, tn * BN, kr, vr);  // in flight during the math
+        if (tn <= hi) load_kv_regs<D>(a, kb, vb, tn * BN, koff, voff, kr, vr);  // in flight during the math
         const uint16_t* Ks = Kbuf[cur];
         const uint16_t* Vs = Vbuf[cur];
 

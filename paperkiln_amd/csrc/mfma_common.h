@@ -119,6 +119,20 @@ __device__ inline bf16x8 lds_read_tr_operand_perm(const uint16_t* tile, int stri
     return *reinterpret_cast<bf16x8*>(&v);
 }
 
+// Rows r0 .. of a [T, D] bf16 matrix (row stride `st` elements, first element at base + elem_off) as a
+// buffer resource over what is left of the matrix from row r0 on. Tile loads then take a per-thread byte
+// offset (row_in_tile * st + column) * 2 that never changes, the tile's position sits in the scalar
+// resource, and rows past the end read as zero without a branch (offsets beyond num_records).
+__device__ inline __amdgpu_buffer_rsrc_t tile_rsrc(const void* base, int64_t elem_off, int64_t st, int r0, int T, int D) {
+    const int64_t left = r0 < T ? (static_cast<int64_t>(T - r0 - 1) * st + D) * 2 : 0;
+    const uint16_t* p = static_cast<const uint16_t*>(base) + elem_off + static_cast<int64_t>(min(r0, T)) * st;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, static_cast<int>(left < 0x7fffffff ? left : 0x7fffffff),
+                                             0x00020000);
+}
+__device__ inline u32x4 tile_load16(__amdgpu_buffer_rsrc_t rsrc, int byte_off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, 0, 0);
+}
+
 // XCD-aware workgroup -> tile mapping. The 256 CUs sit in 8 XCDs, each with
 // its own 4 MB L2, and consecutive workgroup ids go round-robin over the XCDs.
 // Every block of a (batch, KV head) unit re-reads that unit's K/V (or Q/dO),
