@@ -3,8 +3,8 @@
 // ops::fused_attention / ops::swa_attention (paperkiln src/ops.cpp:863-902,
 // 948-995), which materialise a [T,T] fp32 weight matrix per head.
 //
-// One workgroup = 4 wavefronts = one (batch, head, 128*NQ-query block). Each
-// wavefront owns NQ blocks of 32 queries and walks the visible key tiles
+// One workgroup = NW wavefronts (4 or 8) = one (batch, head, 32*NW*NQ-query
+// block). Each wavefront owns NQ blocks of 32 queries and walks the visible key tiles
 // (64 keys per step). The work is phrased TRANSPOSED so that every softmax
 // row lives in one lane pair:
 //   S^T[key, query] = K . Q^T      A = K tile from LDS (ds_read_b128),
@@ -28,19 +28,19 @@ namespace {
 
 constexpr int BN = 64;  // keys per step
 
-template <int D>
+template <int D, int NW>
 struct FwdCfg {
     static constexpr int KS = D + 8;    // K tile row pitch: 4 banks past a multiple of 64 -> b128 row reads conflict-free
     static constexpr int VS = D + 32;   // V tile row pitch: 16 banks past -> the 4-row transposing reads conflict-free
     static constexpr int NCH = D / 8;   // 16-byte chunks per row
-    static constexpr int CPT = BN * NCH / 256;  // chunks per thread per tile
+    static constexpr int CPT = BN * NCH / (64 * NW);  // chunks per thread per tile
 };
 
 // koff / voff: this thread's byte offsets inside a tile (fixed for the whole kernel); keys past the end read as zero
-template <int D>
+template <int D, int NW>
 __device__ inline void load_kv_regs(const AttnArgs& a, int64_t kb, int64_t vb, int n0, const int* koff, const int* voff,
                                     u32x4* kr, u32x4* vr) {
-    using C = FwdCfg<D>;
+    using C = FwdCfg<D, NW>;
     const __amdgpu_buffer_rsrc_t krs = tile_rsrc(a.k, kb, a.k_st, n0, a.T, D);
     const __amdgpu_buffer_rsrc_t vrs = tile_rsrc(a.v, vb, a.v_st, n0, a.T, D);
 #pragma unroll
@@ -50,12 +50,12 @@ __device__ inline void load_kv_regs(const AttnArgs& a, int64_t kb, int64_t vb, i
     }
 }
 
-template <int D>
+template <int D, int NW>
 __device__ inline void store_kv_lds(uint16_t* Ks, uint16_t* Vs, const u32x4* kr, const u32x4* vr) {
-    using C = FwdCfg<D>;
+    using C = FwdCfg<D, NW>;
 #pragma unroll
     for (int i = 0; i < C::CPT; ++i) {
-        const int c = threadIdx.x + 256 * i;
+        const int c = threadIdx.x + 64 * NW * i;
         const int row = c / C::NCH, ch = c % C::NCH;
         *reinterpret_cast<u32x4*>(Ks + row * C::KS + ch * 8) = kr[i];
         *reinterpret_cast<u32x4*>(Vs + row * C::VS + ch * 8) = vr[i];
@@ -70,10 +70,10 @@ __device__ inline void store_kv_lds(uint16_t* Ks, uint16_t* Vs, const u32x4* kr,
 // final O = acc / l and LSE = m*scale + ln(l) are exact for any reference m.
 constexpr float LAZY_T = 6.0f;
 
-template <int D, int NQ, int OCC>
-__global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
-    using C = FwdCfg<D>;
-    constexpr int BM = 128 * NQ;
+template <int D, int NQ, int OCC, int NW>
+__global__ __launch_bounds__(64 * NW, OCC) void mfma_fwd(AttnArgs a) {
+    using C = FwdCfg<D, NW>;
+    constexpr int BM = 32 * NW * NQ;
     constexpr int KK = D / 16;  // k-chunks of the QK^T contraction
     constexpr int DB = D / 32;  // 32-row blocks of O^T
     // two K/V tile buffers: tile t+1 is stored while tile t is being read, one barrier per tile
@@ -140,19 +140,19 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
     int koff[C::CPT], voff[C::CPT];
 #pragma unroll
     for (int i = 0; i < C::CPT; ++i) {
-        const int c = threadIdx.x + 256 * i;
+        const int c = threadIdx.x + 64 * NW * i;
         koff[i] = static_cast<int>((c / C::NCH) * a.k_st + (c % C::NCH) * 8) * 2;
         voff[i] = static_cast<int>((c / C::NCH) * a.v_st + (c % C::NCH) * 8) * 2;
     }
-    load_kv_regs<D>(a, kb, vb, t * BN, koff, voff, kr, vr);
-    store_kv_lds<D>(Kbuf[0], Vbuf[0], kr, vr);
+    load_kv_regs<D, NW>(a, kb, vb, t * BN, koff, voff, kr, vr);
+    store_kv_lds<D, NW>(Kbuf[0], Vbuf[0], kr, vr);
     __syncthreads();
     int cur = 0;
 
     while (t <= hi) {
         const int n0 = t * BN;
         const int tn = (t + 1 == ns) ? lo : t + 1;
-        if (tn <= hi) load_kv_regs<D>(a, kb, vb, tn * BN, koff, voff, kr, vr);  // in flight during the math
+        if (tn <= hi) load_kv_regs<D, NW>(a, kb, vb, tn * BN, koff, voff, kr, vr);  // in flight during the math
         const uint16_t* Ks = Kbuf[cur];
         const uint16_t* Vs = Vbuf[cur];
 
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
         }
 
         // The other buffer was last read one iteration ago, before the previous barrier.
-        if (tn <= hi) store_kv_lds<D>(Kbuf[cur ^ 1], Vbuf[cur ^ 1], kr, vr);
+        if (tn <= hi) store_kv_lds<D, NW>(Kbuf[cur ^ 1], Vbuf[cur ^ 1], kr, vr);
         __syncthreads();
         cur ^= 1;
         t = tn;
@@ -265,13 +265,13 @@ __global__ __launch_bounds__(256, OCC) void mfma_fwd(AttnArgs a) {
   }
 }
 
-template <int D, int NQ, int OCC>
+template <int D, int NQ, int OCC, int NW>
 int launch(const AttnArgs& a, hipStream_t st) {
-    constexpr int BM = 128 * NQ;
+    constexpr int BM = 32 * NW * NQ;
     const int nqb = (a.T + BM - 1) / BM;
     const bool paired = pair_causal_blocks(nqb, a.Hq * a.B, a.causal, a.window);
     dim3 grid(xcd_grid(paired ? (nqb + 1) / 2 : nqb, a.Hq / a.Hkv, a.Hkv * a.B));
-    hipLaunchKernelGGL((mfma_fwd<D, NQ, OCC>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((mfma_fwd<D, NQ, OCC, NW>), grid, dim3(64 * NW), 0, st, a);
     PK_HIP(hipGetLastError());
     return PK_OK;
 }
@@ -301,8 +301,14 @@ bool mfma_supported(const AttnArgs& a) {
 
 int launch_mfma_fwd(const AttnArgs& a, hipStream_t st) {
     // One 32-query block per wavefront, two workgroups per CU.
-    if (a.dk_dim == 128) return launch<128, 1, 2>(a, st);
-    return launch<64, 1, 2>(a, st);
+    // Eight wavefronts (256 queries) per K/V tile halve the tile traffic per MFMA (2.7 % faster at T = 4096, 6 % at
+    // T = 16384; slower at head_dim 64 and with a window). One such workgroup fills a CU, so it is only used where the
+    // paired causal grid still gives every CU at least two of them in turn.
+    const int nqb256 = (a.T + 255) / 256;
+    const bool wide = a.dk_dim == 128 && a.causal && a.window == 0 &&
+                      static_cast<int64_t>((nqb256 + 1) / 2) * a.Hq * a.B >= 512;
+    if (a.dk_dim == 128) return wide ? launch<128, 1, 2, 8>(a, st) : launch<128, 1, 2, 4>(a, st);
+    return launch<64, 1, 2, 4>(a, st);
 }
 
 }  // namespace pk
