@@ -58,16 +58,16 @@ __global__ __launch_bounds__(256) void mfma_delta(AttnArgs a) {
 }
 
 // ---- shared tile movers ---------------------------------------------------
-template <int D, int ROWS>
+template <int D, int ROWS, int NW = 4>
 struct Tile {
     static constexpr int S = D + 8;             // row pitch (elements)
     static constexpr int NCH = D / 8;           // 16-byte chunks per row
-    static constexpr int CPT = ROWS * NCH / 256;
+    static constexpr int CPT = ROWS * NCH / (64 * NW);
     // this thread's byte offsets inside a tile whose rows are st_t elements apart
     __device__ static void offsets(int64_t st_t, int* boff) {
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
-            const int c = threadIdx.x + 256 * i;
+            const int c = threadIdx.x + 64 * NW * i;
             boff[i] = static_cast<int>((c / NCH) * st_t + (c % NCH) * 8) * 2;
         }
     }
@@ -80,7 +80,7 @@ struct Tile {
     __device__ static void store(uint16_t* lds, const u32x4* r) {
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
-            const int c = threadIdx.x + 256 * i;
+            const int c = threadIdx.x + 64 * NW * i;
             const int row = c / NCH, ch = c % NCH;
             *reinterpret_cast<u32x4*>(lds + row * S + ch * 8) = r[i];
         }
@@ -117,11 +117,11 @@ __device__ inline void store4(void* base, int64_t idx, float x0, float x1, float
 // FUSE_DELTA: the workgroup also forms delta for its own 128 rows (it holds their dO
 // already; O costs one more row read), uses it and writes it for the dK/dV kernel,
 // which then has to run after this one. Saves the separate pass over O and dO.
-template <int D, bool GF32, bool FUSE_DELTA>
-__global__ __launch_bounds__(256, 2) void mfma_dq(AttnArgs a) {
-    constexpr int BM = 128, BN = 64;
+template <int D, bool GF32, bool FUSE_DELTA, int NW>
+__global__ __launch_bounds__(64 * NW, 2) void mfma_dq(AttnArgs a) {
+    constexpr int BM = 32 * NW, BN = 64;
     constexpr int KK = D / 16, DB = D / 32;
-    using KT = Tile<D, BN>;
+    using KT = Tile<D, BN, NW>;
     __shared__ __attribute__((aligned(16))) uint16_t Ks[BN * KT::S];
     __shared__ __attribute__((aligned(16))) uint16_t Vs[BN * KT::S];
 
@@ -264,13 +264,20 @@ template <int D, bool GF32>
 int launch(const AttnArgs& a, int stages, hipStream_t st) {
     const int64_t rows = static_cast<int64_t>(a.B) * a.Hq * a.T;
     constexpr int RPB = 256 / (D / 8);
-    const int nb128 = (a.T + 127) / 128;
-    const bool paired = pair_causal_blocks(nb128, a.Hq * a.B, a.causal, a.window);
-    const dim3 dq_grid(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, a.Hq / a.Hkv, a.Hkv * a.B));
+    // dQ with 8 wavefronts (256 queries) per K/V tile where the paired causal grid still gives every CU two
+    // workgroups in turn, as in the forward kernel; 4 wavefronts otherwise.
+    const int nb256 = (a.T + 255) / 256;
+    const bool wide = D == 128 && a.causal && a.window == 0 && static_cast<int64_t>((nb256 + 1) / 2) * a.Hq * a.B >= 512;
+    const int nbq = wide ? nb256 : (a.T + 127) / 128;
+    const bool paired = pair_causal_blocks(nbq, a.Hq * a.B, a.causal, a.window);
+    const dim3 dq_grid(xcd_grid(paired ? (nbq + 1) / 2 : nbq, a.Hq / a.Hkv, a.Hkv * a.B));
     // delta and dQ asked for together: dQ forms delta itself and runs first, dK/dV reads what it wrote
     const bool fused = (stages & PK_BWD_DELTA) && (stages & PK_BWD_DQ);
     if (fused) {
-        hipLaunchKernelGGL((mfma_dq<D, GF32, true>), dq_grid, dim3(256), 0, st, a);
+        if (wide)
+            hipLaunchKernelGGL((mfma_dq<D, GF32, true, 8>), dq_grid, dim3(512), 0, st, a);
+        else
+            hipLaunchKernelGGL((mfma_dq<D, GF32, true, 4>), dq_grid, dim3(256), 0, st, a);
         PK_HIP(hipGetLastError());
     } else if (stages & PK_BWD_DELTA) {
         hipLaunchKernelGGL((mfma_delta<D>), dim3((rows + RPB - 1) / RPB), dim3(256), 0, st, a);
@@ -280,7 +287,10 @@ int launch(const AttnArgs& a, int stages, hipStream_t st) {
         if (int rc = launch_mfma_dkdv2(a, st)) return rc;
     }
     if (!fused && (stages & PK_BWD_DQ)) {
-        hipLaunchKernelGGL((mfma_dq<D, GF32, false>), dq_grid, dim3(256), 0, st, a);
+        if (wide)
+            hipLaunchKernelGGL((mfma_dq<D, GF32, false, 8>), dq_grid, dim3(512), 0, st, a);
+        else
+            hipLaunchKernelGGL((mfma_dq<D, GF32, false, 4>), dq_grid, dim3(256), 0, st, a);
         PK_HIP(hipGetLastError());
     }
     return PK_OK;
