@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
 # HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs
 # (FETCH_SIZE, WRITE_SIZE) scaled by a copy kernel of known size; see
 # profiles/. None until measured for the current kernel.
-MEASURED_TRAFFIC_BYTES = {"dkdv": 4.05e8, "dq": 4.96e8, "fwd": 3.66e8}  # profiles/attn_*_pmc.txt, fetch x2.0 + write x1.0
+MEASURED_TRAFFIC_BYTES = {"dkdv": 4.05e8, "dq": 5.60e8, "fwd": 3.76e8}  # profiles/attn_*_pmc.txt, fetch x2.0 + write x1.0
 
 
 def cpu_baseline(B, T, H, dk, scale):
