@@ -276,8 +276,11 @@ int launch(const AttnArgs& a, hipStream_t st) {
     return PK_OK;
 }
 
+// 16-byte-aligned rows, and a row stride that keeps a tile's per-thread byte offsets
+// (up to 256 rows of a buffer-loaded tile) positive and inside 31 bits.
 bool aligned16(const void* p, int64_t sb, int64_t st, int64_t sh) {
-    return (reinterpret_cast<uintptr_t>(p) % 16 == 0) && sb % 8 == 0 && st % 8 == 0 && sh % 8 == 0;
+    return (reinterpret_cast<uintptr_t>(p) % 16 == 0) && sb % 8 == 0 && st % 8 == 0 && sh % 8 == 0 && st > 0 &&
+           st < (int64_t{1} << 22);
 }
 
 }  // namespace

@@ -338,6 +338,36 @@ def test_strided_qkv_views():
     assert torch.equal(o1, o2) and torch.equal(l1, l2)
 
 
+def test_head_major_and_unaligned_layouts():
+    """The same numbers in three layouts: token-major contiguous, head-major ([B, H, T, dk] memory seen
+    through a transpose), and rows pitched dk+2 elements (no 16-byte alignment: the matrix-core kernels
+    decline it and the scalar kernels take over). Forward and backward agree to the bf16 bar."""
+    B, T, H, dk = 2, 200, 4, 64
+    mk = lambda s: torch.from_numpy(synth.randn(s, (B, T, H, dk))).cuda().bfloat16()
+    q, k, v, d_o = mk(1), mk(2), mk(3), mk(4)
+    o, lse = ops.attn_fwd(q, k, v, 0.125, True)
+    grads = ops.attn_bwd(q, k, v, o, lse, d_o, 0.125, True, grad_dtype=torch.float32)
+
+    def head_major(x):
+        y = x.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+        assert y.stride(2) == T * dk and y.stride(1) == dk
+        return y
+
+    def pitched(x):
+        buf = torch.zeros((B, T, H, dk + 2), dtype=x.dtype, device=x.device)
+        buf[..., :dk] = x
+        return buf[..., :dk]
+
+    for name, view, tol_o, tol_l in (("head-major", head_major, 0.0, 0.0), ("pitched", pitched, BF16_TOL, BF16_LSE_TOL)):
+        qv, kv, vv, gv = view(q), view(k), view(v), view(d_o)
+        o2, lse2 = ops.attn_fwd(qv, kv, vv, 0.125, True)
+        assert maxabs(host(o2), host(o)) <= tol_o, name
+        assert maxabs(host(lse2), host(lse)) <= tol_l, name
+        got = ops.attn_bwd(qv, kv, vv, view(o), lse, gv, 0.125, True, grad_dtype=torch.float32)
+        for gname, a, b in zip(("dQ", "dK", "dV"), got, grads):
+            assert maxabs(host(a), host(b)) <= tol_o, f"{name}: {gname}"
+
+
 def test_reference_op_surface(oracle):
     """ops.fused_attention / ops.swa_attention: per-head [rows, dk] matrices, seq_len stacking,
     autograd through the O+LSE-only node, and the reference's error behaviour."""
