@@ -93,6 +93,7 @@ int pk_attn_fwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k
     a.lse = lse;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (s->dtype == PK_BF16 && mfma_supported(a)) return launch_mfma_fwd(a, st);
+    if (s->dtype == PK_F32 && f32_mfma_supported(a)) return launch_f32_mfma_fwd(a, st);
     return launch_generic_fwd(a, s->dtype == PK_BF16, st);
 }
 
@@ -133,6 +134,7 @@ int pk_attn_bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_ten
     a.delta = static_cast<float*>(workspace);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (s->dtype == PK_BF16 && mfma_supported(a)) return launch_mfma_bwd(a, stages, st);
+    if (s->dtype == PK_F32 && f32_mfma_supported(a)) return launch_f32_mfma_bwd(a, stages, st);
     return launch_generic_bwd(a, s->dtype == PK_BF16, stages, st);
 }
 

@@ -63,6 +63,11 @@ __host__ __device__ inline bool pk_visible(int qi, int kj, int T, int causal, in
 int launch_generic_fwd(const AttnArgs& a, bool bf16_in, hipStream_t st);
 int launch_generic_bwd(const AttnArgs& a, bool bf16_in, int stages, hipStream_t st);
 
+// attn_f32_mfma.hip: fp32 tensors on the fp32 matrix instruction, head_dim 32 / 64 / 128.
+bool f32_mfma_supported(const AttnArgs& a);
+int launch_f32_mfma_fwd(const AttnArgs& a, hipStream_t st);
+int launch_f32_mfma_bwd(const AttnArgs& a, int stages, hipStream_t st);
+
 // attn_fwd_mfma.hip / attn_bwd_mfma.hip: bf16 MFMA kernels, head_dim 64 or 128.
 bool mfma_supported(const AttnArgs& a);
 int launch_mfma_fwd(const AttnArgs& a, hipStream_t st);
