@@ -201,8 +201,11 @@ template <int D, bool FUSE_DELTA>
 __global__ __launch_bounds__(256, 1) void f32_dq(AttnArgs a) {
     constexpr int NI = D / 32, NJ = D / 8, P = D + 4, BM = 128;
     typedef typename FVec<NI>::type FV;
-    __shared__ __attribute__((aligned(16))) float Ks[BN * P];
-    __shared__ __attribute__((aligned(16))) float Vs[BN * P];
+    constexpr int CPT = BN * (D / 4) / 256;  // 16-byte chunks per thread, tensor and tile
+    // two K/V tile buffers: tile t+1 is fetched into registers before the matrix work on tile t and
+    // stored behind it, one barrier per tile
+    __shared__ __attribute__((aligned(16))) float Kbuf[2][BN * P];
+    __shared__ __attribute__((aligned(16))) float Vbuf[2][BN * P];
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -257,15 +260,39 @@ __global__ __launch_bounds__(256, 1) void f32_dq(AttnArgs a) {
     const int ns = a.window > 0 ? min((a.sinks + BN - 1) / BN, lo) : 0;
     const QueryVis vis(qi, a.T, a.causal, a.window, a.sinks);
 
-    for (int t = ns > 0 ? 0 : lo; t <= hi; t = (t + 1 == ns) ? lo : t + 1) {
+    f32x4 kr[CPT], vr[CPT];
+    auto fetch = [&](int n0) {  // rows past the end repeat the last row: every use of them is masked
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int c = threadIdx.x + 256 * i;
+            const int tt = min(n0 + c / (D / 4), a.T - 1), ch = c % (D / 4);
+            kr[i] = *reinterpret_cast<const f32x4*>(kbase + tt * a.k_st + ch * 4);
+            vr[i] = *reinterpret_cast<const f32x4*>(vbase + tt * a.v_st + ch * 4);
+        }
+    };
+    auto commit = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int c = threadIdx.x + 256 * i;
+            const int row = c / (D / 4), ch = c % (D / 4);
+            *reinterpret_cast<f32x4*>(Kbuf[slot] + row * P + ch * 4) = kr[i];
+            *reinterpret_cast<f32x4*>(Vbuf[slot] + row * P + ch * 4) = vr[i];
+        }
+    };
+    int t = ns > 0 ? 0 : lo, cur = 0;
+    fetch(t * BN);
+    commit(0);
+    __syncthreads();
+    for (; t <= hi; cur ^= 1) {
         const int n0 = t * BN;
-        __syncthreads();
-        stage_tile<D, BN>(Ks, kbase, a.k_st, n0, a.T);
-        stage_tile<D, BN>(Vs, vbase, a.v_st, n0, a.T);
-        __syncthreads();
-        if (qlo >= a.T) continue;
+        const int tn = (t + 1 == ns) ? lo : t + 1;
+        t = tn;
+        if (tn <= hi) fetch(tn * BN);  // in flight during the matrix work
+        const float* Ks = Kbuf[cur];
+        const float* Vs = Vbuf[cur];
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
+            if (qlo >= a.T) continue;
             const int nn = n0 + nb * 32;
             // wavefront-uniform: nothing of this 32 x 32 block is visible
             if (nn >= a.T) continue;
@@ -302,6 +329,9 @@ __global__ __launch_bounds__(256, 1) void f32_dq(AttnArgs a) {
                 for (int i = 0; i < NI; ++i) acc[i] = mfma2(fv_get<NI>(kc, i), s[r], acc[i]);
             }
         }
+        // the other buffer was last read one tile ago, before the previous barrier
+        if (tn <= hi) commit(cur ^ 1);
+        __syncthreads();
     }
 
     if (qi >= a.T) return;
