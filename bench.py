@@ -26,6 +26,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
+PEAK_FP32_TFLOPS = 157.3   # MI355X dense fp32 MFMA, published
 
 # HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs
 # (FETCH_SIZE, WRITE_SIZE) scaled by a copy kernel of known size; see
@@ -117,6 +118,34 @@ def window_variant(ops, q, k, v, d_o, out, scale, B, H, T, dk, warmup, steps):
                          "unit": "GB/s", "frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}}
 
 
+def fp32_variant(ops, q, k, v, d_o, scale, B, H, T, dk):
+    """Same shape with fp32 tensors (the reference's own element type): the kernels built on the fp32
+    matrix instruction, priced against the fp32 MFMA peak."""
+    import torch
+    from paperkiln_amd import synth
+    q, k, v, d_o = (x.float() for x in (q, k, v, d_o))
+    out = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
+           torch.empty(ops.bwd_workspace_bytes(q, k), dtype=torch.uint8, device=q.device))
+
+    def step():
+        o, lse = ops.attn_fwd(q, k, v, scale, True)
+        ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, out=out)
+
+    warmup, steps = 3, 10
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    tf = 14.0 * dk * synth.visible_pairs(T, True, 0, 0) * B * H / (ms * 1e-3) / 1e12
+    return {"workload": "same shape, fp32 in/out", "steps": steps, "ms_per_step": round(ms, 3), "tflops": round(tf, 2),
+            "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(tf / PEAK_FP32_TFLOPS, 4)}}
+
+
 def llama_step():
     """Activation-checkpointed Llama training step (BASELINE config 5): 6 layers, d=512, 8 heads, SwiGLU 1376,
     vocab 32000 tied, B=8 x T=1024 tokens, bf16 compute with fp32 master weights. Reports tokens/s, the loss
@@ -165,8 +194,8 @@ def main():
                     help="steps of the timed region that carry per-kernel HIP events: every N-th (each event "
                          "costs a few microseconds on the stream, so instrumenting every step slows the job)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--sections", default="window,llama",
-                    help="extra measurements beside the headline: any of window,llama (empty = headline only, "
+    ap.add_argument("--sections", default="window,fp32,llama",
+                    help="extra measurements beside the headline: any of window,fp32,llama (empty = headline only, "
                          "which is what the profiles under profiles/ were taken with)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -263,6 +292,8 @@ def main():
     if "window" in extras:
         res["window_variant"] = window_variant(ops, q, k, v, d_o, out, scale, B, H, T, dk, args.warmup,
                                                max(args.steps // 2, 1))
+    if "fp32" in extras:
+        res["fp32_variant"] = fp32_variant(ops, q, k, v, d_o, scale, B, H, T, dk)
     if "llama" in extras:
         res["llama_step"] = llama_step()
     if not args.no_cpu_baseline:
