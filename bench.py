@@ -220,7 +220,8 @@ def main():
     d_o = torch.randn((B, T, H, dk), generator=gen, device=dev).bfloat16()
     # outputs and scratch are allocated once; the timed region allocates nothing but O/LSE views
     dq, dkk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    ws = torch.empty(4 * B * H * T, dtype=torch.uint8, device=dev)
+    ws = torch.empty(max(ops.bwd_workspace_bytes(q, k), ops.bwd_workspace_bytes(q, k, window=256, sinks=4)),
+                     dtype=torch.uint8, device=dev)
     out = (dq, dkk, dv, ws)
 
     pairs = synth.visible_pairs(T, True, 0, 0)

@@ -72,8 +72,11 @@ int pk_init(int device, char* arch, size_t arch_len);
 int pk_attn_fwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k,
                 const pk_tensor4* v, const pk_tensor4* o, float* lse, void* stream);
 
-/* Bytes of scratch pk_attn_bwd needs for this shape (row sums D_i and, for
- * GQA / bf16 gradients, nothing more). */
+/* Bytes of scratch pk_attn_bwd needs for this shape AND mask: the row sums
+ * D_i [B,Hq,T] fp32 and, for a band mask with 1..32 sink keys, room for the
+ * partial dK/dV rows of the sink keys (the queries past the band of the first
+ * key block may be handed to extra workgroups whose partial sums are added in
+ * a fixed order). Ask with the window and sinks the backward will run with. */
 size_t pk_attn_bwd_workspace_bytes(const pk_attn_shape* s);
 
 /* Backward closure of the same node (src/ops.cpp:902-933, 997-1026),
@@ -89,8 +92,8 @@ int pk_attn_bwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k
 
 /* The same backward by parts, so that a caller can bracket kernels with
  * events: PK_BWD_DELTA (row sums D_i = sum_d O*dO into the workspace),
- * PK_BWD_DKDV (needs DELTA done), PK_BWD_DQ (needs DELTA done). On the bf16
- * path DELTA | DQ in one call is a single kernel (dQ forms D_i for its own
+ * PK_BWD_DKDV (needs DELTA done), PK_BWD_DQ (needs DELTA done). On the
+ * matrix-core paths DELTA | DQ in one call is a single kernel (dQ forms D_i for its own
  * rows and writes them), and pk_attn_bwd == that kernel followed by DKDV.
  * The reference has no counterpart: its closure is a single host function
  * (src/ops.cpp:902-933). */

@@ -70,11 +70,18 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
     // are taken back to back so that every workgroup carries the same work.
     const bool paired = a.causal && a.window == 0;
     int blk, rr, kvu;
-    if (a.window > 0 && a.sinks > 0 && nkb > 1) {
+    // Band mask with a few sink keys: the queries past block 0's band are cut into chunks that get
+    // workgroups of their own (ids nkb .. nkb + nch - 1 of the unit), see sink_tail.
+    const SinkTail tl = a.tail ? sink_tail(a.T, a.window, a.sinks) : SinkTail{0, 0};
+    if (tl.nch > 0) {
+        if (!xcd_map(nkb + tl.nch, 1, a.Hkv * a.B, blk, rr, kvu)) return;
+    } else if (a.window > 0 && a.sinks > 0 && nkb > 1) {
         if (!xcd_map_block0_first(nkb, a.Hkv * a.B, blk, kvu)) return;
     } else if (!xcd_map(paired ? (nkb + 1) / 2 : nkb, 1, a.Hkv * a.B, blk, rr, kvu)) {
         return;
     }
+    const int chunk = blk >= nkb ? blk - nkb : -1;  // >= 0: this workgroup takes a chunk of the sink tail
+    if (chunk >= 0) blk = 0;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv;
     const float cexp = a.scale * LOG2E;
     const int npass = (paired && blk != nkb - 1 - blk) ? 2 : 1;
@@ -109,8 +116,13 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
 
         // Query tiles that can see keys [k0, k0+127] (paperkiln src/ops.cpp:960-965 inverted).
         const int khi = min(k0 + BNK, a.T) - 1;
-        const int qt_lo = a.causal ? k0 / BMQ : 0;
-        const int qt_hi = (a.window > 0 && k0 >= a.sinks) ? min(a.T - 1, khi + a.window - 1) / BMQ : (a.T - 1) / BMQ;
+        int qt_lo = a.causal ? k0 / BMQ : 0;
+        int qt_hi = (a.window > 0 && (k0 >= a.sinks || tl.nch > 0)) ? min(a.T - 1, khi + a.window - 1) / BMQ
+                                                                    : (a.T - 1) / BMQ;
+        if (chunk >= 0) {
+            qt_lo = (tl.q0 + chunk * TAIL_CHUNK) / BMQ;
+            qt_hi = min(a.T - 1, tl.q0 + (chunk + 1) * TAIL_CHUNK - 1) / BMQ;
+        }
         const int nqt = qt_hi - qt_lo + 1;
         const int steps = nqt * rep;
 
@@ -292,7 +304,20 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
             __syncthreads();
         }
 
-        if (kj < a.T) {
+        // Pieces of a split sink tail: the sink keys' rows go to the workspace as fp32 partial sums
+        // (a chunk writes nothing else; the band part of block 0 writes its other rows as usual).
+        const bool piece = tl.nch > 0 && kblk == 0;
+        if (piece && kbw == 0 && kj < a.sinks) {
+            float* rows = sink_tail_rows(a.tail, kvu, tl.nch, chunk >= 0 ? chunk : tl.nch, role == 0 ? 1 : 0, D) + kj * D;
+            const float sc = role == 0 ? 1.0f : a.scale;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int qd = 0; qd < 4; ++qd)
+                    store4g<true>(rows, TrMap<D>::col0(db, qd, g), acc[db][qd * 4] * sc, acc[db][qd * 4 + 1] * sc,
+                                  acc[db][qd * 4 + 2] * sc, acc[db][qd * 4 + 3] * sc);
+        }
+        if (kj < a.T && chunk < 0 && !(piece && kj < a.sinks)) {
             void* dst = role == 0 ? a.dv : a.dk;
             const int64_t ob = role == 0 ? b * a.dv_sb + hk * a.dv_sh + kj * a.dv_st
                                          : b * a.dk_sb + hk * a.dk_sh + kj * a.dk_st;
@@ -308,17 +333,55 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
     }
 }
 
+// dK / dV rows [0, sinks) of every (batch, KV head) = the band part plus the chunks, in that order.
+template <bool GF32>
+__global__ __launch_bounds__(256) void sink_tail_reduce(AttnArgs a, int nch) {
+    const int kvu = blockIdx.x, hk = kvu % a.Hkv, b = kvu / a.Hkv, D = a.dk_dim;
+    for (int idx = threadIdx.x; idx < 2 * a.sinks * D; idx += 256) {
+        const int which = idx / (a.sinks * D), j = (idx / D) % a.sinks, d = idx % D;
+        float sum = sink_tail_rows(a.tail, kvu, nch, nch, which, D)[j * D + d];
+        for (int c = 0; c < nch; ++c) sum += sink_tail_rows(a.tail, kvu, nch, c, which, D)[j * D + d];
+        void* dst = which == 0 ? a.dk : a.dv;
+        const int64_t at = which == 0 ? b * a.dk_sb + hk * a.dk_sh + j * a.dk_st + d
+                                      : b * a.dv_sb + hk * a.dv_sh + j * a.dv_st + d;
+        if (GF32) {
+            static_cast<float*>(dst)[at] = sum;
+        } else {
+            const uint32_t two = pack_bf16(sum, 0.0f);
+            static_cast<uint16_t*>(dst)[at] = static_cast<uint16_t>(two & 0xffffu);
+        }
+    }
+}
+
 template <int D, bool GF32>
-int launch(const AttnArgs& a, hipStream_t st) {
+int launch(const AttnArgs& a_in, hipStream_t st) {
+    AttnArgs a = a_in;
     const int nb128 = (a.T + 127) / 128;
     const bool paired = a.causal && a.window == 0;
-    hipLaunchKernelGGL((mfma_dkdv2<D, GF32>), dim3(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, 1, a.Hkv * a.B)),
-                       dim3(512), 0, st, a);
+    SinkTail tl = a.tail ? sink_tail(a.T, a.window, a.sinks) : SinkTail{0, 0};
+    // a tail step keeps two of the eight wavefronts busy but takes as long as a full one (measured)
+    if (!sink_tail_pays(tl, a.T, a.window, a.Hkv * a.B, 64, 3, 1.0f)) {
+        a.tail = nullptr;
+        tl.nch = 0;
+    }
+    const int nblk = tl.nch > 0 ? nb128 + tl.nch : paired ? (nb128 + 1) / 2 : nb128;
+    hipLaunchKernelGGL((mfma_dkdv2<D, GF32>), dim3(xcd_grid(nblk, 1, a.Hkv * a.B)), dim3(512), 0, st, a);
     PK_HIP(hipGetLastError());
+    if (tl.nch > 0) return launch_sink_tail_reduce(a, st);
     return PK_OK;
 }
 
 }  // namespace
+
+int launch_sink_tail_reduce(const AttnArgs& a, hipStream_t st) {
+    const int nch = sink_tail(a.T, a.window, a.sinks).nch;
+    if (a.grad_f32)
+        hipLaunchKernelGGL(sink_tail_reduce<true>, dim3(a.Hkv * a.B), dim3(256), 0, st, a, nch);
+    else
+        hipLaunchKernelGGL(sink_tail_reduce<false>, dim3(a.Hkv * a.B), dim3(256), 0, st, a, nch);
+    PK_HIP(hipGetLastError());
+    return PK_OK;
+}
 
 int launch_mfma_dkdv2(const AttnArgs& a, hipStream_t st) {
     if (a.dk_dim == 128) return a.grad_f32 ? launch<128, true>(a, st) : launch<128, false>(a, st);

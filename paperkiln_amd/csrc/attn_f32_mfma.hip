@@ -367,7 +367,12 @@ __global__ __launch_bounds__(256, 1) void f32_dkdv(AttnArgs a) {
     const int g = lane >> 5, c32 = lane & 31;
     const int nkb = (a.T + BNK - 1) / BNK, rep = a.Hq / a.Hkv;
     int kblk, rr, kvu;
-    if (!xcd_map(nkb, 1, a.Hkv * a.B, kblk, rr, kvu)) return;  // key block 0 (seen by every query) first
+    // key block 0 (seen by every query) first; ids nkb .. nkb + nch - 1 of a unit are the chunks of a
+    // split sink tail (see sink_tail)
+    const SinkTail tl = a.tail ? sink_tail(a.T, a.window, a.sinks) : SinkTail{0, 0};
+    if (!xcd_map(nkb + tl.nch, 1, a.Hkv * a.B, kblk, rr, kvu)) return;
+    const int chunk = kblk >= nkb ? kblk - nkb : -1;
+    if (chunk >= 0) kblk = 0;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv;
     const int k0 = kblk * BNK, kw0 = k0 + w * 32, kj = kw0 + c32;
     const float cexp = a.scale * LOG2E;
@@ -391,8 +396,14 @@ __global__ __launch_bounds__(256, 1) void f32_dkdv(AttnArgs a) {
 
     // Query tiles that can see keys [k0, k0+127] (src/ops.cpp:960-965 inverted).
     const int khi = min(k0 + BNK, a.T) - 1;
-    const int qt_lo = a.causal ? k0 / BQ : 0;
-    const int qt_hi = (a.window > 0 && k0 >= a.sinks) ? min(a.T - 1, khi + a.window - 1) / BQ : (a.T - 1) / BQ;
+    int qt_lo = a.causal ? k0 / BQ : 0;
+    int qt_hi = (a.window > 0 && (k0 >= a.sinks || tl.nch > 0)) ? min(a.T - 1, khi + a.window - 1) / BQ : (a.T - 1) / BQ;
+    if (chunk >= 0) {
+        qt_lo = (tl.q0 + chunk * TAIL_CHUNK) / BQ;
+        qt_hi = min(a.T - 1, tl.q0 + (chunk + 1) * TAIL_CHUNK - 1) / BQ;
+    } else if (tl.nch > 0 && kblk == 0) {
+        qt_hi = tl.q0 / BQ - 1;  // the band part ends where the first chunk starts
+    }
     const int nqt = qt_hi - qt_lo + 1;
     const int steps = nqt * rep;
     const KeyVis vis(kj, a.T, a.causal, a.window, a.sinks);
@@ -503,6 +514,17 @@ __global__ __launch_bounds__(256, 1) void f32_dkdv(AttnArgs a) {
     if (kj >= a.T) return;
     float* dkrow = static_cast<float*>(a.dk) + b * a.dk_sb + hk * a.dk_sh + kj * a.dk_st;
     float* dvrow = static_cast<float*>(a.dv) + b * a.dv_sb + hk * a.dv_sh + kj * a.dv_st;
+    if (tl.nch > 0 && kblk == 0) {
+        // a piece of a split sink tail: the sink keys' rows go to the workspace as partial sums
+        // (a chunk writes nothing else; the band part writes its other rows as usual)
+        if (w == 0 && kj < a.sinks) {
+            const int piece = chunk >= 0 ? chunk : tl.nch;
+            dkrow = sink_tail_rows(a.tail, kvu, tl.nch, piece, 0, D) + kj * D;
+            dvrow = sink_tail_rows(a.tail, kvu, tl.nch, piece, 1, D) + kj * D;
+        } else if (chunk >= 0) {
+            return;
+        }
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
         FV ok, ov;
@@ -529,7 +551,11 @@ int launch_fwd(const AttnArgs& a, hipStream_t st) {
 }
 
 template <int D>
-int launch_bwd(const AttnArgs& a, int stages, hipStream_t st) {
+int launch_bwd(const AttnArgs& a_in, int stages, hipStream_t st) {
+    AttnArgs a = a_in;
+    // a tail step is one wavefront's matrix work, as long as a full step's
+    if (!sink_tail_pays(a.tail ? sink_tail(a.T, a.window, a.sinks) : SinkTail{0, 0}, a.T, a.window, a.Hkv * a.B, 32, 1, 1.0f))
+        a.tail = nullptr;
     const dim3 dq_grid(xcd_grid((a.T + 127) / 128, a.Hq / a.Hkv, a.Hkv * a.B));
     const bool fused = (stages & PK_BWD_DELTA) && (stages & PK_BWD_DQ);
     if (fused) {  // dQ forms delta itself and runs first; dK/dV reads what it wrote
@@ -539,9 +565,12 @@ int launch_bwd(const AttnArgs& a, int stages, hipStream_t st) {
         if (int rc = launch_generic_bwd(a, false, PK_BWD_DELTA, st)) return rc;
     }
     if (stages & PK_BWD_DKDV) {
-        const dim3 grid(xcd_grid((a.T + 127) / 128, 1, a.Hkv * a.B));
+        const int nch = a.tail ? sink_tail(a.T, a.window, a.sinks).nch : 0;
+        const dim3 grid(xcd_grid((a.T + 127) / 128 + nch, 1, a.Hkv * a.B));
         hipLaunchKernelGGL(f32_dkdv<D>, grid, dim3(256), 0, st, a);
         PK_HIP(hipGetLastError());
+        if (nch > 0)
+            if (int rc = launch_sink_tail_reduce(a, st)) return rc;
     }
     if (!fused && (stages & PK_BWD_DQ)) {
         hipLaunchKernelGGL((f32_dq<D, false>), dq_grid, dim3(256), 0, st, a);

@@ -44,6 +44,15 @@ int check_shape(const pk_attn_shape* s, const char* who) {
 
 bool bad(const pk_tensor4* t) { return !t || !t->ptr; }
 
+// workspace = delta [B, Hq, T] fp32, then (band mask with 1..32 sink keys only) the sink-tail partial rows
+size_t delta_bytes(const pk_attn_shape* s) { return sizeof(float) * static_cast<size_t>(s->B) * s->Hq * s->T; }
+size_t tail_bytes(const pk_attn_shape* s) {
+    const SinkTail t = sink_tail(s->T, s->window, s->sinks);
+    if (t.nch == 0) return 0;
+    const size_t pad = (256 - delta_bytes(s) % 256) % 256;
+    return pad + sink_tail_bytes(s->B * s->Hkv, t.nch, s->dk);
+}
+
 void fill_common(AttnArgs& a, const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k,
                  const pk_tensor4* v, const pk_tensor4* o) {
     std::memset(&a, 0, sizeof a);
@@ -99,7 +108,7 @@ int pk_attn_fwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k
 
 size_t pk_attn_bwd_workspace_bytes(const pk_attn_shape* s) {
     if (check_shape(s, "pk_attn_bwd_workspace_bytes")) return 0;
-    return sizeof(float) * static_cast<size_t>(s->B) * s->Hq * s->T;
+    return delta_bytes(s) + tail_bytes(s);
 }
 
 int pk_attn_bwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k, const pk_tensor4* v,
@@ -132,6 +141,10 @@ int pk_attn_bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_ten
     a.dk = dk->ptr; a.dk_sb = dk->stride_b; a.dk_st = dk->stride_t; a.dk_sh = dk->stride_h;
     a.dv = dv->ptr; a.dv_sb = dv->stride_b; a.dv_st = dv->stride_t; a.dv_sh = dv->stride_h;
     a.delta = static_cast<float*>(workspace);
+    if (tail_bytes(s)) {
+        const size_t db = delta_bytes(s);
+        a.tail = reinterpret_cast<float*>(static_cast<char*>(workspace) + db + (256 - db % 256) % 256);
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (s->dtype == PK_BF16 && mfma_supported(a)) return launch_mfma_bwd(a, stages, st);
     if (s->dtype == PK_F32 && f32_mfma_supported(a)) return launch_f32_mfma_bwd(a, stages, st);

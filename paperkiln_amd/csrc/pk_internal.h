@@ -33,6 +33,7 @@ struct AttnArgs {
     void* dk;
     void* dv;
     float* delta;    // bwd scratch: rowsum(dO .* O)   [B,Hq,T]
+    float* tail;     // bwd scratch: partial dK/dV rows of the sink keys (see sink_tail), or null
     int64_t q_sb, q_st, q_sh;
     int64_t k_sb, k_st, k_sh;
     int64_t v_sb, v_st, v_sh;
@@ -57,6 +58,50 @@ __host__ __device__ inline bool pk_visible(int qi, int kj, int T, int causal, in
     if (window > 0 && kj + window <= qi && kj >= sinks) return false;
     return true;
 }
+
+// Sink tail. With a band mask and a few sink keys (window > 0, 0 < sinks <= 32) the queries past the
+// band of key block 0 see nothing of that block but the sink keys, yet the workgroup that owns the
+// block would walk every one of them alone: the longest chain of the dK/dV launch by far. The
+// matrix-core dK/dV kernels cut that tail into chunks of TAIL_CHUNK queries, each taken by a
+// workgroup of its own. Every piece -- the block's own band part and each chunk -- writes its fp32
+// partial dK and dV rows of the sink keys into the workspace,
+//   tail[((unit * (nch + 1) + piece) * 2 + {0: dK, 1: dV}) * 32 + key][head_dim],   piece nch = band part,
+// and a small kernel adds the pieces in a fixed order into the output rows (no atomics, repeatable).
+constexpr int TAIL_CHUNK = 512;
+struct SinkTail {
+    int q0;   // first query of the tail, a multiple of 64
+    int nch;  // number of chunks; 0 = the tail is not split
+};
+__host__ __device__ inline SinkTail sink_tail(int T, int window, int sinks) {
+    SinkTail t = {0, 0};
+    if (window <= 0 || sinks <= 0 || sinks > 32) return t;
+    const long long q0 = ((127LL + window - 1) / 64 + 1) * 64;  // first 64-query tile wholly past block 0's band
+    if (q0 >= T) return t;
+    t.q0 = static_cast<int>(q0);
+    t.nch = (T - t.q0 + TAIL_CHUNK - 1) / TAIL_CHUNK;
+    return t;
+}
+__host__ __device__ inline size_t sink_tail_bytes(int kv_units, int nch, int dk) {
+    return nch > 0 ? sizeof(float) * static_cast<size_t>(kv_units) * (nch + 1) * 2 * 32 * dk : 0;
+}
+__host__ __device__ inline float* sink_tail_rows(float* tail, int unit, int nch, int piece, int which, int dk) {
+    return tail + ((static_cast<size_t>(unit) * (nch + 1) + piece) * 2 + which) * 32 * dk;
+}
+// Whether splitting pays: the tail is one chain of (T - q0) / step query steps (at `speedup` times the
+// pace of a full step), the rest of the launch is about
+// ceil(workgroups / 256 CUs) workgroups in turn of (128 + window) / step + `prologue` steps each; the
+// chunks cost a prologue apiece, so the tail is only split where it would outlast the rest.
+__host__ inline bool sink_tail_pays(const SinkTail& t, int T, int window, int kv_units, int step, int prologue,
+                                    float speedup) {
+    if (t.nch == 0) return false;
+    const float chain = static_cast<float>(T - t.q0) / step / speedup;
+    const int nkb = (T + 127) / 128;
+    const float rest = static_cast<float>((static_cast<int64_t>(nkb) * kv_units + 255) / 256) *
+                       ((128 + window) / step + prologue);
+    return chain > rest;
+}
+// adds the pieces into dK/dV rows [0, sinks) of every (batch, KV head); attn_bwd_dkdv2.hip
+int launch_sink_tail_reduce(const AttnArgs& a, hipStream_t st);
 
 // attn_generic.hip: fp32-math kernels for any head_dim <= 256 and either
 // element type. The fp32 contract (max-abs 1e-5 vs the CPU reference) lives here.

@@ -58,9 +58,10 @@ def attn_fwd(q, k, v, scale, causal=True, window=0, sinks=0):
 BWD_DELTA, BWD_DKDV, BWD_DQ, BWD_ALL = 1, 2, 4, 7
 
 
-def bwd_workspace_bytes(q, k, grad_dtype=None):
-    """Bytes of scratch pk_attn_bwd needs for these shapes (pk_attn_bwd_workspace_bytes)."""
-    sh = _shape(q, k, 1.0, True, 0, 0, grad_dtype or q.dtype)
+def bwd_workspace_bytes(q, k, grad_dtype=None, window=0, sinks=0):
+    """Bytes of scratch pk_attn_bwd needs for these shapes and this mask (pk_attn_bwd_workspace_bytes):
+    a band mask with sink keys needs more than the plain causal mask."""
+    sh = _shape(q, k, 1.0, True, window, sinks, grad_dtype or q.dtype)
     return max(int(_lib.lib().pk_attn_bwd_workspace_bytes(C.byref(sh))), 16)
 
 

@@ -189,6 +189,36 @@ def test_fp32_matrix_core_long_sequence(oracle, dk, window, sinks):
         assert e < grad_bar(w_)
 
 
+@pytest.mark.parametrize("dtype,dk,grad", [(torch.bfloat16, 128, torch.float32), (torch.bfloat16, 64, torch.bfloat16),
+                                           (torch.float32, 128, None), (torch.float32, 32, None)],
+                         ids=["bf16_d128", "bf16_d64_bf16grads", "fp32_d128", "fp32_d32"])
+@pytest.mark.parametrize("T,window,sinks", [(1501, 16, 3), (1100, 100, 32), (2048, 40, 1)])
+def test_split_sink_tail_against_oracle(oracle, dtype, dk, grad, T, window, sinks):
+    """Long sequence, narrow band, a few sink keys, few (batch, head) units: the shape where the dK/dV kernels
+    hand the queries past key block 0's band to extra workgroups and add their partial sink rows afterwards.
+    Everything against the oracle; the sink rows of dK and dV are the ones that path produces."""
+    B, Hq, Hkv = 1, 2, 1
+    q, k, v, d_o = make(B, T, Hq, Hkv, dk, 1.0, 600 + T + dk)
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
+    want_o, want_lse = oracle.attn_fwd(q, k, v, scale, True, window, sinks)
+    want = (want_o, want_lse) + oracle.attn_bwd(q, k, v, d_o, scale, True, window, sinks)
+    got = run_gpu(q, k, v, d_o, scale, True, window, sinks, dtype, grad)
+    errs = report(f"split tail T{T} w{window} s{sinks} d{dk}", got, want)
+    if dtype == torch.float32:
+        assert max(errs[:2]) < FP32_TOL
+        for e, w_ in zip(errs[2:], want[2:]):
+            assert e < grad_bar(w_)
+    else:
+        # the sink rows sum over every query of the sequence: hold them relative to their own size
+        assert errs[0] < BF16_TOL and errs[1] < BF16_LSE_TOL
+        for g_, w_ in zip(got[2:], want[2:]):
+            assert maxabs(g_, w_) < BF16_TOL * max(1.0, float(np.abs(w_).max()))
+    # the rows the partial sums feed, on their own
+    for g_, w_ in zip(got[3:], want[3:]):
+        rel = maxabs(g_[:, :sinks], w_[:, :sinks]) / max(1.0, float(np.abs(w_[:, :sinks]).max()))
+        assert rel < (FP32_TOL if dtype == torch.float32 else BF16_TOL)
+
+
 @pytest.mark.parametrize("dk", [64, 128])
 def test_bf16_large_scores(oracle, dk):
     """Scores spread over +-60 natural-log units (softmax close to one-hot, running max moving by far more than the
@@ -238,7 +268,7 @@ def test_backward_by_parts_equals_one_call(dtype, window, sinks):
     o, lse = ops.attn_fwd(q, k, v, scale, True, window, sinks)
     one = ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, window, sinks)
     out = tuple(torch.full_like(x, float("nan")) for x in (q, k, v))
-    ws = torch.empty(ops.bwd_workspace_bytes(q, k), dtype=torch.uint8, device="cuda")
+    ws = torch.empty(ops.bwd_workspace_bytes(q, k, window=window, sinks=sinks), dtype=torch.uint8, device="cuda")
     for st in (ops.BWD_DELTA, ops.BWD_DKDV, ops.BWD_DQ):
         ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, window, sinks, out=out + (ws,), stages=st)
     torch.cuda.synchronize()
@@ -344,7 +374,7 @@ def test_forward_backward_under_graph_capture():
     gen = torch.Generator(device="cuda").manual_seed(31)
     q, k, v, d_o = (torch.randn((B, T, H, dk), generator=gen, device="cuda").bfloat16() for _ in range(4))
     dq, dk_, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    ws = torch.empty(ops.bwd_workspace_bytes(q, k), dtype=torch.uint8, device="cuda")
+    ws = torch.empty(ops.bwd_workspace_bytes(q, k, window=64, sinks=2), dtype=torch.uint8, device="cuda")
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):  # warm-up outside the capture, as torch asks
