@@ -43,7 +43,9 @@ __device__ inline void store4g(void* base, int64_t idx, float x0, float x1, floa
     }
 }
 
-template <int D, bool GF32>
+// TAIL: the launch carries the extra workgroups of a split sink tail (a separate instantiation, so
+// that the plain causal kernel keeps its register budget)
+template <int D, bool GF32, bool TAIL>
 __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
     constexpr int KK = D / 16, DB = D / 32;
     constexpr int S = D + 8;            // tile row pitch (elements): 16-byte row reads conflict-free
@@ -72,16 +74,16 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
     int blk, rr, kvu;
     // Band mask with a few sink keys: the queries past block 0's band are cut into chunks that get
     // workgroups of their own (ids nkb .. nkb + nch - 1 of the unit), see sink_tail.
-    const SinkTail tl = a.tail ? sink_tail(a.T, a.window, a.sinks) : SinkTail{0, 0};
-    if (tl.nch > 0) {
+    const SinkTail tl = TAIL ? sink_tail(a.T, a.window, a.sinks) : SinkTail{0, 0};
+    if (TAIL) {
         if (!xcd_map(nkb + tl.nch, 1, a.Hkv * a.B, blk, rr, kvu)) return;
     } else if (a.window > 0 && a.sinks > 0 && nkb > 1) {
         if (!xcd_map_block0_first(nkb, a.Hkv * a.B, blk, kvu)) return;
     } else if (!xcd_map(paired ? (nkb + 1) / 2 : nkb, 1, a.Hkv * a.B, blk, rr, kvu)) {
         return;
     }
-    const int chunk = blk >= nkb ? blk - nkb : -1;  // >= 0: this workgroup takes a chunk of the sink tail
-    if (chunk >= 0) blk = 0;
+    const int chunk = (TAIL && blk >= nkb) ? blk - nkb : -1;  // >= 0: this workgroup takes a chunk of the sink tail
+    if (TAIL && chunk >= 0) blk = 0;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv;
     const float cexp = a.scale * LOG2E;
     const int npass = (paired && blk != nkb - 1 - blk) ? 2 : 1;
@@ -117,9 +119,9 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
         // Query tiles that can see keys [k0, k0+127] (paperkiln src/ops.cpp:960-965 inverted).
         const int khi = min(k0 + BNK, a.T) - 1;
         int qt_lo = a.causal ? k0 / BMQ : 0;
-        int qt_hi = (a.window > 0 && (k0 >= a.sinks || tl.nch > 0)) ? min(a.T - 1, khi + a.window - 1) / BMQ
-                                                                    : (a.T - 1) / BMQ;
-        if (chunk >= 0) {
+        int qt_hi = (a.window > 0 && (k0 >= a.sinks || TAIL)) ? min(a.T - 1, khi + a.window - 1) / BMQ
+                                                              : (a.T - 1) / BMQ;
+        if (TAIL && chunk >= 0) {
             qt_lo = (tl.q0 + chunk * TAIL_CHUNK) / BMQ;
             qt_hi = min(a.T - 1, tl.q0 + (chunk + 1) * TAIL_CHUNK - 1) / BMQ;
         }
@@ -306,7 +308,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
 
         // Pieces of a split sink tail: the sink keys' rows go to the workspace as fp32 partial sums
         // (a chunk writes nothing else; the band part of block 0 writes its other rows as usual).
-        const bool piece = tl.nch > 0 && kblk == 0;
+        const bool piece = TAIL && kblk == 0;
         if (piece && kbw == 0 && kj < a.sinks) {
             float* rows = sink_tail_rows(a.tail, kvu, tl.nch, chunk >= 0 ? chunk : tl.nch, role == 0 ? 1 : 0, D) + kj * D;
             const float sc = role == 0 ? 1.0f : a.scale;
@@ -364,10 +366,14 @@ int launch(const AttnArgs& a_in, hipStream_t st) {
         a.tail = nullptr;
         tl.nch = 0;
     }
-    const int nblk = tl.nch > 0 ? nb128 + tl.nch : paired ? (nb128 + 1) / 2 : nb128;
-    hipLaunchKernelGGL((mfma_dkdv2<D, GF32>), dim3(xcd_grid(nblk, 1, a.Hkv * a.B)), dim3(512), 0, st, a);
+    if (tl.nch > 0) {
+        hipLaunchKernelGGL((mfma_dkdv2<D, GF32, true>), dim3(xcd_grid(nb128 + tl.nch, 1, a.Hkv * a.B)), dim3(512), 0, st, a);
+        PK_HIP(hipGetLastError());
+        return launch_sink_tail_reduce(a, st);
+    }
+    hipLaunchKernelGGL((mfma_dkdv2<D, GF32, false>), dim3(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, 1, a.Hkv * a.B)),
+                       dim3(512), 0, st, a);
     PK_HIP(hipGetLastError());
-    if (tl.nch > 0) return launch_sink_tail_reduce(a, st);
     return PK_OK;
 }
 
