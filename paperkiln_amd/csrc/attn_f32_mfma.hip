@@ -79,10 +79,16 @@ __global__ __launch_bounds__(256, 2) void f32_fwd(AttnArgs a) {
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = lane >> 5, c32 = lane & 31;
     const int nqb = (a.T + BM - 1) / BM, rep = a.Hq / a.Hkv;
+    // Full-causal work per query block grows with its index: a workgroup takes blocks i and
+    // nqb-1-i back to back where the halved grid still fills the chip (pair_causal_blocks), else the
+    // blocks are dispatched singly, heaviest first.
+    const bool paired = pair_causal_blocks(nqb, a.Hq * a.B, a.causal, a.window);
     int blk, rr, kvu;
-    if (!xcd_map(nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
+    if (!xcd_map(paired ? (nqb + 1) / 2 : nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv, h = hk * rep + rr;
-    const int q0 = (nqb - 1 - blk) * BM;  // heaviest causal blocks first
+    const int npass = (paired && blk != nqb - 1 - blk) ? 2 : 1;
+  for (int pass = 0; pass < npass; ++pass) {
+    const int q0 = (pass == 0 ? nqb - 1 - blk : blk) * BM;
     const int qlo = q0 + w * 32, qhi = qlo + 31, qi = qlo + c32;
     const float* kbase = static_cast<const float*>(a.k) + b * a.k_sb + hk * a.k_sh;
     const float* vbase = static_cast<const float*>(a.v) + b * a.v_sb + hk * a.v_sh;
@@ -179,17 +185,19 @@ __global__ __launch_bounds__(256, 2) void f32_fwd(AttnArgs a) {
     }
 
     const float lt = xhalf_sum(l);
-    if (qi >= a.T) return;
-    const float inv = 1.0f / lt;
-    float* orow = static_cast<float*>(a.o) + b * a.o_sb + h * a.o_sh + qi * a.o_st;
+    if (qi < a.T) {
+        const float inv = 1.0f / lt;
+        float* orow = static_cast<float*>(a.o) + b * a.o_sb + h * a.o_sh + qi * a.o_st;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        FV out;
+        for (int r = 0; r < 16; ++r) {
+            FV out;
 #pragma unroll
-        for (int i = 0; i < NI; ++i) fv_set<NI>(out, i, acc[i][r] * inv);
-        *reinterpret_cast<FV*>(orow + NI * crow(r, g)) = out;
+            for (int i = 0; i < NI; ++i) fv_set<NI>(out, i, acc[i][r] * inv);
+            *reinterpret_cast<FV*>(orow + NI * crow(r, g)) = out;
+        }
+        if (g == 0) a.lse[(static_cast<int64_t>(b) * a.Hq + h) * a.T + qi] = m * a.scale + logf(lt);
     }
-    if (g == 0) a.lse[(static_cast<int64_t>(b) * a.Hq + h) * a.T + qi] = m * a.scale + logf(lt);
+  }
 }
 
 // ---------------------------------------------------------------- dQ
@@ -211,10 +219,13 @@ __global__ __launch_bounds__(256, 1) void f32_dq(AttnArgs a) {
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int g = lane >> 5, c32 = lane & 31;
     const int nqb = (a.T + BM - 1) / BM, rep = a.Hq / a.Hkv;
+    const bool paired = pair_causal_blocks(nqb, a.Hq * a.B, a.causal, a.window);  // as in the forward
     int blk, rr, kvu;
-    if (!xcd_map(nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
+    if (!xcd_map(paired ? (nqb + 1) / 2 : nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv, h = hk * rep + rr;
-    const int q0 = (nqb - 1 - blk) * BM;
+    const int npass = (paired && blk != nqb - 1 - blk) ? 2 : 1;
+  for (int pass = 0; pass < npass; ++pass) {
+    const int q0 = (pass == 0 ? nqb - 1 - blk : blk) * BM;
     const int qlo = q0 + w * 32, qhi = qlo + 31, qi = qlo + c32;
     const int qc = min(qi, a.T - 1);
     const float* kbase = static_cast<const float*>(a.k) + b * a.k_sb + hk * a.k_sh;
@@ -301,14 +312,31 @@ __global__ __launch_bounds__(256, 1) void f32_dq(AttnArgs a) {
             f32x16 s, dp;
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.0f;
+            // One wavefront per SIMD: nothing else covers the LDS latency, so every fragment is read one
+            // group of MFMAs ahead of its use and the order is pinned (reads of the next group, then
+            // the MFMAs of this one).
+            {
+                f32x4 kf = *reinterpret_cast<const f32x4*>(Ks + (nb * 32 + c32) * P + 4 * g);
+                f32x4 vf = *reinterpret_cast<const f32x4*>(Vs + (nb * 32 + c32) * P + 4 * g);
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                const f32x4 kf = *reinterpret_cast<const f32x4*>(Ks + (nb * 32 + c32) * P + 8 * j + 4 * g);
-                const f32x4 vf = *reinterpret_cast<const f32x4*>(Vs + (nb * 32 + c32) * P + 8 * j + 4 * g);
+                for (int j = 0; j < NJ; ++j) {
+                    f32x4 nk = kf, nv = vf;
+                    if (j + 1 < NJ) {
+                        nk = *reinterpret_cast<const f32x4*>(Ks + (nb * 32 + c32) * P + 8 * (j + 1) + 4 * g);
+                        nv = *reinterpret_cast<const f32x4*>(Vs + (nb * 32 + c32) * P + 8 * (j + 1) + 4 * g);
+                    }
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    s = mfma2(kf[i], qreg[j][i], s);
-                    dp = mfma2(vf[i], greg[j][i], dp);
+                    for (int i = 0; i < 4; ++i) {
+                        s = mfma2(kf[i], qreg[j][i], s);
+                        dp = mfma2(vf[i], greg[j][i], dp);
+                    }
+                    kf = nk;
+                    vf = nv;
+                }
+#pragma unroll
+                for (int j = 0; j + 1 < NJ; ++j) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
                 }
             }
             const bool full = (nn + 31 < a.T) && (!a.causal || nn + 31 <= qlo) &&
@@ -322,11 +350,21 @@ __global__ __launch_bounds__(256, 1) void f32_dq(AttnArgs a) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s[r] = vis(nn + crow(r, g)) ? s[r] : 0.0f;
             }
+            {
+                FV kc = *reinterpret_cast<const FV*>(Ks + (nb * 32 + crow(0, g)) * P + NI * c32);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const FV kc = *reinterpret_cast<const FV*>(Ks + (nb * 32 + crow(r, g)) * P + NI * c32);
+                for (int r = 0; r < 16; ++r) {
+                    FV nc = kc;
+                    if (r + 1 < 16) nc = *reinterpret_cast<const FV*>(Ks + (nb * 32 + crow(r + 1, g)) * P + NI * c32);
 #pragma unroll
-                for (int i = 0; i < NI; ++i) acc[i] = mfma2(fv_get<NI>(kc, i), s[r], acc[i]);
+                    for (int i = 0; i < NI; ++i) acc[i] = mfma2(fv_get<NI>(kc, i), s[r], acc[i]);
+                    kc = nc;
+                }
+#pragma unroll
+                for (int r = 0; r + 1 < 16; ++r) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, NI, 0);
+                }
             }
         }
         // the other buffer was last read one tile ago, before the previous barrier
@@ -334,15 +372,17 @@ __global__ __launch_bounds__(256, 1) void f32_dq(AttnArgs a) {
         __syncthreads();
     }
 
-    if (qi >= a.T) return;
-    float* drow = static_cast<float*>(a.dq) + b * a.dq_sb + h * a.dq_sh + qi * a.dq_st;
+    if (qi < a.T) {
+        float* drow = static_cast<float*>(a.dq) + b * a.dq_sb + h * a.dq_sh + qi * a.dq_st;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        FV out;
+        for (int r = 0; r < 16; ++r) {
+            FV out;
 #pragma unroll
-        for (int i = 0; i < NI; ++i) fv_set<NI>(out, i, acc[i][r] * a.scale);
-        *reinterpret_cast<FV*>(drow + NI * crow(r, g)) = out;
+            for (int i = 0; i < NI; ++i) fv_set<NI>(out, i, acc[i][r] * a.scale);
+            *reinterpret_cast<FV*>(drow + NI * crow(r, g)) = out;
+        }
     }
+  }
 }
 
 // ---------------------------------------------------------------- dK, dV
@@ -370,12 +410,19 @@ __global__ __launch_bounds__(256, 1) void f32_dkdv(AttnArgs a) {
     // key block 0 (seen by every query) first; ids nkb .. nkb + nch - 1 of a unit are the chunks of a
     // split sink tail (see sink_tail)
     const SinkTail tl = a.tail ? sink_tail(a.T, a.window, a.sinks) : SinkTail{0, 0};
-    if (!xcd_map(nkb + tl.nch, 1, a.Hkv * a.B, kblk, rr, kvu)) return;
-    const int chunk = kblk >= nkb ? kblk - nkb : -1;
-    if (chunk >= 0) kblk = 0;
+    // Full-causal: key block i is seen by T - 128 i queries; blocks i and nkb-1-i are taken back to
+    // back so that every workgroup carries the same work.
+    const bool paired = a.causal && a.window == 0;
+    int blk0;
+    if (!xcd_map(paired ? (nkb + 1) / 2 : nkb + tl.nch, 1, a.Hkv * a.B, blk0, rr, kvu)) return;
+    const int chunk = blk0 >= nkb ? blk0 - nkb : -1;
+    if (chunk >= 0) blk0 = 0;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv;
-    const int k0 = kblk * BNK, kw0 = k0 + w * 32, kj = kw0 + c32;
     const float cexp = a.scale * LOG2E;
+    const int npass = (paired && blk0 != nkb - 1 - blk0) ? 2 : 1;
+  for (int pass = 0; pass < npass; ++pass) {
+    kblk = pass == 0 ? blk0 : nkb - 1 - blk0;  // heavy block first
+    const int k0 = kblk * BNK, kw0 = k0 + w * 32, kj = kw0 + c32;
 
     f32x4 kreg[NJ], vreg[NJ];
     {
@@ -462,14 +509,29 @@ __global__ __launch_bounds__(256, 1) void f32_dkdv(AttnArgs a) {
             f32x16 sc, dp;
 #pragma unroll
             for (int r = 0; r < 16; ++r) sc[r] = dp[r] = 0.0f;
+            // One wavefront per SIMD: fragments are read one group of MFMAs ahead, order pinned.
+            {
+                f32x4 qf = *reinterpret_cast<const f32x4*>(Qt + c32 * P + 4 * g);
+                f32x4 gf = *reinterpret_cast<const f32x4*>(Gt + c32 * P + 4 * g);
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                const f32x4 qf = *reinterpret_cast<const f32x4*>(Qt + c32 * P + 8 * j + 4 * g);
-                const f32x4 gf = *reinterpret_cast<const f32x4*>(Gt + c32 * P + 8 * j + 4 * g);
+                for (int j = 0; j < NJ; ++j) {
+                    f32x4 nq = qf, ng = gf;
+                    if (j + 1 < NJ) {
+                        nq = *reinterpret_cast<const f32x4*>(Qt + c32 * P + 8 * (j + 1) + 4 * g);
+                        ng = *reinterpret_cast<const f32x4*>(Gt + c32 * P + 8 * (j + 1) + 4 * g);
+                    }
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    sc = mfma2(qf[i], kreg[j][i], sc);
-                    dp = mfma2(gf[i], vreg[j][i], dp);
+                    for (int i = 0; i < 4; ++i) {
+                        sc = mfma2(qf[i], kreg[j][i], sc);
+                        dp = mfma2(gf[i], vreg[j][i], dp);
+                    }
+                    qf = nq;
+                    gf = ng;
+                }
+#pragma unroll
+                for (int j = 0; j + 1 < NJ; ++j) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
                 }
             }
             const bool full = qhi < a.T && kw0 + 31 < a.T && (!a.causal || kw0 + 31 <= qlo) &&
@@ -495,14 +557,28 @@ __global__ __launch_bounds__(256, 1) void f32_dkdv(AttnArgs a) {
                     dp[r] = v ? dp[r] : 0.0f;
                 }
             }
+            {
+                FV gc = *reinterpret_cast<const FV*>(Gt + crow(0, g) * P + NI * c32);
+                FV qc = *reinterpret_cast<const FV*>(Qt + crow(0, g) * P + NI * c32);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const FV gc = *reinterpret_cast<const FV*>(Gt + crow(r, g) * P + NI * c32);
-                const FV qc = *reinterpret_cast<const FV*>(Qt + crow(r, g) * P + NI * c32);
+                for (int r = 0; r < 16; ++r) {
+                    FV ngc = gc, nqc = qc;
+                    if (r + 1 < 16) {
+                        ngc = *reinterpret_cast<const FV*>(Gt + crow(r + 1, g) * P + NI * c32);
+                        nqc = *reinterpret_cast<const FV*>(Qt + crow(r + 1, g) * P + NI * c32);
+                    }
 #pragma unroll
-                for (int i = 0; i < NI; ++i) {
-                    acc_v[i] = mfma2(fv_get<NI>(gc, i), sc[r], acc_v[i]);
-                    acc_k[i] = mfma2(fv_get<NI>(qc, i), dp[r], acc_k[i]);
+                    for (int i = 0; i < NI; ++i) {
+                        acc_v[i] = mfma2(fv_get<NI>(gc, i), sc[r], acc_v[i]);
+                        acc_k[i] = mfma2(fv_get<NI>(qc, i), dp[r], acc_k[i]);
+                    }
+                    gc = ngc;
+                    qc = nqc;
+                }
+#pragma unroll
+                for (int r = 0; r + 1 < 16; ++r) {
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 2 * NI, 0);
                 }
             }
         }
@@ -511,7 +587,7 @@ __global__ __launch_bounds__(256, 1) void f32_dkdv(AttnArgs a) {
         __syncthreads();
     }
 
-    if (kj >= a.T) return;
+    bool store = kj < a.T;
     float* dkrow = static_cast<float*>(a.dk) + b * a.dk_sb + hk * a.dk_sh + kj * a.dk_st;
     float* dvrow = static_cast<float*>(a.dv) + b * a.dv_sb + hk * a.dv_sh + kj * a.dv_st;
     if (tl.nch > 0 && kblk == 0) {
@@ -522,20 +598,23 @@ __global__ __launch_bounds__(256, 1) void f32_dkdv(AttnArgs a) {
             dkrow = sink_tail_rows(a.tail, kvu, tl.nch, piece, 0, D) + kj * D;
             dvrow = sink_tail_rows(a.tail, kvu, tl.nch, piece, 1, D) + kj * D;
         } else if (chunk >= 0) {
-            return;
+            store = false;
         }
     }
+    if (store) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        FV ok, ov;
+        for (int r = 0; r < 16; ++r) {
+            FV ok, ov;
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            fv_set<NI>(ok, i, acc_k[i][r] * a.scale);
-            fv_set<NI>(ov, i, acc_v[i][r]);
+            for (int i = 0; i < NI; ++i) {
+                fv_set<NI>(ok, i, acc_k[i][r] * a.scale);
+                fv_set<NI>(ov, i, acc_v[i][r]);
+            }
+            *reinterpret_cast<FV*>(dkrow + NI * crow(r, g)) = ok;
+            *reinterpret_cast<FV*>(dvrow + NI * crow(r, g)) = ov;
         }
-        *reinterpret_cast<FV*>(dkrow + NI * crow(r, g)) = ok;
-        *reinterpret_cast<FV*>(dvrow + NI * crow(r, g)) = ov;
     }
+  }
 }
 
 bool aligned_f32(const void* p, int64_t sb, int64_t st, int64_t sh) {
@@ -544,7 +623,9 @@ bool aligned_f32(const void* p, int64_t sb, int64_t st, int64_t sh) {
 
 template <int D>
 int launch_fwd(const AttnArgs& a, hipStream_t st) {
-    const dim3 grid(xcd_grid((a.T + 127) / 128, a.Hq / a.Hkv, a.Hkv * a.B));
+    const int nqb = (a.T + 127) / 128;
+    const bool paired = pair_causal_blocks(nqb, a.Hq * a.B, a.causal, a.window);
+    const dim3 grid(xcd_grid(paired ? (nqb + 1) / 2 : nqb, a.Hq / a.Hkv, a.Hkv * a.B));
     hipLaunchKernelGGL(f32_fwd<D>, grid, dim3(256), 0, st, a);
     PK_HIP(hipGetLastError());
     return PK_OK;
@@ -556,7 +637,9 @@ int launch_bwd(const AttnArgs& a_in, int stages, hipStream_t st) {
     // a tail step is one wavefront's matrix work, as long as a full step's
     if (!sink_tail_pays(a.tail ? sink_tail(a.T, a.window, a.sinks) : SinkTail{0, 0}, a.T, a.window, a.Hkv * a.B, 32, 1, 1.0f))
         a.tail = nullptr;
-    const dim3 dq_grid(xcd_grid((a.T + 127) / 128, a.Hq / a.Hkv, a.Hkv * a.B));
+    const int nqb = (a.T + 127) / 128;
+    const bool paired = pair_causal_blocks(nqb, a.Hq * a.B, a.causal, a.window);
+    const dim3 dq_grid(xcd_grid(paired ? (nqb + 1) / 2 : nqb, a.Hq / a.Hkv, a.Hkv * a.B));
     const bool fused = (stages & PK_BWD_DELTA) && (stages & PK_BWD_DQ);
     if (fused) {  // dQ forms delta itself and runs first; dK/dV reads what it wrote
         hipLaunchKernelGGL((f32_dq<D, true>), dq_grid, dim3(256), 0, st, a);
@@ -566,7 +649,9 @@ int launch_bwd(const AttnArgs& a_in, int stages, hipStream_t st) {
     }
     if (stages & PK_BWD_DKDV) {
         const int nch = a.tail ? sink_tail(a.T, a.window, a.sinks).nch : 0;
-        const dim3 grid(xcd_grid((a.T + 127) / 128 + nch, 1, a.Hkv * a.B));
+        const int nkb = (a.T + 127) / 128;
+        const bool paired = a.causal && a.window == 0;
+        const dim3 grid(xcd_grid(paired ? (nkb + 1) / 2 : nkb + nch, 1, a.Hkv * a.B));
         hipLaunchKernelGGL(f32_dkdv<D>, grid, dim3(256), 0, st, a);
         PK_HIP(hipGetLastError());
         if (nch > 0)
