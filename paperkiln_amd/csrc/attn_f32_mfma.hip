@@ -386,62 +386,62 @@ __global__ __launch_bounds__(256, 1) void f32_dq(AttnArgs a) {
 }
 
 // ---------------------------------------------------------------- dK, dV
-// One workgroup = 4 wavefronts = 128 keys of one (batch, KV head); each wavefront keeps its 32 keys'
-// K and V rows in registers (B operands) and both accumulators, and walks the query tiles that can
-// see the block, 32 queries per step, for every query head of the group. S = Q K^T and dP = dO V^T
-// (lane = key), then dV^T += dO^T P and dK^T += Q^T dS with P and dS taken from the C registers.
-// Q / dO tiles are double-buffered: the next step's rows are fetched into registers before the
-// matrix work of this step and stored behind it, one barrier per step.
+// One workgroup = 8 wavefronts = 128 keys of one (batch, KV head), walking the query tiles that can see
+// the block, 32 queries per step, for every query head of the group. The work of a step is split
+// between two sets of wavefronts, as in the bf16 kernel; wavefront kbw of each role owns keys
+// 32 kbw .. +31 of the block:
+//   role 0 (wavefronts 0-3): S = Q K^T -> P = exp(S*scale - LSE) -> dV^T += dO^T P     (K rows resident)
+//   role 1 (wavefronts 4-7): dP = dO V^T -> dS = P .* (dP - delta) -> dK^T += Q^T dS   (V rows resident)
+// Each role holds one resident operand and one accumulator set, which fits 256 registers: two
+// wavefronts per SIMD, all MFMAs in the plain-register form. P goes from role 0 to role 1 through
+// LDS as it lies in the C registers (both roles have lane = key, element r = query m(r, g)), and
+// role 1 runs one step behind role 0, so one barrier per step orders the hand-over and the
+// three-slot Q / dO ring (role 0 reads step s, role 1 step s-1, step s+1 is being stored).
 template <int D>
-__global__ __launch_bounds__(256, 1) void f32_dkdv(AttnArgs a) {
-    constexpr int NI = D / 32, NJ = D / 8, P = D + 4, BNK = 128;
-    constexpr int CPT = BQ * (D / 4) / 256;  // 16-byte chunks per thread, tensor and step
+__global__ __launch_bounds__(512, 1) void f32_dkdv(AttnArgs a) {
+    constexpr int NI = D / 32, NJ = D / 8, P = D + 4, BNK = 128, NCH = D / 4;
+    constexpr int CPT = (BQ * NCH + 511) / 512;  // 16-byte chunks per thread, tensor and step
     typedef typename FVec<NI>::type FV;
-    __shared__ __attribute__((aligned(16))) float Qs[2][BQ * P];
-    __shared__ __attribute__((aligned(16))) float Gs[2][BQ * P];
-    __shared__ __attribute__((aligned(16))) float nlse_s[2][BQ];
-    __shared__ __attribute__((aligned(16))) float dl_s[2][BQ];
+    __shared__ __attribute__((aligned(16))) float Qs[3][BQ * P];
+    __shared__ __attribute__((aligned(16))) float Gs[3][BQ * P];
+    __shared__ __attribute__((aligned(16))) float Pbuf[2][4][4 * 64 * 4];  // [step parity][kbw][r/4][lane][4]
+    __shared__ __attribute__((aligned(16))) float nlse_s[3][BQ];
+    __shared__ __attribute__((aligned(16))) float dl_s[3][BQ];
 
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int role = w >> 2, kbw = w & 3;
     const int g = lane >> 5, c32 = lane & 31;
     const int nkb = (a.T + BNK - 1) / BNK, rep = a.Hq / a.Hkv;
-    int kblk, rr, kvu;
-    // key block 0 (seen by every query) first; ids nkb .. nkb + nch - 1 of a unit are the chunks of a
-    // split sink tail (see sink_tail)
     const SinkTail tl = a.tail ? sink_tail(a.T, a.window, a.sinks) : SinkTail{0, 0};
-    // Full-causal: key block i is seen by T - 128 i queries; blocks i and nkb-1-i are taken back to
-    // back so that every workgroup carries the same work.
     const bool paired = a.causal && a.window == 0;
-    int blk0;
+    int blk0, rr, kvu;
     if (!xcd_map(paired ? (nkb + 1) / 2 : nkb + tl.nch, 1, a.Hkv * a.B, blk0, rr, kvu)) return;
     const int chunk = blk0 >= nkb ? blk0 - nkb : -1;
     if (chunk >= 0) blk0 = 0;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv;
     const float cexp = a.scale * LOG2E;
     const int npass = (paired && blk0 != nkb - 1 - blk0) ? 2 : 1;
-  for (int pass = 0; pass < npass; ++pass) {
-    kblk = pass == 0 ? blk0 : nkb - 1 - blk0;  // heavy block first
-    const int k0 = kblk * BNK, kw0 = k0 + w * 32, kj = kw0 + c32;
 
-    f32x4 kreg[NJ], vreg[NJ];
+  for (int pass = 0; pass < npass; ++pass) {
+    const int kblk = pass == 0 ? blk0 : nkb - 1 - blk0;  // heavy block first
+    const int k0 = kblk * BNK, kw0 = k0 + kbw * 32, kj = kw0 + c32;
+
+    // the resident operand: K rows for role 0, V rows for role 1 (lane = key, chunk j = d 8j + 4g .. +3)
+    f32x4 kv[NJ];
     {
-        const int t = min(kj, a.T - 1);
-        const float* krow = static_cast<const float*>(a.k) + b * a.k_sb + hk * a.k_sh + t * a.k_st;
-        const float* vrow = static_cast<const float*>(a.v) + b * a.v_sb + hk * a.v_sh + t * a.v_st;
+        const float* src = role == 0 ? static_cast<const float*>(a.k) + b * a.k_sb + hk * a.k_sh
+                                     : static_cast<const float*>(a.v) + b * a.v_sb + hk * a.v_sh;
+        const float* row = src + min(kj, a.T - 1) * (role == 0 ? a.k_st : a.v_st);
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            kreg[j] = *reinterpret_cast<const f32x4*>(krow + 8 * j + 4 * g);
-            vreg[j] = *reinterpret_cast<const f32x4*>(vrow + 8 * j + 4 * g);
-        }
+        for (int j = 0; j < NJ; ++j) kv[j] = *reinterpret_cast<const f32x4*>(row + 8 * j + 4 * g);
     }
-    f32x16 acc_k[NI], acc_v[NI];
+    f32x16 acc[NI];  // dV^T (role 0) or dK^T (role 1)
 #pragma unroll
     for (int i = 0; i < NI; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc_k[i][r] = acc_v[i][r] = 0.0f;
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0.0f;
 
-    // Query tiles that can see keys [k0, k0+127] (src/ops.cpp:960-965 inverted).
     const int khi = min(k0 + BNK, a.T) - 1;
     int qt_lo = a.causal ? k0 / BQ : 0;
     int qt_hi = (a.window > 0 && (k0 >= a.sinks || tl.nch > 0)) ? min(a.T - 1, khi + a.window - 1) / BQ : (a.T - 1) / BQ;
@@ -463,11 +463,12 @@ __global__ __launch_bounds__(256, 1) void f32_dkdv(AttnArgs a) {
         const float* gb = static_cast<const float*>(a.d_o) + b * a.do_sb + h * a.do_sh;
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
-            const int c = threadIdx.x + 256 * i;
-            const int row = c / (D / 4), ch = c % (D / 4);
-            const int t = min(q0 + row, a.T - 1);
-            qr[i] = *reinterpret_cast<const f32x4*>(qb + t * a.q_st + ch * 4);
-            gr[i] = *reinterpret_cast<const f32x4*>(gb + t * a.do_st + ch * 4);
+            const int c = threadIdx.x + 512 * i;
+            if (c < BQ * NCH) {
+                const int t = min(q0 + c / NCH, a.T - 1), ch = c % NCH;
+                qr[i] = *reinterpret_cast<const f32x4*>(qb + t * a.q_st + ch * 4);
+                gr[i] = *reinterpret_cast<const f32x4*>(gb + t * a.do_st + ch * 4);
+            }
         }
         if (threadIdx.x < BQ) {
             const int t = min(q0 + static_cast<int>(threadIdx.x), a.T - 1);
@@ -479,141 +480,128 @@ __global__ __launch_bounds__(256, 1) void f32_dkdv(AttnArgs a) {
     auto commit = [&](int slot) {
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
-            const int c = threadIdx.x + 256 * i;
-            const int row = c / (D / 4), ch = c % (D / 4);
-            *reinterpret_cast<f32x4*>(Qs[slot] + row * P + ch * 4) = qr[i];
-            *reinterpret_cast<f32x4*>(Gs[slot] + row * P + ch * 4) = gr[i];
+            const int c = threadIdx.x + 512 * i;
+            if (c < BQ * NCH) {
+                const int row = c / NCH, ch = c % NCH;
+                *reinterpret_cast<f32x4*>(Qs[slot] + row * P + ch * 4) = qr[i];
+                *reinterpret_cast<f32x4*>(Gs[slot] + row * P + ch * 4) = gr[i];
+            }
         }
         if (threadIdx.x < BQ) {
             nlse_s[slot][threadIdx.x] = lse_r;
             dl_s[slot][threadIdx.x] = dl_r;
         }
     };
+    // wavefront-uniform: is anything of (query tile of step `step`) x (this wavefront's 32 keys) visible?
+    auto tile_live = [&](int step, int& qlo) {
+        qlo = (qt_lo + step % nqt) * BQ;
+        const int qhi = qlo + 31;
+        if (qlo >= a.T || kw0 >= a.T) return false;
+        if (a.causal && kw0 > qhi) return false;
+        if (a.window > 0 && kw0 + 31 + a.window <= qlo && kw0 >= a.sinks) return false;
+        return true;
+    };
 
     if (steps > 0) {
         fetch(0);
         commit(0);
+        if (steps > 1) fetch(1);
     }
     __syncthreads();
-    for (int s = 0; s < steps; ++s) {
-        const int cur = s & 1;
-        if (s + 1 < steps) fetch(s + 1);  // in flight during the matrix work
-        const int qlo = (qt_lo + s % nqt) * BQ, qhi = qlo + 31;
-        // wavefront-uniform: is anything of (this query tile) x (this wavefront's 32 keys) visible?
-        bool live = qlo < a.T && kw0 < a.T;
-        if (a.causal && kw0 > qhi) live = false;
-        if (a.window > 0 && kw0 + 31 + a.window <= qlo && kw0 >= a.sinks) live = false;
-        if (live) {
-            const float* Qt = Qs[cur];
-            const float* Gt = Gs[cur];
-            f32x16 sc, dp;
+    // iteration s: role 0 works on step s, role 1 on step s-1
+    for (int s = 0; s <= steps; ++s) {
+        if (s + 1 < steps) {
+            commit((s + 1) % 3);  // slot last read (by role 1) before the previous barrier
+            if (s + 2 < steps) fetch(s + 2);
+        }
+        const int st = role == 0 ? s : s - 1;
+        int qlo;
+        if (st >= 0 && st < steps && tile_live(st, qlo)) {
+            const float* Qt = Qs[st % 3];
+            const float* Gt = Gs[st % 3];
+            const float* At = role == 0 ? Qt : Gt;  // rows contracted over head_dim: Q for S, dO for dP
+            const float* Ct = role == 0 ? Gt : Qt;  // rows that multiply the C tile: dO for dV, Q for dK
+            float* pb = &Pbuf[st & 1][kbw][lane * 4];
+            f32x16 t;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sc[r] = dp[r] = 0.0f;
-            // One wavefront per SIMD: fragments are read one group of MFMAs ahead, order pinned.
+            for (int r = 0; r < 16; ++r) t[r] = 0.0f;
             {
-                f32x4 qf = *reinterpret_cast<const f32x4*>(Qt + c32 * P + 4 * g);
-                f32x4 gf = *reinterpret_cast<const f32x4*>(Gt + c32 * P + 4 * g);
+                f32x4 af = *reinterpret_cast<const f32x4*>(At + c32 * P + 4 * g);
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
-                    f32x4 nq = qf, ng = gf;
-                    if (j + 1 < NJ) {
-                        nq = *reinterpret_cast<const f32x4*>(Qt + c32 * P + 8 * (j + 1) + 4 * g);
-                        ng = *reinterpret_cast<const f32x4*>(Gt + c32 * P + 8 * (j + 1) + 4 * g);
-                    }
+                    f32x4 nf = af;
+                    if (j + 1 < NJ) nf = *reinterpret_cast<const f32x4*>(At + c32 * P + 8 * (j + 1) + 4 * g);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        sc = mfma2(qf[i], kreg[j][i], sc);
-                        dp = mfma2(gf[i], vreg[j][i], dp);
-                    }
-                    qf = nq;
-                    gf = ng;
-                }
-#pragma unroll
-                for (int j = 0; j + 1 < NJ; ++j) {
-                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+                    for (int i = 0; i < 4; ++i) t = mfma2(af[i], kv[j][i], t);
+                    af = nf;
                 }
             }
-            const bool full = qhi < a.T && kw0 + 31 < a.T && (!a.causal || kw0 + 31 <= qlo) &&
-                              (a.window == 0 || kw0 + a.window > qhi || kw0 + 31 < a.sinks);
-            // lane = key kj; element r = query qlo + crow(r, g): four consecutive queries per r/4
+            if (role == 0) {
+                const int qhi = qlo + 31;
+                const bool full = qhi < a.T && kw0 + 31 < a.T && (!a.causal || kw0 + 31 <= qlo) &&
+                                  (a.window == 0 || kw0 + a.window > qhi || kw0 + 31 < a.sinks);
+                // lane = key kj; element r = query qlo + crow(r, g): four consecutive queries per r/4
 #pragma unroll
-            for (int qd = 0; qd < 4; ++qd) {
-                const f32x4 nl = *reinterpret_cast<const f32x4*>(&nlse_s[cur][qd * 8 + 4 * g]);
-                const f32x4 dl = *reinterpret_cast<const f32x4*>(&dl_s[cur][qd * 8 + 4 * g]);
+                for (int qd = 0; qd < 4; ++qd) {
+                    const f32x4 nl = *reinterpret_cast<const f32x4*>(&nlse_s[st % 3][qd * 8 + 4 * g]);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int r = qd * 4 + e;
-                    const float p = __builtin_amdgcn_exp2f(fmaf(sc[r], cexp, nl[e]));
-                    sc[r] = p;
-                    dp[r] = p * (dp[r] - dl[e]);
+                    for (int e = 0; e < 4; ++e) t[qd * 4 + e] = __builtin_amdgcn_exp2f(fmaf(t[qd * 4 + e], cexp, nl[e]));
                 }
-            }
-            if (!full) {
+                if (!full) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const bool v = vis(qlo + crow(r, g));
-                    sc[r] = v ? sc[r] : 0.0f;
-                    dp[r] = v ? dp[r] : 0.0f;
+                    for (int r = 0; r < 16; ++r) t[r] = vis(qlo + crow(r, g)) ? t[r] : 0.0f;
+                }
+#pragma unroll
+                for (int qd = 0; qd < 4; ++qd) {
+                    const f32x4 pv = {t[qd * 4], t[qd * 4 + 1], t[qd * 4 + 2], t[qd * 4 + 3]};
+                    *reinterpret_cast<f32x4*>(pb + qd * 256) = pv;
+                }
+            } else {
+#pragma unroll
+                for (int qd = 0; qd < 4; ++qd) {
+                    const f32x4 pv = *reinterpret_cast<const f32x4*>(pb + qd * 256);
+                    const f32x4 dl = *reinterpret_cast<const f32x4*>(&dl_s[st % 3][qd * 8 + 4 * g]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) t[qd * 4 + e] = pv[e] * (t[qd * 4 + e] - dl[e]);
                 }
             }
             {
-                FV gc = *reinterpret_cast<const FV*>(Gt + crow(0, g) * P + NI * c32);
-                FV qc = *reinterpret_cast<const FV*>(Qt + crow(0, g) * P + NI * c32);
+                FV cf = *reinterpret_cast<const FV*>(Ct + crow(0, g) * P + NI * c32);
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    FV ngc = gc, nqc = qc;
-                    if (r + 1 < 16) {
-                        ngc = *reinterpret_cast<const FV*>(Gt + crow(r + 1, g) * P + NI * c32);
-                        nqc = *reinterpret_cast<const FV*>(Qt + crow(r + 1, g) * P + NI * c32);
-                    }
+                    FV nf = cf;
+                    if (r + 1 < 16) nf = *reinterpret_cast<const FV*>(Ct + crow(r + 1, g) * P + NI * c32);
 #pragma unroll
-                    for (int i = 0; i < NI; ++i) {
-                        acc_v[i] = mfma2(fv_get<NI>(gc, i), sc[r], acc_v[i]);
-                        acc_k[i] = mfma2(fv_get<NI>(qc, i), dp[r], acc_k[i]);
-                    }
-                    gc = ngc;
-                    qc = nqc;
-                }
-#pragma unroll
-                for (int r = 0; r + 1 < 16; ++r) {
-                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x008, 2 * NI, 0);
+                    for (int i = 0; i < NI; ++i) acc[i] = mfma2(fv_get<NI>(cf, i), t[r], acc[i]);
+                    cf = nf;
                 }
             }
         }
-        // the other buffer was last read one step ago, before the previous barrier
-        if (s + 1 < steps) commit(cur ^ 1);
         __syncthreads();
     }
 
     bool store = kj < a.T;
-    float* dkrow = static_cast<float*>(a.dk) + b * a.dk_sb + hk * a.dk_sh + kj * a.dk_st;
-    float* dvrow = static_cast<float*>(a.dv) + b * a.dv_sb + hk * a.dv_sh + kj * a.dv_st;
+    float* orow = role == 0 ? static_cast<float*>(a.dv) + b * a.dv_sb + hk * a.dv_sh + kj * a.dv_st
+                            : static_cast<float*>(a.dk) + b * a.dk_sb + hk * a.dk_sh + kj * a.dk_st;
     if (tl.nch > 0 && kblk == 0) {
         // a piece of a split sink tail: the sink keys' rows go to the workspace as partial sums
         // (a chunk writes nothing else; the band part writes its other rows as usual)
-        if (w == 0 && kj < a.sinks) {
-            const int piece = chunk >= 0 ? chunk : tl.nch;
-            dkrow = sink_tail_rows(a.tail, kvu, tl.nch, piece, 0, D) + kj * D;
-            dvrow = sink_tail_rows(a.tail, kvu, tl.nch, piece, 1, D) + kj * D;
-        } else if (chunk >= 0) {
+        if (kbw == 0 && kj < a.sinks)
+            orow = sink_tail_rows(a.tail, kvu, tl.nch, chunk >= 0 ? chunk : tl.nch, role == 0 ? 1 : 0, D) + kj * D;
+        else if (chunk >= 0)
             store = false;
-        }
     }
     if (store) {
+        const float sc = role == 0 ? 1.0f : a.scale;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            FV ok, ov;
+            FV out;
 #pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                fv_set<NI>(ok, i, acc_k[i][r] * a.scale);
-                fv_set<NI>(ov, i, acc_v[i][r]);
-            }
-            *reinterpret_cast<FV*>(dkrow + NI * crow(r, g)) = ok;
-            *reinterpret_cast<FV*>(dvrow + NI * crow(r, g)) = ov;
+            for (int i = 0; i < NI; ++i) fv_set<NI>(out, i, acc[i][r] * sc);
+            *reinterpret_cast<FV*>(orow + NI * crow(r, g)) = out;
         }
     }
+    __syncthreads();  // the next pass refills the ring
   }
 }
 
@@ -652,7 +640,7 @@ int launch_bwd(const AttnArgs& a_in, int stages, hipStream_t st) {
         const int nkb = (a.T + 127) / 128;
         const bool paired = a.causal && a.window == 0;
         const dim3 grid(xcd_grid(paired ? (nkb + 1) / 2 : nkb + nch, 1, a.Hkv * a.B));
-        hipLaunchKernelGGL(f32_dkdv<D>, grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(f32_dkdv<D>, grid, dim3(512), 0, st, a);
         PK_HIP(hipGetLastError());
         if (nch > 0)
             if (int rc = launch_sink_tail_reduce(a, st)) return rc;
