@@ -219,6 +219,23 @@ def test_split_sink_tail_against_oracle(oracle, dtype, dk, grad, T, window, sink
         assert rel < (FP32_TOL if dtype == torch.float32 else BF16_TOL)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+def test_split_sink_tail_many_units(oracle, dtype):
+    """The split sink tail with more (batch, KV head) units than XCDs (3 x 3 = 9) and a GQA ratio of 2: every
+    unit's partial rows land in its own part of the workspace and in its own output rows."""
+    B, T, Hq, Hkv, dk, window, sinks = 3, 900, 6, 3, 64, 24, 4
+    q, k, v, d_o = make(B, T, Hq, Hkv, dk, 1.0, 4242)
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
+    want_o, want_lse = oracle.attn_fwd(q, k, v, scale, True, window, sinks)
+    want = (want_o, want_lse) + oracle.attn_bwd(q, k, v, d_o, scale, True, window, sinks)
+    got = run_gpu(q, k, v, d_o, scale, True, window, sinks, dtype, torch.float32)
+    errs = report("split tail, 9 units", got, want)
+    tol = FP32_TOL if dtype == torch.float32 else BF16_TOL
+    assert errs[0] < tol and errs[1] < (FP32_TOL if dtype == torch.float32 else BF16_LSE_TOL)
+    for g_, w_ in zip(got[2:], want[2:]):
+        assert maxabs(g_, w_) < tol * max(1.0, float(np.abs(w_).max()))
+
+
 @pytest.mark.parametrize("dk", [64, 128])
 def test_bf16_large_scores(oracle, dk):
     """Scores spread over +-60 natural-log units (softmax close to one-hot, running max moving by far more than the
