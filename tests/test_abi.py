@@ -40,3 +40,26 @@ def test_argument_errors_do_not_need_a_gpu():
     sh = _lib.AttnShape(1, 8, 2, 2, 4, 1, 0, 0, 0.5, _lib.PK_F32, _lib.PK_F32)
     assert L.pk_attn_fwd(ctypes.byref(sh), ctypes.byref(t), ctypes.byref(t), ctypes.byref(t), ctypes.byref(t), None, None) == 2  # null tensors
     assert L.pk_attn_bwd_workspace_bytes(ctypes.byref(sh)) == 4 * 1 * 2 * 8
+
+
+def test_backward_workspace_follows_the_mask():
+    """pk_attn_bwd_workspace_bytes: delta [B, Hq, T] fp32 for every mask; a band mask with 1..32 sink keys on a
+    sequence longer than key block 0's band adds the partial sink rows of a split sink tail
+    ((chunks of 512 queries + 1) x {dK, dV} x 32 rows x head_dim fp32 per (batch, KV head), 256-byte aligned)."""
+    L = _lib.lib()
+    B, T, Hq, Hkv, dk = 2, 4096, 8, 4, 128
+    delta = 4 * B * Hq * T
+
+    def ws(window, sinks, t=T):
+        sh = _lib.AttnShape(B, t, Hq, Hkv, dk, 1, window, sinks, 0.5, _lib.PK_BF16, _lib.PK_BF16)
+        return L.pk_attn_bwd_workspace_bytes(ctypes.byref(sh))
+
+    assert ws(0, 0) == delta
+    assert ws(256, 0) == delta          # no sink keys: nothing to split
+    assert ws(256, 33) == delta         # more sink keys than one wavefront owns: not split
+    q0 = ((127 + 256 - 1) // 64 + 1) * 64   # first 64-query tile wholly past key block 0's band
+    nch = -(-(T - q0) // 512)
+    assert ws(256, 4) == delta + 4 * B * Hkv * (nch + 1) * 2 * 32 * dk
+    assert ws(256, 4, t=q0) == 4 * B * Hq * q0   # the sequence ends with the band: no tail
+    odd = 4 * B * Hq * 4001                      # delta not a multiple of 256 bytes: the tail starts aligned
+    assert ws(256, 4, t=4001) == odd + (256 - odd % 256) % 256 + 4 * B * Hkv * (-(-(4001 - q0) // 512) + 1) * 2 * 32 * dk
