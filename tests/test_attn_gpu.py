@@ -456,6 +456,47 @@ def test_head_major_and_unaligned_layouts():
             assert maxabs(host(a), host(b)) <= tol_o, f"{name}: {gname}"
 
 
+def test_matrix_core_paths_agree_with_scalar_kernels():
+    """Sixty seeded draws of element type, head size, batch, GQA ratio, length (up to 2500), mask, window and sink
+    count: the matrix-core kernels against the scalar kernels of the same library (forced with a row pitch of
+    dk + 2 elements, which the matrix-core paths decline). Both are held to the oracle elsewhere; this one reaches
+    lengths and unit counts the single-threaded oracle is too slow for."""
+    rng = np.random.default_rng(2025)
+
+    def pitched(x):
+        buf = torch.zeros(x.shape[:-1] + (x.shape[-1] + 2,), dtype=x.dtype, device=x.device)
+        buf[..., :x.shape[-1]] = x
+        return buf[..., :x.shape[-1]]
+
+    for it in range(60):
+        dtype = torch.bfloat16 if rng.integers(0, 2) else torch.float32
+        dk = int(rng.choice([64, 128] if dtype == torch.bfloat16 else [32, 64, 128]))
+        B, Hkv, rep = (int(rng.integers(1, 4)) for _ in range(3))
+        T = int(rng.choice([1, 3, 63, 65, 129, 255, 257, 333, 700, 1025, 1500, 2047, 2500]))
+        causal = bool(rng.integers(0, 5) > 0)
+        window = int(rng.choice([0, 0, 1, 17, 64, 100, 300, 5000])) if causal else 0
+        sinks = int(rng.choice([0, 1, 3, 32, 33, 100, 200])) if window else 0
+        gen = torch.Generator(device="cuda").manual_seed(1000 + it)
+        mk = lambda h: (torch.randn((B, T, h, dk), generator=gen, device="cuda") * 0.8).to(dtype)
+        q, k, v, d_o = mk(Hkv * rep), mk(Hkv), mk(Hkv), mk(Hkv * rep)
+        scale = float(1 / np.sqrt(dk))
+        tag = f"draw {it}: {dtype} B={B} T={T} Hq={Hkv * rep} Hkv={Hkv} dk={dk} causal={causal} w={window} s={sinks}"
+        print("\n  " + tag, flush=True)
+        o, lse = ops.attn_fwd(q, k, v, scale, causal, window, sinks)
+        grads = ops.attn_bwd(q, k, v, o, lse, d_o, scale, causal, window, sinks, grad_dtype=torch.float32)
+        o2, lse2 = ops.attn_fwd(pitched(q), pitched(k), pitched(v), scale, causal, window, sinks)
+        grads2 = ops.attn_bwd(pitched(q), pitched(k), pitched(v), pitched(o2), lse2, pitched(d_o), scale, causal,
+                              window, sinks, grad_dtype=torch.float32)
+        torch.cuda.synchronize()
+        tol, tol_lse = (BF16_TOL, BF16_LSE_TOL) if dtype == torch.bfloat16 else (FP32_TOL, FP32_TOL)
+        for name, a, b in (("O", o, o2), ("LSE", lse, lse2), ("dQ", grads[0], grads2[0]), ("dK", grads[1], grads2[1]),
+                           ("dV", grads[2], grads2[2])):
+            a, b = host(a.float()), host(b.float())
+            assert np.isfinite(a).all(), f"{tag}: {name}"
+            bar = (tol_lse if name == "LSE" else tol) * max(1.0, float(np.abs(b).max()))
+            assert maxabs(a, b) <= bar, f"{tag}: {name} {maxabs(a, b):.3e} > {bar:.3e}"
+
+
 def test_reference_op_surface(oracle):
     """ops.fused_attention / ops.swa_attention: per-head [rows, dk] matrices, seq_len stacking,
     autograd through the O+LSE-only node, and the reference's error behaviour."""
