@@ -497,6 +497,29 @@ def test_matrix_core_paths_agree_with_scalar_kernels():
             assert maxabs(a, b) <= bar, f"{tag}: {name} {maxabs(a, b):.3e} > {bar:.3e}"
 
 
+@pytest.mark.parametrize("dtype,T", [(torch.bfloat16, 65536), (torch.float32, 16384)], ids=["bf16_T65536", "fp32_T16384"])
+def test_prefix_property_both_element_types(dtype, T):
+    """Causal attention over a long sequence: O, LSE and dQ of the first 1024 rows depend on the first 1024 tokens
+    only, so they must match a run over that prefix alone (different tile schedule, hence the element type's bar,
+    not bitwise); every output of the long run is finite."""
+    B, H, dk, Tp = 1, 2, 128, 1024
+    gen = torch.Generator(device="cuda").manual_seed(77)
+    q, k, v, d_o = ((torch.randn((B, T, H, dk), generator=gen, device="cuda") * 0.5).to(dtype) for _ in range(4))
+    scale = float(1 / np.sqrt(dk))
+    o, lse = ops.attn_fwd(q, k, v, scale, True)
+    dq, dk_, dv = ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, grad_dtype=torch.float32)
+    qp, kp, vp, gp = (x[:, :Tp].contiguous() for x in (q, k, v, d_o))
+    op, lsep = ops.attn_fwd(qp, kp, vp, scale, True)
+    dqp, _, _ = ops.attn_bwd(qp, kp, vp, op, lsep, gp, scale, True, grad_dtype=torch.float32)
+    torch.cuda.synchronize()
+    for x in (o, lse, dq, dk_, dv):
+        assert torch.isfinite(x).all()
+    tol, tol_lse = (BF16_TOL, BF16_LSE_TOL) if dtype == torch.bfloat16 else (FP32_TOL, FP32_TOL)
+    assert maxabs(host(o[:, :Tp].float()), host(op.float())) <= tol
+    assert maxabs(host(lse[:, :, :Tp]), host(lsep)) <= tol_lse
+    assert maxabs(host(dq[:, :Tp]), host(dqp)) <= tol * max(1.0, float(dqp.abs().max()))
+
+
 def test_reference_op_surface(oracle):
     """ops.fused_attention / ops.swa_attention: per-head [rows, dk] matrices, seq_len stacking,
     autograd through the O+LSE-only node, and the reference's error behaviour."""
