@@ -114,7 +114,7 @@ int pk_attn_bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_ten
  * the earlier work that used the block), which is how one model's tape runs.
  * Memory that several streams touch must come from elsewhere. */
 int pk_alloc(size_t bytes, void** out);
-int pk_free(void* p);
+int pk_free(void* p);   /* PK_ERR_ARGUMENT for a pointer pk_alloc did not return or that was freed before */
 size_t pk_live_bytes(void);
 size_t pk_peak_bytes(void);
 void pk_reset_peak(void);
@@ -143,7 +143,12 @@ typedef struct pk_llama_stats {
                                                optimizer state and bf16 parameter shadows excluded */
 } pk_llama_stats;
 
-/* Llama::Llama(cfg, seed): N(0, 0.02) Linear / Embedding weights, unit norm gains. */
+/* Llama::Llama(cfg, seed): N(0, 0.02) Linear / Embedding weights, unit norm gains.
+ * A model owns its tape state (element type, stream, parameter shadows): models of different compute_dtype
+ * may live side by side, and each may be driven from a host thread of its own on a stream of its own; calls
+ * on ONE model are serialised by a lock inside it. pk_llama_adamw_step and the parameter accessors run on
+ * the stream of the model's last pk_llama_loss_backward. The byte counters (pk_live_bytes, pk_peak_bytes,
+ * pk_llama_stats) are process-wide, so they are only meaningful while one model steps at a time. */
 int pk_llama_create(const pk_llama_config* cfg, unsigned seed, void** handle);
 int pk_llama_destroy(void* handle);
 int pk_llama_num_params(void* handle);
@@ -161,6 +166,10 @@ int pk_llama_loss_backward(void* handle, const int* host_ids, const int* host_ta
 /* ops::clip_grad_norm (src/ops.cpp:1046-1064; skipped when max_norm <= 0) then nn::AdamW::step (src/nn.cpp:301-321). */
 int pk_llama_adamw_step(void* handle, float lr, float b1, float b2, float eps, float wd, float max_norm,
                         float* total_norm);
+/* Rows of the tied head (llama.cpp:88 + ops::cross_entropy, src/ops.cpp:350-376) evaluated at a time when
+ * fused_head = 1: the [n, vocab] logits the reference materialises exist here one [rows, vocab] chunk at a
+ * time. Default 2048; smaller chunks lower the activation peak, larger ones run fewer, larger GEMMs. */
+int pk_llama_set_head_chunk(void* handle, int64_t rows);
 
 /* ---- block operators -------------------------------------------------------
  * The operators of one Llama block as single calls on device memory: row-major

@@ -50,6 +50,7 @@ EXPORTS = ["pk_last_error", "pk_init", "pk_attn_fwd", "pk_attn_bwd_workspace_byt
            "pk_alloc", "pk_free", "pk_live_bytes", "pk_peak_bytes", "pk_reset_peak", "pk_trim",
            "pk_llama_create", "pk_llama_destroy", "pk_llama_num_params", "pk_llama_param_info", "pk_llama_set_param",
            "pk_llama_get_param", "pk_llama_get_grad", "pk_llama_loss_backward", "pk_llama_adamw_step",
+           "pk_llama_set_head_chunk",
            "pk_op_add", "pk_op_mul", "pk_op_scale", "pk_op_axpy", "pk_op_fill", "pk_op_silu_fwd", "pk_op_silu_bwd", "pk_op_silu_mul_fwd", "pk_op_silu_mul_bwd",
            "pk_op_rmsnorm_fwd", "pk_op_rmsnorm_bwd", "pk_op_rope", "pk_op_embedding_fwd", "pk_op_embedding_bwd",
            "pk_op_cross_entropy", "pk_op_adamw", "pk_op_sumsq", "pk_op_gemm"]
@@ -90,6 +91,7 @@ def lib() -> C.CDLL:
         L.pk_llama_loss_backward.argtypes = [C.c_void_p, i32p, i32p, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int,
                                              f32p, C.POINTER(LlamaStats), C.c_void_p]
         L.pk_llama_adamw_step.argtypes = [C.c_void_p] + [C.c_float] * 6 + [f32p]
+        L.pk_llama_set_head_chunk.argtypes = [C.c_void_p, C.c_int64]
         vp, i64, ci, cf = C.c_void_p, C.c_int64, C.c_int, C.c_float
         L.pk_op_add.argtypes = [vp, vp, vp, i64, ci, vp]
         L.pk_op_mul.argtypes = [vp, vp, vp, i64, ci, vp]

@@ -29,7 +29,10 @@ struct BF16 {
     }
     __device__ static void st(void* p, int64_t i, float x) {
         uint32_t u = __float_as_uint(x);
-        u += 0x7FFFu + ((u >> 16) & 1u);  // round to nearest even
+        if ((u & 0x7FFFFFFFu) > 0x7F800000u)
+            u |= 0x00400000u;  // NaN stays NaN: no rounding carry into the exponent
+        else
+            u += 0x7FFFu + ((u >> 16) & 1u);  // round to nearest even
         static_cast<uint16_t*>(p)[i] = static_cast<uint16_t>(u >> 16);
     }
 };

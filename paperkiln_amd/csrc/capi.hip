@@ -32,6 +32,8 @@ int check_shape(const pk_attn_shape* s, const char* who) {
         return fail(PK_ERR_SHAPE, std::string(who) + ": shape mismatch (non-positive dimension)");
     if (s->Hq % s->Hkv != 0)
         return fail(PK_ERR_SHAPE, std::string(who) + ": shape mismatch (Hq not a multiple of Hkv)");
+    if (s->T > (1 << 24))  // index + window sums stay far inside 32 bits
+        return fail(PK_ERR_SHAPE, std::string(who) + ": more than 2^24 tokens per sequence not supported");
     if (s->dk > 256) return fail(PK_ERR_SHAPE, std::string(who) + ": head_dim > 256 not supported");
     if (s->window < 0 || s->sinks < 0)
         return fail(PK_ERR_ARGUMENT, std::string(who) + ": window and sinks must be >= 0");
@@ -44,10 +46,26 @@ int check_shape(const pk_attn_shape* s, const char* who) {
 
 bool bad(const pk_tensor4* t) { return !t || !t->ptr; }
 
+// The mask the kernels run with. The reference takes size_t arguments and defines a window that covers the
+// whole sequence as plain causal attention (tests/test_swa.cpp:47-57), so "window = INT32_MAX" is a legal way
+// to ask for no band; the kernels add the window to key and query indices in 32-bit arithmetic, so the values
+// are brought into [0, T] here, once, and every later use (tile skipping, sink tail, workspace size) sees these.
+struct Mask {
+    int window, sinks;
+};
+Mask effective_mask(const pk_attn_shape* s) {
+    Mask m = {s->window, s->sinks};
+    if (m.window >= s->T) m.window = 0, m.sinks = 0;  // every key at or before the query is inside the window
+    if (m.window == 0) m.sinks = 0;                    // sinks only matter under a band
+    if (m.sinks > s->T) m.sinks = s->T;
+    return m;
+}
+
 // workspace = delta [B, Hq, T] fp32, then (band mask with 1..32 sink keys only) the sink-tail partial rows
 size_t delta_bytes(const pk_attn_shape* s) { return sizeof(float) * static_cast<size_t>(s->B) * s->Hq * s->T; }
 size_t tail_bytes(const pk_attn_shape* s) {
-    const SinkTail t = sink_tail(s->T, s->window, s->sinks);
+    const Mask m = effective_mask(s);
+    const SinkTail t = sink_tail(s->T, m.window, m.sinks);
     if (t.nch == 0) return 0;
     const size_t pad = (256 - delta_bytes(s) % 256) % 256;
     return pad + sink_tail_bytes(s->B * s->Hkv, t.nch, s->dk);
@@ -61,7 +79,8 @@ void fill_common(AttnArgs& a, const pk_attn_shape* s, const pk_tensor4* q, const
     a.v = v->ptr; a.v_sb = v->stride_b; a.v_st = v->stride_t; a.v_sh = v->stride_h;
     a.o = o->ptr; a.o_sb = o->stride_b; a.o_st = o->stride_t; a.o_sh = o->stride_h;
     a.B = s->B; a.T = s->T; a.Hq = s->Hq; a.Hkv = s->Hkv; a.dk_dim = s->dk;
-    a.causal = s->causal != 0; a.window = s->window; a.sinks = s->sinks;
+    const Mask m = effective_mask(s);
+    a.causal = s->causal != 0; a.window = m.window; a.sinks = m.sinks;
     a.scale = s->scale;
     a.grad_f32 = s->grad_dtype == PK_F32;
 }

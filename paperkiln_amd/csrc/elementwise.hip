@@ -3,6 +3,7 @@
 // (paperkiln src/cuda_ops.cu:76-381, write-through host->device->host per call)
 // but are device-resident: operands and results stay in HBM between ops.
 // Formulas are those of the CPU tape in src/ops.cpp, cited per kernel.
+#include <hipcub/hipcub.hpp>
 #include <rocblas/rocblas.h>
 
 #include <map>
@@ -17,7 +18,14 @@
 namespace pk {
 
 void hip_check(hipError_t e, const char* what) {
-    if (e != hipSuccess) throw std::runtime_error(std::string("HIP error: ") + hipGetErrorString(e) + " in " + what);
+    if (e == hipSuccess) return;
+    const std::string msg = std::string("HIP error: ") + hipGetErrorString(e) + " in " + what;
+    throw Error(e == hipErrorOutOfMemory ? PK_ERR_OOM : PK_ERR_HIP, msg);
+}
+int status_of(const std::exception& e) {
+    if (const Error* pe = dynamic_cast<const Error*>(&e)) return pe->code;
+    if (dynamic_cast<const std::bad_alloc*>(&e)) return PK_ERR_OOM;
+    return PK_ERR_ARGUMENT;
 }
 #define HIPCHK(x) ::pk::hip_check((x), #x)
 
@@ -25,9 +33,20 @@ void hip_check(hipError_t e, const char* what) {
 namespace {
 struct Pool {
     std::mutex mu;
-    std::multimap<size_t, void*> free_blocks;         // size -> block
+    // cached blocks by (stream that last used them, size): a block is handed out again without waiting for the
+    // GPU, which is only safe for work queued behind its last use, i.e. on that same stream
+    std::multimap<std::pair<hipStream_t, size_t>, void*> free_blocks;
     std::unordered_map<void*, size_t> sizes;          // every block handed out or cached
+    std::unordered_map<void*, bool> handed_out;       // blocks a caller holds right now
     size_t live = 0, peak = 0, reserved = 0;
+    void release_cached() {  // give every cached block back to the driver (hipFree waits for the device)
+        for (auto& kv : free_blocks) {
+            (void)hipFree(kv.second);
+            reserved -= kv.first.second;
+            sizes.erase(kv.second);
+        }
+        free_blocks.clear();
+    }
 };
 Pool& pool() {
     static Pool p;
@@ -38,64 +57,76 @@ size_t round_up(size_t n) {
     if (n < (1u << 20)) return (n + 511) & ~size_t(511);
     return (n + ((1u << 20) - 1)) & ~size_t((1u << 20) - 1);  // 1 MiB granules above 1 MiB
 }
-thread_local hipStream_t g_stream = nullptr;  // per host thread: the block operators of the C ABI set it around each call
 }  // namespace
-
-hipStream_t tape_stream() { return g_stream; }
-void set_tape_stream(hipStream_t s) { g_stream = s; }
 
 void* dev_alloc(size_t bytes) {
     const size_t n = round_up(bytes);
+    const hipStream_t st = tape_stream();
     Pool& P = pool();
     std::lock_guard<std::mutex> lk(P.mu);
     void* p = nullptr;
-    auto it = P.free_blocks.lower_bound(n);
-    if (it != P.free_blocks.end() && it->first <= n + n / 4 + 512) {  // reuse only near-fitting blocks
+    auto it = P.free_blocks.lower_bound({st, n});
+    if (it != P.free_blocks.end() && it->first.first == st && it->first.second <= n + n / 4 + 512) {  // near-fitting only
         p = it->second;
-        P.live += it->first;
+        P.live += it->first.second;
         P.free_blocks.erase(it);
     } else {
         hipError_t e = hipMalloc(&p, n);
         if (e != hipSuccess) {  // give cached blocks back and retry once
-            for (auto& kv : P.free_blocks) {
-                (void)hipFree(kv.second);
-                P.reserved -= kv.first;
-                P.sizes.erase(kv.second);
+            (void)hipGetLastError();
+            P.release_cached();
+            e = hipMalloc(&p, n);
+            if (e != hipSuccess) {
+                (void)hipGetLastError();
+                throw Error(PK_ERR_OOM, "out of device memory: hipMalloc of " + std::to_string(n) + " bytes failed (" +
+                                            hipGetErrorString(e) + ")");
             }
-            P.free_blocks.clear();
-            hip_check(hipMalloc(&p, n), "hipMalloc");
         }
         P.sizes[p] = n;
         P.reserved += n;
         P.live += n;
     }
+    P.handed_out[p] = true;
     if (P.live > P.peak) P.peak = P.live;
     return p;
 }
 
-void dev_free(void* p) {
-    if (!p) return;
+bool dev_free(void* p) {
+    if (!p) return true;
     Pool& P = pool();
     std::lock_guard<std::mutex> lk(P.mu);
-    auto it = P.sizes.find(p);
-    if (it == P.sizes.end()) return;
-    P.live -= it->second;
-    P.free_blocks.emplace(it->second, p);
+    auto held = P.handed_out.find(p);
+    if (held == P.handed_out.end()) return false;
+    P.handed_out.erase(held);
+    const size_t n = P.sizes.at(p);
+    P.live -= n;
+    P.free_blocks.emplace(std::make_pair(tape_stream(), n), p);
+    return true;
 }
 
-size_t dev_live_bytes() { return pool().live; }
-size_t dev_peak_bytes() { return pool().peak; }
-void dev_reset_peak() { pool().peak = pool().live; }
+bool dev_owns(const void* p) {
+    Pool& P = pool();
+    std::lock_guard<std::mutex> lk(P.mu);
+    return P.handed_out.count(const_cast<void*>(p)) != 0;
+}
+
+size_t dev_live_bytes() {
+    std::lock_guard<std::mutex> lk(pool().mu);
+    return pool().live;
+}
+size_t dev_peak_bytes() {
+    std::lock_guard<std::mutex> lk(pool().mu);
+    return pool().peak;
+}
+void dev_reset_peak() {
+    std::lock_guard<std::mutex> lk(pool().mu);
+    pool().peak = pool().live;
+}
 void dev_trim() {
     Pool& P = pool();
     std::lock_guard<std::mutex> lk(P.mu);
     (void)hipDeviceSynchronize();
-    for (auto& kv : P.free_blocks) {
-        (void)hipFree(kv.second);
-        P.reserved -= kv.first;
-        P.sizes.erase(kv.second);
-    }
-    P.free_blocks.clear();
+    P.release_cached();
 }
 
 // ---- element access --------------------------------------------------------
@@ -106,6 +137,10 @@ __device__ inline float ldf(const uint16_t* p, int64_t i) { return __uint_as_flo
 __device__ inline void stf(float* p, int64_t i, float x) { p[i] = x; }
 __device__ inline void stf(uint16_t* p, int64_t i, float x) {
     uint32_t u = __float_as_uint(x);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) {  // NaN: keep it one (the rounding carry could turn it into an infinity)
+        p[i] = static_cast<uint16_t>((u >> 16) | 0x0040u);
+        return;
+    }
     u += 0x7FFFu + ((u >> 16) & 1u);  // round to nearest even
     p[i] = static_cast<uint16_t>(u >> 16);
 }
@@ -510,10 +545,28 @@ __global__ void emb_fwd(const float* table, const int* ids, T* y, int64_t n, int
     for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n * d; i += static_cast<int64_t>(gridDim.x) * NT)
         stf(y, i, table[static_cast<int64_t>(ids[i / d]) * d + i % d]);
 }
+// Scatter-add without atomics. The rows are visited in the order of a stable sort by id (sorted_id, row_of), so
+// the rows that share an id are neighbours, in ascending row order. The block at the head of such a run adds the
+// run's rows one after another and is the only writer of that table row; every other block leaves at once. The
+// sum for an id is therefore formed in the reference's own order (rows ascending, src/ops.cpp:338-347) and is
+// the same on every run.
+__global__ void iota_i32(int* x, int n) {
+    const int i = blockIdx.x * NT + threadIdx.x;
+    if (i < n) x[i] = i;
+}
 template <typename T>
-__global__ void emb_bwd(const T* dy, const int* ids, float* dtable, int64_t n, int d) {
-    for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n * d; i += static_cast<int64_t>(gridDim.x) * NT)
-        atomicAdd(dtable + static_cast<int64_t>(ids[i / d]) * d + i % d, ldf(dy, i));
+__global__ void emb_bwd_runs(const T* dy, const int* sorted_id, const int* row_of, float* dtable, int n, int d) {
+    const int p = blockIdx.x;
+    const int id = sorted_id[p];
+    if (p > 0 && sorted_id[p - 1] == id) return;
+    int end = p + 1;
+    while (end < n && sorted_id[end] == id) ++end;
+    for (int c = threadIdx.x; c < d; c += NT) {
+        float* dst = dtable + static_cast<int64_t>(id) * d + c;
+        float acc = *dst;
+        for (int r = p; r < end; ++r) acc += ldf(dy, static_cast<int64_t>(row_of[r]) * d + c);
+        *dst = acc;
+    }
 }
 
 __device__ inline float block_reduce(float x, bool is_max, float* sh) {
@@ -883,9 +936,21 @@ void k_embedding_fwd(const Tensor& table, const int* ids, const Tensor& y) {
     post();
 }
 void k_embedding_bwd(const Tensor& dy, const int* ids, const Tensor& dtable) {
-    PK_DISPATCH1(T, dy.dtype, hipLaunchKernelGGL((emb_bwd<T>), ew_grid(dy.numel()), dim3(NT), 0, tape_stream(),
-                                                 static_cast<const T*>(dy.ptr()), ids, static_cast<float*>(dtable.ptr()),
-                                                 dy.rows, static_cast<int>(dy.cols)));
+    if (dy.rows > (1 << 30)) shape_fail("embedding: more than 2^30 rows");
+    const int n = static_cast<int>(dy.rows), d = static_cast<int>(dy.cols);
+    const hipStream_t st = tape_stream();
+    Buffer rows_in(sizeof(int) * n), rows_out(sizeof(int) * n), ids_out(sizeof(int) * n);
+    int* const r_in = static_cast<int*>(rows_in.p);
+    int* const r_out = static_cast<int*>(rows_out.p);
+    int* const i_out = static_cast<int*>(ids_out.p);
+    hipLaunchKernelGGL(iota_i32, dim3((n + NT - 1) / NT), dim3(NT), 0, st, r_in, n);
+    size_t tmp_bytes = 0;  // radix sort is stable: equal ids keep their rows in ascending order
+    HIPCHK(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, ids, i_out, r_in, r_out, n, 0, 32, st));
+    Buffer tmp(tmp_bytes ? tmp_bytes : 16);
+    HIPCHK(hipcub::DeviceRadixSort::SortPairs(tmp.p, tmp_bytes, ids, i_out, r_in, r_out, n, 0, 32, st));
+    PK_DISPATCH1(T, dy.dtype, hipLaunchKernelGGL((emb_bwd_runs<T>), dim3(n), dim3(NT), 0, st,
+                                                 static_cast<const T*>(dy.ptr()), i_out, r_out,
+                                                 static_cast<float*>(dtable.ptr()), n, d));
     post();
 }
 void k_ce_rows(const Tensor& logits, const int* targets, float gscale, float* nll_rows) {

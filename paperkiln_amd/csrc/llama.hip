@@ -6,6 +6,7 @@
 // receipt here is bytes from the allocator's high-water mark, not a node count.
 #include <cmath>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -65,6 +66,11 @@ struct Block {
 
 struct Model {
     pk_llama_config cfg;
+    // The model's own tape state (stream, element type, parameter shadows) and the lock that keeps two host
+    // threads from running the same model at once; every C entry holds both for the length of the call.
+    TapeContext ctx;
+    std::mutex mu;
+    int64_t head_chunk_rows = 2048;  // rows of the tied head evaluated at a time (linear_cross_entropy)
     Var embed, norm_w;
     std::vector<Block> blocks;
     std::vector<std::pair<std::string, Var>> named;
@@ -78,7 +84,7 @@ struct Model {
     void reg(const std::string& name, const Var& p) { named.emplace_back(name, p); }
 
     Model(const pk_llama_config& c, unsigned seed) : cfg(c) {
-        if (c.d % c.n_heads != 0) throw std::runtime_error("llama: d must divide by n_heads");
+        if (c.d % c.n_heads != 0) shape_fail("llama: d must divide by n_heads");
         const int64_t d = c.d, ff = c.d_ff;
         auto lin = [&](int64_t in, int64_t out, unsigned s) {
             return make_param(in, out, randn_host(static_cast<uint64_t>(s) * 7919u + 1u, in * out, 0.02f));
@@ -168,7 +174,7 @@ struct Model {
     // Llama::forward (llama.cpp:71-89) up to the final norm; positions restart per sequence.
     Var hidden(const std::shared_ptr<Buffer>& ids, int64_t n, int64_t seq_len) const {
         const int64_t sl = seq_len == 0 ? n : seq_len;
-        if (n % sl != 0) throw std::runtime_error("ids not a multiple of seq_len");
+        if (n % sl != 0) shape_fail("ids not a multiple of seq_len");
         std::vector<int> pos(n);
         for (int64_t i = 0; i < n; ++i) pos[i] = static_cast<int>(i % sl);
         auto pos_dev = ints_to_dev(pos.data(), pos.size());
@@ -195,8 +201,23 @@ int guarded(F&& f) {
     } catch (const std::exception& e) {
         g_llama_err = e.what();
         set_error(g_llama_err);
-        return PK_ERR_ARGUMENT;
+        return status_of(e);
     }
+}
+
+Model* model_of(void* handle) {
+    if (!handle) throw Error(PK_ERR_ARGUMENT, "null model handle");
+    return static_cast<Model*>(handle);
+}
+// Runs f(model) as the model's own tape: its lock held, its context current on this thread.
+template <typename F>
+int with_model(void* handle, F&& f) {
+    return guarded([&] {
+        Model* m = model_of(handle);
+        std::lock_guard<std::mutex> lk(m->mu);
+        ContextScope scope(m->ctx);
+        f(m);
+    });
 }
 
 }  // namespace
@@ -207,10 +228,15 @@ using namespace pk;
 extern "C" {
 
 int pk_alloc(size_t bytes, void** out) {
-    return guarded([&] { *out = dev_alloc(bytes); });
+    return guarded([&] {
+        if (!out) throw Error(PK_ERR_ARGUMENT, "pk_alloc: null result pointer");
+        *out = dev_alloc(bytes);
+    });
 }
 int pk_free(void* p) {
-    return guarded([&] { dev_free(p); });
+    return guarded([&] {
+        if (!dev_free(p)) throw Error(PK_ERR_ARGUMENT, "pk_free: not a pointer pk_alloc returned (or already freed)");
+    });
 }
 size_t pk_live_bytes(void) { return dev_live_bytes(); }
 size_t pk_peak_bytes(void) { return dev_peak_bytes(); }
@@ -219,44 +245,62 @@ void pk_trim(void) { dev_trim(); }
 
 int pk_llama_create(const pk_llama_config* cfg, unsigned seed, void** handle) {
     return guarded([&] {
-        if (!cfg || !handle) throw std::runtime_error("pk_llama_create: null argument");
+        if (!cfg || !handle) throw Error(PK_ERR_ARGUMENT, "pk_llama_create: null argument");
+        // the parameters are created under a context of the model's element type, which the model then keeps
+        TapeContext ctx;
+        ContextScope scope(ctx);
         set_compute_dtype(cfg->compute_dtype);
-        *handle = new Model(*cfg, seed);
+        Model* m = new Model(*cfg, seed);
+        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+        m->ctx = ctx;
+        *handle = m;
     });
 }
 int pk_llama_destroy(void* h) {
-    return guarded([&] { delete static_cast<Model*>(h); });
-}
-int pk_llama_num_params(void* h) { return static_cast<int>(static_cast<Model*>(h)->named.size()); }
-int pk_llama_param_info(void* h, int i, char* name, size_t name_len, int64_t* rows, int64_t* cols) {
     return guarded([&] {
+        if (!h) return;
         Model* m = static_cast<Model*>(h);
-        if (i < 0 || i >= static_cast<int>(m->named.size())) throw std::runtime_error("parameter index out of range");
+        {
+            std::lock_guard<std::mutex> lk(m->mu);
+            ContextScope scope(m->ctx);
+            hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+            m->ctx.shadows.reset();  // the shadows' memory goes back tagged with the model's stream
+        }
+        TapeContext last = m->ctx;  // parameters and slabs are freed under the model's stream as well
+        ContextScope scope(last);
+        delete m;
+    });
+}
+int pk_llama_num_params(void* h) { return h ? static_cast<int>(static_cast<Model*>(h)->named.size()) : -1; }
+int pk_llama_param_info(void* h, int i, char* name, size_t name_len, int64_t* rows, int64_t* cols) {
+    return with_model(h, [&](Model* m) {
+        if (i < 0 || i >= static_cast<int>(m->named.size())) throw Error(PK_ERR_ARGUMENT, "parameter index out of range");
         if (name && name_len) std::snprintf(name, name_len, "%s", m->named[i].first.c_str());
-        *rows = m->named[i].second->data.rows;
-        *cols = m->named[i].second->data.cols;
+        if (rows) *rows = m->named[i].second->data.rows;
+        if (cols) *cols = m->named[i].second->data.cols;
     });
 }
 int pk_llama_set_param(void* h, int i, const float* host) {
-    return guarded([&] {
-        Model* m = static_cast<Model*>(h);
-        const Tensor& t = m->named.at(i).second->data;
+    return with_model(h, [&](Model* m) {
+        if (i < 0 || i >= static_cast<int>(m->named.size()) || !host) throw Error(PK_ERR_ARGUMENT, "parameter index out of range or null data");
+        const Tensor& t = m->named[i].second->data;
+        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
         hip_check(hipMemcpy(t.ptr(), host, sizeof(float) * t.numel(), hipMemcpyHostToDevice), "hipMemcpy");
         invalidate_shadows();
     });
 }
 int pk_llama_get_param(void* h, int i, float* host) {
-    return guarded([&] {
-        Model* m = static_cast<Model*>(h);
-        const Tensor& t = m->named.at(i).second->data;
+    return with_model(h, [&](Model* m) {
+        if (i < 0 || i >= static_cast<int>(m->named.size()) || !host) throw Error(PK_ERR_ARGUMENT, "parameter index out of range or null data");
+        const Tensor& t = m->named[i].second->data;
         hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
         hip_check(hipMemcpy(host, t.ptr(), sizeof(float) * t.numel(), hipMemcpyDeviceToHost), "hipMemcpy");
     });
 }
 int pk_llama_get_grad(void* h, int i, float* host) {
-    return guarded([&] {
-        Model* m = static_cast<Model*>(h);
-        const Var& p = m->named.at(i).second;
+    return with_model(h, [&](Model* m) {
+        if (i < 0 || i >= static_cast<int>(m->named.size()) || !host) throw Error(PK_ERR_ARGUMENT, "parameter index out of range or null data");
+        const Var& p = m->named[i].second;
         hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
         if (p->grad.empty())
             std::memset(host, 0, sizeof(float) * p->data.numel());
@@ -264,13 +308,19 @@ int pk_llama_get_grad(void* h, int i, float* host) {
             hip_check(hipMemcpy(host, p->grad.ptr(), sizeof(float) * p->data.numel(), hipMemcpyDeviceToHost), "hipMemcpy");
     });
 }
+int pk_llama_set_head_chunk(void* h, int64_t rows) {
+    return with_model(h, [&](Model* m) {
+        if (rows <= 0) throw Error(PK_ERR_ARGUMENT, "pk_llama_set_head_chunk: rows must be positive");
+        m->head_chunk_rows = rows;
+    });
+}
 
 int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets, int64_t n, int64_t seq_len,
                            int checkpoint_blocks, int do_backward, int fused_head, float* loss, pk_llama_stats* stats,
                            void* stream) {
-    return guarded([&] {
-        Model* m = static_cast<Model*>(h);
-        set_tape_stream(static_cast<hipStream_t>(stream));
+    return with_model(h, [&](Model* m) {
+        if (!host_ids || !host_targets || !loss || n <= 0) throw Error(PK_ERR_ARGUMENT, "pk_llama_loss_backward: null or empty argument");
+        set_tape_stream(static_cast<hipStream_t>(stream));  // the model keeps it: the optimiser step runs there too
         for (int64_t i = 0; i < n; ++i)
             if (host_ids[i] < 0 || host_ids[i] >= m->cfg.vocab) throw std::runtime_error("embedding: id out of range");
         for (int64_t i = 0; i < n; ++i)
@@ -301,7 +351,7 @@ int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets
         dev_reset_peak();
         const size_t live0 = live_variables();
         Var hid = m->hidden(ids, n, seq_len);
-        Var l = fused_head ? ops::linear_cross_entropy(hid, m->embed, tg, 2048)
+        Var l = fused_head ? ops::linear_cross_entropy(hid, m->embed, tg, m->head_chunk_rows)
                            : ops::cross_entropy(ops::matmul_nt(hid, m->embed), tg);
         hid.reset();
         hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
@@ -319,8 +369,7 @@ int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets
 }
 
 int pk_llama_adamw_step(void* h, float lr, float b1, float b2, float eps, float wd, float max_norm, float* total_norm) {
-    return guarded([&] {
-        Model* m = static_cast<Model*>(h);
+    return with_model(h, [&](Model* m) {
         if (m->mslab.empty()) {
             m->mslab = Tensor::make(1, m->pslab.cols, PK_F32);
             m->vslab = Tensor::make(1, m->pslab.cols, PK_F32);

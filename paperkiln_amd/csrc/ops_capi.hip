@@ -31,7 +31,7 @@ int op_guard(void* stream, F&& f) {
     } catch (const std::exception& e) {
         g_op_err = e.what();
         set_error(g_op_err);
-        return PK_ERR_ARGUMENT;
+        return status_of(e);
     }
 }
 

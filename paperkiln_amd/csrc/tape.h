@@ -113,8 +113,10 @@ double clip_grad_norm(const std::vector<Var>& params, float max_norm);  // ops.c
 
 }  // namespace ops
 
-// Refresh the compute-dtype shadows of parameters after an optimizer step.
-void set_compute_dtype(int dtype);  // PK_F32 or PK_BF16, process-wide like device::set (device.cpp:41-46)
+// Element type of activations and GEMM operands on the current context (PK_F32 or PK_BF16; the reference's
+// device::set, device.cpp:41-46, is the nearest counterpart), and the compute-dtype shadows of its parameters,
+// which go stale with every optimizer step.
+void set_compute_dtype(int dtype);
 int compute_dtype();
 void invalidate_shadows();
 

@@ -6,7 +6,6 @@
 #include <cmath>
 #include <cstring>
 #include <unordered_map>
-#include <unordered_set>
 
 namespace pk {
 
@@ -15,59 +14,81 @@ std::atomic<size_t> g_live_vars{0};
 }
 size_t live_variables() { return detail::g_live_vars.load(); }
 
+// compute-dtype copies of a context's fp32 parameters, valid until the next optimizer step
+struct TapeContext::Shadows {
+    std::unordered_map<const Variable*, Tensor> single;  // one weight
+    std::unordered_map<const Variable*, Tensor> cat;     // [W_0 | W_1 | ...], keyed by the first weight
+};
+
 namespace {
 thread_local bool g_grad_enabled = true;
-int g_compute = PK_F32;
-// compute-dtype copies of fp32 parameters, valid until the next optimizer step
-std::unordered_map<const Variable*, Tensor> g_shadow;
+thread_local TapeContext g_own_context;            // what a thread works on outside any ContextScope
+thread_local TapeContext* g_context = nullptr;
+
+TapeContext::Shadows& shadows() {
+    TapeContext& c = tape_context();
+    if (!c.shadows) c.shadows = std::make_shared<TapeContext::Shadows>();
+    return *c.shadows;
+}
 
 const Tensor& shadow_of(const Var& W) {
-    if (g_compute == PK_F32 || W->data.dtype != PK_F32) return W->data;
-    auto it = g_shadow.find(W.get());
-    if (it == g_shadow.end()) {
-        Tensor t = Tensor::make(W->data.rows, W->data.cols, g_compute);
+    const int compute = tape_context().compute;
+    if (compute == PK_F32 || W->data.dtype != PK_F32) return W->data;
+    auto& map = shadows().single;
+    auto it = map.find(W.get());
+    if (it == map.end()) {
+        Tensor t = Tensor::make(W->data.rows, W->data.cols, compute);
         k_cast(W->data, t);
-        it = g_shadow.emplace(W.get(), std::move(t)).first;
+        it = map.emplace(W.get(), std::move(t)).first;
     }
     return it->second;
 }
 
-// [W_0 | W_1 | ...] in the compute dtype, keyed by the first weight; rebuilt after every optimizer step
-std::unordered_map<const Variable*, Tensor> g_shadow_cat;
 const Tensor& shadow_cat(const std::vector<Var>& Ws) {
-    auto it = g_shadow_cat.find(Ws[0].get());
-    if (it == g_shadow_cat.end()) {
+    auto& map = shadows().cat;
+    auto it = map.find(Ws[0].get());
+    if (it == map.end()) {
         const int64_t d = Ws[0]->data.cols;
-        Tensor t = Tensor::make(Ws[0]->data.rows, d * static_cast<int64_t>(Ws.size()), g_compute);
+        Tensor t = Tensor::make(Ws[0]->data.rows, d * static_cast<int64_t>(Ws.size()), tape_context().compute);
         for (size_t k = 0; k < Ws.size(); ++k) k_cast_cols(Ws[k]->data, t, static_cast<int64_t>(k) * d);
-        it = g_shadow_cat.emplace(Ws[0].get(), std::move(t)).first;
+        it = map.emplace(Ws[0].get(), std::move(t)).first;
     }
     return it->second;
 }
 
-// Post-order DFS over parents, iterative (autograd.cpp:31-45).
-void topo(const Var& root, std::vector<Variable*>& order) {
-    std::unordered_set<Variable*> seen;
-    std::vector<std::pair<Variable*, size_t>> stack{{root.get(), 0}};
-    seen.insert(root.get());
-    while (!stack.empty()) {
-        auto& [node, next] = stack.back();
-        if (next < node->parents.size()) {
-            Variable* p = node->parents[next++].get();
-            if (seen.insert(p).second) stack.emplace_back(p, 0);
-        } else {
-            order.push_back(node);
-            stack.pop_back();
+// The order the backward closures run in: the root first, every other node once all the nodes that consume it
+// have run, so its gradient is complete by then. The reference gets such an order by reversing a depth-first
+// post-order (src/autograd.cpp:31-45, 58-65); here the consumers of each node are counted first and a node is
+// released when its count reaches zero, which needs no recursion either and visits each edge twice.
+std::vector<Variable*> backward_order(const Var& root) {
+    std::unordered_map<Variable*, int> consumers_left;
+    std::vector<Variable*> frontier{root.get()};
+    consumers_left[root.get()] = 0;
+    while (!frontier.empty()) {
+        Variable* n = frontier.back();
+        frontier.pop_back();
+        for (const Var& p : n->parents) {
+            auto found = consumers_left.try_emplace(p.get(), 0);
+            ++found.first->second;
+            if (found.second) frontier.push_back(p.get());
         }
     }
+    std::vector<Variable*> order;
+    order.reserve(consumers_left.size());
+    std::vector<Variable*> ready{root.get()};
+    while (!ready.empty()) {
+        Variable* n = ready.back();
+        ready.pop_back();
+        order.push_back(n);
+        for (const Var& p : n->parents)
+            if (--consumers_left[p.get()] == 0) ready.push_back(p.get());
+    }
+    return order;
 }
 
 void run_backward(const Var& root) {
-    std::vector<Variable*> order;
-    topo(root, order);
-    for (auto it = order.rbegin(); it != order.rend(); ++it) {
-        if ((*it)->backward_fn && !(*it)->grad.empty()) (*it)->backward_fn();
-    }
+    for (Variable* n : backward_order(root))
+        if (n->backward_fn && !n->grad.empty()) n->backward_fn();
 }
 
 float scalar_to_host(const Tensor& t) {
@@ -94,22 +115,22 @@ pk_tensor4 view4(const void* base, int64_t elem_off, size_t esize, int64_t sb, i
     return t;
 }
 void attn_check(int rc) {
-    if (rc != PK_OK) throw std::runtime_error(pk_last_error());
+    if (rc != PK_OK) throw Error(rc, pk_last_error());
 }
 
 }  // namespace
 
+TapeContext& tape_context() { return g_context ? *g_context : g_own_context; }
+ContextScope::ContextScope(TapeContext& c) : prev_(g_context) { g_context = &c; }
+ContextScope::~ContextScope() { g_context = prev_; }
+
 void set_compute_dtype(int dtype) {
     if (dtype != PK_F32 && dtype != PK_BF16) throw std::runtime_error("compute dtype must be PK_F32 or PK_BF16");
-    g_compute = dtype;
-    g_shadow.clear();
-    g_shadow_cat.clear();
+    tape_context().compute = dtype;
+    tape_context().shadows.reset();
 }
-int compute_dtype() { return g_compute; }
-void invalidate_shadows() {
-    g_shadow.clear();
-    g_shadow_cat.clear();
-}
+int compute_dtype() { return tape_context().compute; }
+void invalidate_shadows() { tape_context().shadows.reset(); }
 
 Tensor& Variable::ensure_grad() {
     if (grad.empty()) {
@@ -120,7 +141,7 @@ Tensor& Variable::ensure_grad() {
 }
 
 void Variable::accumulate(const Tensor& g, float a) {
-    if (g.rows != data.rows || g.cols != data.cols) throw std::runtime_error("accumulate: gradient shape mismatch");
+    if (g.rows != data.rows || g.cols != data.cols) shape_fail("accumulate: gradient shape mismatch");
     if (grad.empty()) {
         grad = Tensor::make(data.rows, data.cols, is_param ? PK_F32 : data.dtype);
         k_scale(g, a, grad);  // first contribution: grad = a * g, no zero fill
@@ -173,35 +194,35 @@ void zero_grad(const std::vector<Var>& vars) {
 
 Var checkpoint(const std::function<Var(const Var&)>& fn, const Var& x) {
     if (!grad_enabled()) return fn(x);  // eval: nothing to rematerialise
-    Tensor out_data;
+    Tensor boundary;
     {
-        NoGrad ng;
-        out_data = fn(x)->data;  // the inner tape never exists
+        NoGrad tape_off;
+        boundary = fn(x)->data;  // only the segment's output survives this scope
     }
-    Var out = make_var(std::move(out_data), true);
-    out->parents = {x};
-    Variable* self = out.get();
-    auto fn_copy = fn;
-    out->backward_fn = [self, fn_copy]() {
-        const Var& xin = self->parents[0];
-        // Re-run the segment on a detached leaf that shares the input's storage: no op writes
-        // into a tensor it did not produce itself, so the copy the reference makes
-        // (autograd.cpp:86) is not needed.
-        Var x2 = make_var(xin->data, /*requires_grad=*/true);
-        Var y2 = fn_copy(x2);
-        if (y2->data.rows != self->grad.rows || y2->data.cols != self->grad.cols)
-            throw std::runtime_error("checkpoint: recomputed output shape mismatch");
-        y2->accumulate_owned(std::move(self->grad));  // this node's gradient has no other reader
-        run_backward(y2);  // parameters inside fn are the model's own, their grads land in place
-        if (xin->requires_grad && !x2->grad.empty()) xin->accumulate_owned(std::move(x2->grad));
+    Var node = make_var(std::move(boundary), true);
+    node->parents = {x};
+    Variable* raw = node.get();
+    node->backward_fn = [raw, segment = fn]() {
+        const Var& input = raw->parents[0];
+        // Rebuild the segment's tape from a fresh leaf that shares the input's storage (no op writes into a
+        // tensor it did not produce, so the reference's copy of x, autograd.cpp:86, is not needed), hand it this
+        // node's gradient -- nobody else reads it -- and run the rebuilt tape. Parameters used inside the
+        // segment are the model's own Variables, so their gradients land where they belong.
+        Var leaf = make_var(input->data, /*requires_grad=*/true);
+        Var rebuilt = segment(leaf);
+        if (rebuilt->data.rows != raw->grad.rows || rebuilt->data.cols != raw->grad.cols)
+            shape_fail("checkpoint: recomputed output shape mismatch");
+        rebuilt->accumulate_owned(std::move(raw->grad));
+        run_backward(rebuilt);
+        if (input->requires_grad && !leaf->grad.empty()) input->accumulate_owned(std::move(leaf->grad));
     };
-    return out;
+    return node;
 }
 
 namespace ops {
 
 Var linear(const Var& x, const Var& W) {
-    if (x->data.cols != W->data.rows) throw std::runtime_error("matmul: inner dimensions disagree");
+    if (x->data.cols != W->data.rows) shape_fail("matmul: inner dimensions disagree");
     const Tensor& Wc = shadow_of(W);
     Tensor y = Tensor::make(x->data.rows, W->data.cols, x->data.dtype);
     gemm(x->data, false, Wc, false, y.ptr(), y.dtype, y.rows, y.cols, y.cols, 0.0f);
@@ -228,7 +249,7 @@ Var linear_cat(const Var& x, const std::vector<Var>& Ws) {
     if (Ws.empty() || Ws.size() > 4) throw std::runtime_error("linear_cat: 1 to 4 weights");
     const int64_t N = x->data.rows, d = Ws[0]->data.cols;
     for (const Var& W : Ws)
-        if (W->data.cols != d || W->data.rows != x->data.cols) throw std::runtime_error("matmul: inner dimensions disagree");
+        if (W->data.cols != d || W->data.rows != x->data.cols) shape_fail("matmul: inner dimensions disagree");
     const int n = static_cast<int>(Ws.size());
     Tensor y = Tensor::make(N, n * d, x->data.dtype);
     gemm(x->data, false, shadow_cat(Ws), false, y.ptr(), y.dtype, N, n * d, n * d, 0.0f);
@@ -314,7 +335,7 @@ Var silu(const Var& x) {
 }
 
 Var silu_mul(const Var& gate, const Var& up) {
-    if (gate->data.rows != up->data.rows || gate->data.cols != up->data.cols) throw std::runtime_error("mul: shape mismatch");
+    if (gate->data.rows != up->data.rows || gate->data.cols != up->data.cols) shape_fail("mul: shape mismatch");
     Tensor y = Tensor::make(gate->data.rows, gate->data.cols, gate->data.dtype);
     k_silu_mul_fwd(gate->data, up->data, y);
     return record(std::move(y), {gate, up}, [](Variable* self) {
@@ -330,7 +351,7 @@ Var silu_mul(const Var& gate, const Var& up) {
 }
 
 Var silu_mul_cat(const Var& gu) {
-    if (gu->data.cols % 2 != 0) throw std::runtime_error("mul: shape mismatch");
+    if (gu->data.cols % 2 != 0) shape_fail("mul: shape mismatch");
     Tensor y = Tensor::make(gu->data.rows, gu->data.cols / 2, gu->data.dtype);
     k_silu_mul_cat_fwd(gu->data, y);
     return record(std::move(y), {gu}, [](Variable* self) {
@@ -343,7 +364,7 @@ Var silu_mul_cat(const Var& gu) {
 }
 
 Var rmsnorm(const Var& x, const Var& w) {
-    if (w->data.rows != 1 || w->data.cols != x->data.cols) throw std::runtime_error("rmsnorm: w must be [1, cols(x)]");
+    if (w->data.rows != 1 || w->data.cols != x->data.cols) shape_fail("rmsnorm: w must be [1, cols(x)]");
     auto rinv = std::make_shared<Buffer>(sizeof(float) * x->data.rows);
     Tensor y = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
     k_rmsnorm_fwd(x->data, w->data, 1e-5f, y, static_cast<float*>(rinv->p));
@@ -360,7 +381,7 @@ Var rmsnorm(const Var& x, const Var& w) {
 }
 
 Var apply_rope(const Var& qkv, const std::shared_ptr<Buffer>& pos, float theta, int head_dim, int rot_heads, bool in_place) {
-    if (qkv->data.cols % 3 != 0) throw std::runtime_error("apply_rope: cols must be divisible by 3");
+    if (qkv->data.cols % 3 != 0) shape_fail("apply_rope: cols must be divisible by 3");
     const int d = static_cast<int>(qkv->data.cols / 3);
     if (in_place) {
         // The caller hands over a projection nobody else reads (a Linear's backward needs its input and weight, not
@@ -424,9 +445,9 @@ pk_attn_shape shape_of(const AttnGeom& g, int dtype) {
 
 Var attention_qkv(const Var& qkv, int n_heads, float scale, int64_t seq_len, bool causal, int window, int sinks) {
     const int64_t N = qkv->data.rows, d3 = qkv->data.cols;
-    if (d3 % 3 != 0 || (d3 / 3) % n_heads != 0) throw std::runtime_error("fused_attention: shape mismatch");
+    if (d3 % 3 != 0 || (d3 / 3) % n_heads != 0) shape_fail("fused_attention: shape mismatch");
     const int64_t d = d3 / 3, sl = seq_len == 0 ? N : seq_len;
-    if (N % sl != 0) throw std::runtime_error("fused_attention: rows not a multiple of seq_len");
+    if (N % sl != 0) shape_fail("fused_attention: rows not a multiple of seq_len");
     AttnGeom g{N / sl, sl, n_heads, static_cast<int>(d / n_heads), scale, causal, window, sinks};
     const int dt = qkv->data.dtype;
     const size_t es = qkv->data.esize();
@@ -462,9 +483,9 @@ Var head_attention(const Var& q, const Var& k, const Var& v, float scale, int64_
                    int sinks, const char* who) {
     const int64_t T = q->data.rows;
     if (k->data.rows != T || v->data.rows != T || q->data.cols != k->data.cols || v->data.cols != k->data.cols)
-        throw std::runtime_error(std::string(who) + ": shape mismatch");
+        shape_fail(std::string(who) + ": shape mismatch");
     const int64_t sl = seq_len == 0 ? T : seq_len;
-    if (T % sl != 0) throw std::runtime_error(std::string(who) + ": rows not a multiple of seq_len");
+    if (T % sl != 0) shape_fail(std::string(who) + ": rows not a multiple of seq_len");
     const int dk = static_cast<int>(q->data.cols);
     AttnGeom g{T / sl, sl, 1, dk, scale, causal, window, sinks};
     const int dt = q->data.dtype;
@@ -507,7 +528,7 @@ Var swa_attention(const Var& q, const Var& k, const Var& v, float scale, int64_t
 }
 
 Var matmul_nt(const Var& h, const Var& E) {
-    if (h->data.cols != E->data.cols) throw std::runtime_error("matmul: inner dimensions disagree");
+    if (h->data.cols != E->data.cols) shape_fail("matmul: inner dimensions disagree");
     Tensor y = Tensor::make(h->data.rows, E->data.rows, PK_F32);  // logits stay fp32, as in the reference
     gemm(h->data, false, shadow_of(E), true, y.ptr(), y.dtype, y.rows, y.cols, y.cols, 0.0f);
     return record(std::move(y), {h, E}, [](Variable* self) {
@@ -549,7 +570,7 @@ Var cross_entropy(const Var& logits, const std::shared_ptr<Buffer>& targets) {
 
 Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffer>& targets, int64_t chunk_rows) {
     const int64_t N = h->data.rows, V = E->data.rows, d = h->data.cols;
-    if (d != E->data.cols) throw std::runtime_error("matmul: inner dimensions disagree");
+    if (d != E->data.cols) shape_fail("matmul: inner dimensions disagree");
     if (chunk_rows <= 0) chunk_rows = 1024;
     const int* tg = static_cast<const int*>(targets->p);
     const size_t hes = h->data.esize();

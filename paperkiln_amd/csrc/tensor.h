@@ -13,16 +13,28 @@
 
 namespace pk {
 
+// What the host side throws. It is a std::runtime_error, as every failure of the reference is (shape faults,
+// src/ops.cpp:866-870; runtime-API faults, src/cuda_ops.cu:34-38), and carries the status the C ABI returns.
+struct Error : std::runtime_error {
+    int code;
+    Error(int c, const std::string& msg) : std::runtime_error(msg), code(c) {}
+};
+[[noreturn]] inline void shape_fail(const std::string& msg) { throw Error(PK_ERR_SHAPE, msg); }
+// The status of an exception caught at the C ABI: an Error's own code, PK_ERR_OOM for bad_alloc, else PK_ERR_ARGUMENT.
+int status_of(const std::exception& e);
+
 // ---- allocator -------------------------------------------------------------
 // Caching device allocator with a byte-level high-water mark. It replaces the
 // per-call cudaMalloc / cudaFree of the reference's device seam (paperkiln
 // src/cuda_resident.cu:226-263, src/cuda_ops.cu:63-72) and supplies the memory
 // receipt the reference can only give as a node count (live_variables(),
 // include/microtorch/autograd.hpp:61-64). Blocks are recycled in stream order:
-// all work of one tape runs on one stream, so a freed block may be handed out
-// again immediately.
+// a freed block remembers the stream of the thread that freed it (tape_stream())
+// and is handed out again at once, but only to a request made for that same
+// stream, whose later work is ordered after the work that last used the block.
 void* dev_alloc(size_t bytes);
-void dev_free(void* p);
+bool dev_free(void* p);       // false: not a block this allocator has handed out (nothing is done then)
+bool dev_owns(const void* p);  // a block this allocator handed out and has not been given back
 size_t dev_live_bytes();
 size_t dev_peak_bytes();
 void dev_reset_peak();
@@ -35,7 +47,7 @@ struct Buffer {
     explicit Buffer(size_t n) : p(dev_alloc(n)), bytes(n) {}
     Buffer(void* caller_memory, size_t n) : p(caller_memory), bytes(n), owned(false) {}  // a view of caller memory
     ~Buffer() {
-        if (owned) dev_free(p);
+        if (owned) (void)dev_free(p);
     }
     Buffer(const Buffer&) = delete;
     Buffer& operator=(const Buffer&) = delete;
@@ -53,7 +65,7 @@ struct Tensor {
     int64_t numel() const { return rows * cols; }
     size_t esize() const { return dtype == PK_F32 ? 4 : 2; }
     static Tensor make(int64_t r, int64_t c, int dt) {
-        if (r <= 0 || c <= 0) throw std::runtime_error("Matrix: zero dimension");  // components.cpp:29-58
+        if (r <= 0 || c <= 0) shape_fail("Matrix: zero dimension");  // components.cpp:29-58
         Tensor t;
         t.rows = r;
         t.cols = c;
@@ -63,7 +75,7 @@ struct Tensor {
     }
     static Tensor borrow(const void* p, int64_t r, int64_t c, int dt) {  // caller-owned device memory, never freed here
         if (!p) throw std::runtime_error("null device pointer");
-        if (r <= 0 || c <= 0) throw std::runtime_error("Matrix: zero dimension");
+        if (r <= 0 || c <= 0) shape_fail("Matrix: zero dimension");
         if (dt != PK_F32 && dt != PK_BF16) throw std::runtime_error("unknown element type");
         Tensor t;
         t.rows = r;
@@ -80,9 +92,35 @@ struct Tensor {
     }
 };
 
-void hip_check(hipError_t e, const char* what);  // throws std::runtime_error, as cuda_check does (cuda_ops.cu:34-38)
-hipStream_t tape_stream();
-void set_tape_stream(hipStream_t s);
+void hip_check(hipError_t e, const char* what);  // throws Error(PK_ERR_HIP), as cuda_check throws (cuda_ops.cu:34-38)
+
+// ---- per-tape state ---------------------------------------------------------
+// Everything a tape needs besides its Variables: the stream its kernels are
+// enqueued on and the element type activations and GEMM operands are held in.
+// The reference keeps the like in process-wide globals (device::set,
+// src/device.cpp:22,41-46); here a model owns one, and the C ABI makes it the
+// calling thread's current context for the length of each call, so two models
+// of different element types, or on different streams, do not see each other.
+// A thread that never entered a scope works on a context of its own.
+struct TapeContext {
+    hipStream_t stream = nullptr;
+    int compute = PK_F32;
+    struct Shadows;  // compute-dtype copies of fp32 parameters (tape.hip)
+    std::shared_ptr<Shadows> shadows;
+};
+TapeContext& tape_context();
+class ContextScope {
+public:
+    explicit ContextScope(TapeContext& c);
+    ~ContextScope();
+    ContextScope(const ContextScope&) = delete;
+    ContextScope& operator=(const ContextScope&) = delete;
+
+private:
+    TapeContext* prev_;
+};
+inline hipStream_t tape_stream() { return tape_context().stream; }
+inline void set_tape_stream(hipStream_t s) { tape_context().stream = s; }
 
 // ---- kernel launchers (elementwise.hip) -----------------------------------
 // All take row-major contiguous tensors; T = fp32 or bf16 storage, fp32 math.

@@ -65,8 +65,13 @@ class Llama:
     def grads(self):
         return self._get(self.L.pk_llama_get_grad)
 
-    def loss_backward(self, ids, targets, seq_len=0, checkpoint=False, backward=True, fused_head=True):
-        """zero_grad -> forward -> cross-entropy -> backward. Returns (loss, stats dict)."""
+    def set_head_chunk(self, rows):
+        """Rows of the tied head evaluated at a time when fused_head=True (default 2048)."""
+        _lib.check(self.L.pk_llama_set_head_chunk(self.h, int(rows)))
+
+    def loss_backward(self, ids, targets, seq_len=0, checkpoint=False, backward=True, fused_head=True, stream=None):
+        """zero_grad -> forward -> cross-entropy -> backward. Returns (loss, stats dict).
+        stream: a HIP stream handle (int) the step is enqueued on; None = the default stream."""
         ids = np.ascontiguousarray(ids, np.int32)
         targets = np.ascontiguousarray(targets, np.int32)
         if len(ids) != len(targets):
@@ -74,7 +79,7 @@ class Llama:
         loss, st = C.c_float(), LlamaStats()
         _lib.check(self.L.pk_llama_loss_backward(self.h, ids.ctypes.data_as(_i32p), targets.ctypes.data_as(_i32p),
                                                  len(ids), seq_len, int(checkpoint), int(backward), int(fused_head),
-                                                 C.byref(loss), C.byref(st), None))
+                                                 C.byref(loss), C.byref(st), C.c_void_p(stream) if stream else None))
         return loss.value, {"live_vars_after_forward": st.live_vars_after_forward,
                             "activation_bytes_after_forward": st.activation_bytes_after_forward,
                             "peak_activation_bytes": st.peak_activation_bytes}

@@ -63,3 +63,41 @@ def test_backward_workspace_follows_the_mask():
     assert ws(256, 4, t=q0) == 4 * B * Hq * q0   # the sequence ends with the band: no tail
     odd = 4 * B * Hq * 4001                      # delta not a multiple of 256 bytes: the tail starts aligned
     assert ws(256, 4, t=4001) == odd + (256 - odd % 256) % 256 + 4 * B * Hkv * (-(-(4001 - q0) // 512) + 1) * 2 * 32 * dk
+
+
+def test_a_window_that_covers_the_sequence_is_no_band():
+    """The reference takes size_t window / sinks and defines window >= seq_len as plain causal attention
+    (tests/test_swa.cpp:47-57), so INT32_MAX is a legal "no band": the shape is brought into range on the host,
+    before any index arithmetic, and sizes its workspace as the causal mask does."""
+    L = _lib.lib()
+    B, T, Hq, Hkv, dk = 2, 4096, 8, 4, 128
+
+    def ws(window, sinks):
+        sh = _lib.AttnShape(B, T, Hq, Hkv, dk, 1, window, sinks, 0.5, _lib.PK_BF16, _lib.PK_BF16)
+        return L.pk_attn_bwd_workspace_bytes(ctypes.byref(sh))
+
+    causal = ws(0, 0)
+    assert causal == 4 * B * Hq * T
+    for window in (T, T + 1, 2**31 - 1):
+        for sinks in (0, 4, 2**31 - 1):
+            assert ws(window, sinks) == causal
+    assert ws(T // 2, 4) > causal         # a real band with sink keys still gets its sink-tail rows
+    assert ws(256, 2**31 - 1) == causal   # more sink keys than tokens: every key is a sink, nothing to split
+    sh = _lib.AttnShape(1, 2**24 + 1, 1, 1, 64, 1, 0, 0, 0.5, _lib.PK_BF16, _lib.PK_BF16)
+    assert L.pk_attn_bwd_workspace_bytes(ctypes.byref(sh)) == 0 and b"2^24" in L.pk_last_error()
+
+
+def test_handle_and_pointer_errors_do_not_need_a_gpu():
+    """A NULL model handle and a pointer pk_alloc never returned are reported, not dereferenced or ignored."""
+    L = _lib.lib()
+    r, c = ctypes.c_int64(), ctypes.c_int64()
+    assert L.pk_llama_param_info(None, 0, None, 0, ctypes.byref(r), ctypes.byref(c)) == 2
+    assert b"null model handle" in L.pk_last_error()
+    assert L.pk_llama_num_params(None) == -1
+    assert L.pk_llama_adamw_step(None, 1e-3, 0.9, 0.999, 1e-8, 0.0, 0.0, None) == 2
+    assert L.pk_llama_set_head_chunk(None, 128) == 2
+    assert L.pk_llama_destroy(None) == 0
+    buf = ctypes.create_string_buffer(64)
+    assert L.pk_free(ctypes.cast(buf, ctypes.c_void_p)) == 2 and b"pk_alloc" in L.pk_last_error()
+    assert L.pk_free(None) == 0
+    assert L.pk_alloc(64, None) == 2

@@ -99,6 +99,20 @@ def test_embedding_vs_reference_vectors(bo, vec):
     close(dt, vec["emb_dtable"], F32_TOL)
 
 
+def test_embedding_gradient_is_summed_in_row_order(bo, oracle):
+    """Heavily repeated ids (3000 rows over 7 table rows, plus a table far larger than the row count): the
+    scatter-add forms each table row's sum in ascending row order, as the reference's loop does
+    (src/ops.cpp:338-347), so it equals the CPU restatement bit for bit and is the same on every run."""
+    for vocab, n, seed in ((7, 3000, 51), (40_000, 257, 52)):
+        table = synth.randn(seed, (vocab, 48), 0.5)
+        ids = synth.randint(seed + 100, n, vocab).astype(np.int32)
+        g = synth.randn(seed + 200, (n, 48), 1.0)
+        _, want = oracle.embedding(table, ids, g)
+        runs = [host(bo.embedding(dev(table), dev(ids), dev(g))[1]) for _ in range(3)]
+        assert np.array_equal(runs[0], want)
+        assert np.array_equal(runs[1], runs[0]) and np.array_equal(runs[2], runs[0])
+
+
 @pytest.mark.parametrize("name", ["llama_T16_single"])
 def test_clip_and_adamw_vs_reference_optimiser(bo, name):
     z = np.load(os.path.join(GOLDEN, name + ".npz"))

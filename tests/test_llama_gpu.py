@@ -137,3 +137,134 @@ def test_errors():
     with pytest.raises(RuntimeError, match="not a multiple of seq_len"):
         m.loss_backward([1, 2, 3], [1, 2, 3], seq_len=2)
     m.close()
+
+
+def reldiff(a, b):
+    """Largest |a - b| over all parameters, relative to the largest |b| of the same parameter."""
+    return max(float(np.abs(a[k].astype(np.float64) - b[k]).max() / max(float(np.abs(b[k]).max()), 1e-30)) for k in a)
+
+
+# (dtype, vocab, tokens, seq_len, rows per head chunk or None = the library's default of 2048)
+HEAD_CASES = [
+    ("fp32", 4096, 5000, 1000, None),     # 3 chunks of the default size, the last one ragged (904 rows)
+    ("bf16", 4096, 5000, 1000, None),     # the same through the bf16 dlogits that overlay the fp32 logits
+    ("fp32", 4096, 1500, 500, 256),       # 6 chunks, ragged tail of 220
+    ("bf16", 4096, 1500, 500, 256),
+    ("fp32", 1001, 700, 350, 256),        # vocab % 4 != 0: the generic row kernel (+ cast in bf16)
+    ("bf16", 1001, 700, 350, 256),
+    ("fp32", 50257, 600, 300, 256),       # vocab > 32768: a row no longer fits the one-pass kernel's registers
+    ("bf16", 50257, 600, 300, 256),
+]
+
+
+@pytest.mark.parametrize("case", HEAD_CASES, ids=lambda c: f"{c[0]}_V{c[1]}_N{c[2]}_chunk{c[4]}")
+def test_chunked_tied_head_matches_the_materialised_head(case):
+    """ops::cross_entropy over llama.cpp:88's logits (src/ops.cpp:350-376), evaluated chunk by chunk, against the
+    same head with the [N, vocab] logits materialised as the reference does: loss and every gradient, with more
+    than two chunks, a ragged last chunk, and both fall-back row kernels. The chunk loop accumulates dE across
+    chunks, offsets the per-row losses, targets and dh rows by the chunk start, and (bf16) writes dlogits over
+    the first half of each fp32 logits row; an error in any of these shows as a difference here."""
+    dtype, vocab, n, sl, chunk = case
+    cfg = dict(vocab=vocab, d=64, n_layers=1, n_heads=2, d_ff=176)
+    m = Llama(compute_dtype=dtype, rope_all_heads=True, seed=21, **cfg)
+    if chunk:
+        m.set_head_chunk(chunk)
+    toks = synth.randint(31, n + 1, vocab)
+    x, y = toks[:-1], toks[1:]
+    loss_mat, _ = m.loss_backward(x, y, sl, fused_head=False)
+    g_mat = m.grads()
+    loss_chunked, _ = m.loss_backward(x, y, sl, fused_head=True)
+    g_chunked = m.grads()
+    d_abs, d_rel = maxdiff(g_chunked, g_mat), reldiff(g_chunked, g_mat)
+    print(f"\n  {dtype} V={vocab} N={n} chunk={chunk}: loss {loss_chunked:.7f} vs {loss_mat:.7f}, "
+          f"grad diff abs {d_abs:.2e} rel {d_rel:.2e}", flush=True)
+    if dtype == "fp32":
+        assert abs(loss_chunked - loss_mat) < 1e-6 and d_abs < 1e-6 and d_rel < 1e-4
+    else:
+        # both heads round dlogits to bf16 once and accumulate in fp32; what differs is the order of the sums
+        assert abs(loss_chunked - loss_mat) < 1e-5 and d_abs < 1e-4 and d_rel < 2e-2
+    # one chunk that holds every row is the degenerate case and must agree with many chunks
+    m.set_head_chunk(n)
+    loss_one, _ = m.loss_backward(x, y, sl, fused_head=True)
+    assert abs(loss_one - loss_chunked) < 1e-6
+    assert maxdiff(m.grads(), g_chunked) < (1e-6 if dtype == "fp32" else 1e-4)
+    m.close()
+
+
+def test_config5_full_size_checkpointing_bars():
+    """BASELINE config 5 at full size (6 layers, d 512, 8 heads of 64, d_ff 1376, vocab 32000 tied, B=8 x T=1024,
+    bf16 compute over fp32 master weights): the checkpointed step's loss equals the plain step's within 1e-4 and
+    its peak activation memory is at least 3x lower (tests/test_checkpointing.cpp:72-90 states the same pair of
+    claims as loss equality and a node count). Gradients are compared too: same kernels on the same inputs."""
+    cfg = dict(vocab=32000, d=512, n_layers=6, n_heads=8, d_ff=1376)
+    B, T = 8, 1024
+    m = Llama(compute_dtype="bf16", seed=0, **cfg)
+    toks = synth.randint(9, B * T + 1, cfg["vocab"])
+    x, y = toks[:-1], toks[1:]
+    loss_p, st_p = m.loss_backward(x, y, T, checkpoint=False)
+    g_p = m.grads()
+    loss_c, st_c = m.loss_backward(x, y, T, checkpoint=True)
+    g_c = m.grads()
+    ratio = st_p["peak_activation_bytes"] / st_c["peak_activation_bytes"]
+    print(f"\n  config 5: loss plain {loss_p:.6f} checkpointed {loss_c:.6f}; peak activation bytes "
+          f"{st_p['peak_activation_bytes']} -> {st_c['peak_activation_bytes']} ({ratio:.2f}x); "
+          f"grad diff {maxdiff(g_c, g_p):.1e}", flush=True)
+    assert np.isfinite(loss_p) and abs(loss_p - np.log(cfg["vocab"])) < 0.5   # random init: loss ~ log(vocab)
+    assert abs(loss_c - loss_p) <= 1e-4
+    assert ratio >= 3.0
+    assert maxdiff(g_c, g_p) <= 1e-4
+    # the full-size head against two other chunkings of the same rows (4 chunks by default)
+    m.set_head_chunk(1024)
+    loss_8, _ = m.loss_backward(x, y, T, checkpoint=True)
+    assert abs(loss_8 - loss_c) <= 1e-5 and reldiff(m.grads(), g_c) < 2e-2
+    m.close()
+
+
+def test_two_models_of_different_element_types_side_by_side():
+    """A bf16 and an fp32 model alive together, stepped in turn on streams of their own from two host threads:
+    each gives exactly what it gives alone. (Element type, stream and parameter shadows belong to the model.)"""
+    import threading
+
+    import torch
+
+    cfg = dict(vocab=512, d=128, n_layers=2, n_heads=2, d_ff=344)
+    toks = synth.randint(17, 2 * 160 + 1, cfg["vocab"])
+    x, y, sl = toks[:-1], toks[1:], 160
+
+    def alone(dtype):
+        m = Llama(compute_dtype=dtype, rope_all_heads=True, seed=9, **cfg)
+        out = []
+        for _ in range(3):
+            loss, _ = m.loss_backward(x, y, sl, checkpoint=True)
+            out.append((loss, m.grads()))
+            m.adamw_step(1e-3, max_norm=1.0)
+        m.close()
+        return out
+
+    want = {dt: alone(dt) for dt in ("bf16", "fp32")}
+    models = {"bf16": Llama(compute_dtype="bf16", rope_all_heads=True, seed=9, **cfg)}
+    models["fp32"] = Llama(compute_dtype="fp32", rope_all_heads=True, seed=9, **cfg)  # created second: it must not
+    got = {"bf16": [], "fp32": []}                                                   # change the first one's type
+    streams = {dt: torch.cuda.Stream() for dt in models}
+    errors = []
+
+    def drive(dt):
+        try:
+            for _ in range(3):
+                loss, _ = models[dt].loss_backward(x, y, sl, checkpoint=True, stream=streams[dt].cuda_stream)
+                got[dt].append((loss, models[dt].grads()))
+                models[dt].adamw_step(1e-3, max_norm=1.0)
+        except Exception as e:  # noqa: BLE001
+            errors.append((dt, e))
+
+    threads = [threading.Thread(target=drive, args=(dt,)) for dt in models]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for dt in models:
+        for (l_got, g_got), (l_want, g_want) in zip(got[dt], want[dt]):
+            assert l_got == l_want and maxdiff(g_got, g_want) == 0.0, dt
+        models[dt].close()
+    assert want["bf16"][0][0] != want["fp32"][0][0]   # the two element types really differ
