@@ -104,6 +104,19 @@ int pk_attn_bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_ten
                        const pk_tensor4* dv, void* workspace, size_t workspace_bytes, int stages,
                        void* stream);
 
+/* pk_attn_bwd without a workspace argument and without any allocation: the scratch is a device array inside
+ * the library (PK_ATTN_BWD_STATIC_MAX_WORKSPACE bytes on every GPU the library runs on, held until the process
+ * ends). It has no counterpart in the reference; it is for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc. Same kernels and same results as pk_attn_bwd.
+ * A shape whose pk_attn_bwd_workspace_bytes() exceeds the array is refused with PK_ERR_WORKSPACE. All calls on
+ * one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race; calls
+ * on one stream are ordered and safe. pk_init looks the array up for its device; otherwise the first call does. */
+#define PK_ATTN_BWD_STATIC_MAX_WORKSPACE ((size_t)32 << 20)
+int pk_attn_bwd_static(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k,
+                       const pk_tensor4* v, const pk_tensor4* o, const float* lse,
+                       const pk_tensor4* d_o, const pk_tensor4* dq, const pk_tensor4* dk,
+                       const pk_tensor4* dv, void* stream);
+
 /* ---- device memory ------------------------------------------------------
  * Caching allocator with a byte-level high-water mark: the HIP counterpart of
  * the per-call cudaMalloc/cudaFree in src/cuda_resident.cu:226-263 and

@@ -46,7 +46,7 @@ class PkError(RuntimeError):
 _lib = None
 
 # every symbol include/paperkiln_amd.h declares
-EXPORTS = ["pk_last_error", "pk_init", "pk_attn_fwd", "pk_attn_bwd_workspace_bytes", "pk_attn_bwd", "pk_attn_bwd_stages",
+EXPORTS = ["pk_last_error", "pk_init", "pk_attn_fwd", "pk_attn_bwd_workspace_bytes", "pk_attn_bwd", "pk_attn_bwd_stages", "pk_attn_bwd_static",
            "pk_alloc", "pk_free", "pk_live_bytes", "pk_peak_bytes", "pk_reset_peak", "pk_trim",
            "pk_llama_create", "pk_llama_destroy", "pk_llama_num_params", "pk_llama_param_info", "pk_llama_set_param",
            "pk_llama_get_param", "pk_llama_get_grad", "pk_llama_loss_backward", "pk_llama_adamw_step",
@@ -73,6 +73,7 @@ def lib() -> C.CDLL:
         L.pk_attn_bwd.argtypes = [SH, T4, T4, T4, T4, C.c_void_p, T4, T4, T4, T4, C.c_void_p, C.c_size_t, C.c_void_p]
         L.pk_attn_bwd_stages.argtypes = [SH, T4, T4, T4, T4, C.c_void_p, T4, T4, T4, T4, C.c_void_p, C.c_size_t,
                                          C.c_int, C.c_void_p]
+        L.pk_attn_bwd_static.argtypes = [SH, T4, T4, T4, T4, C.c_void_p, T4, T4, T4, T4, C.c_void_p]
         f32p, i32p = C.POINTER(C.c_float), C.POINTER(C.c_int)
         L.pk_alloc.argtypes = [C.c_size_t, C.POINTER(C.c_void_p)]
         L.pk_free.argtypes = [C.c_void_p]

@@ -3,6 +3,7 @@
 // no CPU path behind any entry: without a gfx950 device every call fails.
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "pk_internal.h"
 
@@ -11,6 +12,35 @@ namespace pk {
 namespace {
 thread_local std::string g_err;
 }
+
+// Scratch of pk_attn_bwd_static: the backward's workspace (row sums D_i and, for a band mask with sink keys, the
+// partial sink rows) as a device array of the library itself, so that the call needs no allocation by anybody.
+// `scratch` is a host-side stand-in for the symbol, never a device address: every GPU holds its own copy at its
+// own address, looked up once per device with hipGetSymbolAddress and used through that pointer only.
+constexpr size_t SCRATCH_BYTES = PK_ATTN_BWD_STATIC_MAX_WORKSPACE;
+static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[MAX_DEVICES] = {};
+
+// The current device's copy of `scratch`; the lookup runs once per device, with that device current.
+int scratch_of_current_device(void** out) {
+    int dev = -1;
+    PK_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return fail(PK_ERR_ARGUMENT, "device index beyond the scratch table");
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        PK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(PK_ERR_HIP, "hipGetSymbolAddress returned a null address for the scratch array");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return PK_OK;
+}
+}  // namespace
 
 void set_error(const std::string& msg) { g_err = msg; }
 
@@ -108,7 +138,8 @@ int pk_init(int device, char* arch, size_t arch_len) {
     }
     if (std::strncmp(p.gcnArchName, "gfx950", 6) != 0)
         return fail(PK_ERR_HIP, std::string("pk_init: kernels are built for gfx950 only, found ") + p.gcnArchName);
-    return PK_OK;
+    void* scratch_ptr = nullptr;  // this device's copy of the static scratch, so the first static call finds it
+    return scratch_of_current_device(&scratch_ptr);
 }
 
 int pk_attn_fwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k, const pk_tensor4* v,
@@ -136,6 +167,22 @@ int pk_attn_bwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k
                 void* stream) {
     return pk_attn_bwd_stages(s, q, k, v, o, lse, d_o, dq, dk, dv, workspace, workspace_bytes,
                               PK_BWD_ALL, stream);
+}
+
+int pk_attn_bwd_static(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k, const pk_tensor4* v,
+                       const pk_tensor4* o, const float* lse, const pk_tensor4* d_o, const pk_tensor4* dq,
+                       const pk_tensor4* dk, const pk_tensor4* dv, void* stream) {
+    if (int rc = check_shape(s, "pk_attn_bwd_static")) return rc;
+    const size_t need = delta_bytes(s) + tail_bytes(s);
+    if (need > SCRATCH_BYTES)
+        return fail(PK_ERR_WORKSPACE, "pk_attn_bwd_static: this shape needs " + std::to_string(need) +
+                                          " bytes of scratch, the static array holds " + std::to_string(SCRATCH_BYTES) +
+                                          " (PK_ATTN_BWD_STATIC_MAX_WORKSPACE); use pk_attn_bwd with a workspace");
+    void* ws = nullptr;
+    if (int rc = scratch_of_current_device(&ws)) return rc;
+    // Every word of the workspace the kernels read they have written earlier in the same call (D_i by the dQ
+    // kernel, each piece's partial sink rows by its own workgroup), so nothing has to be cleared between calls.
+    return pk_attn_bwd_stages(s, q, k, v, o, lse, d_o, dq, dk, dv, ws, SCRATCH_BYTES, PK_BWD_ALL, stream);
 }
 
 int pk_attn_bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k,

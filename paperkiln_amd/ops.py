@@ -88,6 +88,19 @@ def attn_bwd(q, k, v, o, lse, d_o, scale, causal=True, window=0, sinks=0, grad_d
     return dq, dk, dv
 
 
+def attn_bwd_static(q, k, v, o, lse, d_o, scale, causal=True, window=0, sinks=0, out=None):
+    """pk_attn_bwd_static: the same backward with the library's own static scratch instead of a workspace. The
+    call itself allocates nothing; ``out`` supplies (dq, dk, dv), which are allocated here only when it is None."""
+    if out is None:
+        out = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
+    dq, dk, dv = out
+    sh = _shape(q, k, scale, causal, window, sinks, dq.dtype)
+    _lib.check(_lib.lib().pk_attn_bwd_static(C.byref(sh), C.byref(_t4(q)), C.byref(_t4(k)), C.byref(_t4(v)),
+                                              C.byref(_t4(o)), C.c_void_p(lse.data_ptr()), C.byref(_t4(d_o)),
+                                              C.byref(_t4(dq)), C.byref(_t4(dk)), C.byref(_t4(dv)), _stream()))
+    return dq, dk, dv
+
+
 class _AttnFn(torch.autograd.Function):
     """Tape node that keeps O and LSE only (plus its parents Q, K, V), in place
     of the reference closure's captured [T,T] matrix A (src/ops.cpp:902)."""
