@@ -128,6 +128,11 @@ int pk_attn_bwd_static(const pk_attn_shape* s, const pk_tensor4* q, const pk_ten
  * Memory that several streams touch must come from elsewhere. */
 int pk_alloc(size_t bytes, void** out);
 int pk_free(void* p);   /* PK_ERR_ARGUMENT for a pointer pk_alloc did not return or that was freed before */
+/* Host <-> device copies on `stream`; both return after the copy has completed. They stand where the
+ * reference's h2d / d2h helpers and its RAII upload buffer do (src/cuda_ops.cu:45-72), for host code that
+ * keeps the reference's host-in / host-out convention and has no HIP header of its own. */
+int pk_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void* stream);
+int pk_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream);
 size_t pk_live_bytes(void);
 size_t pk_peak_bytes(void);
 void pk_reset_peak(void);

@@ -47,7 +47,7 @@ _lib = None
 
 # every symbol include/paperkiln_amd.h declares
 EXPORTS = ["pk_last_error", "pk_init", "pk_attn_fwd", "pk_attn_bwd_workspace_bytes", "pk_attn_bwd", "pk_attn_bwd_stages", "pk_attn_bwd_static",
-           "pk_alloc", "pk_free", "pk_live_bytes", "pk_peak_bytes", "pk_reset_peak", "pk_trim",
+           "pk_alloc", "pk_free", "pk_memcpy_h2d", "pk_memcpy_d2h", "pk_live_bytes", "pk_peak_bytes", "pk_reset_peak", "pk_trim",
            "pk_llama_create", "pk_llama_destroy", "pk_llama_num_params", "pk_llama_param_info", "pk_llama_set_param",
            "pk_llama_get_param", "pk_llama_get_grad", "pk_llama_loss_backward", "pk_llama_adamw_step",
            "pk_llama_set_head_chunk",
@@ -77,6 +77,8 @@ def lib() -> C.CDLL:
         f32p, i32p = C.POINTER(C.c_float), C.POINTER(C.c_int)
         L.pk_alloc.argtypes = [C.c_size_t, C.POINTER(C.c_void_p)]
         L.pk_free.argtypes = [C.c_void_p]
+        L.pk_memcpy_h2d.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.pk_memcpy_d2h.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
         for fn in (L.pk_live_bytes, L.pk_peak_bytes):
             fn.restype = C.c_size_t
         L.pk_reset_peak.restype = None

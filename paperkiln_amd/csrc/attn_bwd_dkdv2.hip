@@ -182,6 +182,11 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
             commit(0);
             if (steps > 1) fetch(1);
         }
+        // Every load issued so far -- the resident K / V rows above all -- has landed before the step loop is
+        // entered. Without this the wait-count bookkeeping carries "kv may still be in flight" around the loop
+        // and puts a vmcnt wait in front of each MFMA that reads kv, which in every later step waits for the
+        // NEXT tile's prefetch instead (a full memory latency per step).
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
 
         // transposed operand (k-chunk = rows row0 + {4g..4g+3} u {8+4g..}) of column block db, from a

@@ -44,6 +44,23 @@ using namespace pk;
 
 extern "C" {
 
+int pk_memcpy_h2d(void* dst_device, const void* src_host, size_t bytes, void* stream) {
+    return op_guard(stream, [&] {
+        if (bytes == 0) return;
+        if (!dst_device || !src_host) throw Error(PK_ERR_ARGUMENT, "pk_memcpy_h2d: null pointer");
+        hip_check(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, tape_stream()), "hipMemcpyAsync");
+        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+    });
+}
+int pk_memcpy_d2h(void* dst_host, const void* src_device, size_t bytes, void* stream) {
+    return op_guard(stream, [&] {
+        if (bytes == 0) return;
+        if (!dst_host || !src_device) throw Error(PK_ERR_ARGUMENT, "pk_memcpy_d2h: null pointer");
+        hip_check(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, tape_stream()), "hipMemcpyAsync");
+        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+    });
+}
+
 int pk_op_add(const void* a, const void* b, void* y, int64_t n, int dtype, void* stream) {
     return op_guard(stream, [&] { k_add(vec(a, n, dtype), vec(b, n, dtype), vec(y, n, dtype)); });
 }

@@ -120,6 +120,32 @@ void attn_check(int rc) {
 
 }  // namespace
 
+Tensor upload(const float* host, int64_t rows, int64_t cols, int dtype) {
+    if (!host) throw Error(PK_ERR_ARGUMENT, "upload: null host pointer");
+    Tensor staged = Tensor::make(rows, cols, PK_F32);
+    hip_check(hipMemcpyAsync(staged.ptr(), host, sizeof(float) * rows * cols, hipMemcpyHostToDevice, tape_stream()),
+              "hipMemcpyAsync");
+    Tensor out = staged;
+    if (dtype != PK_F32) {
+        out = Tensor::make(rows, cols, dtype);
+        k_cast(staged, out);
+    }
+    hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+    return out;
+}
+
+void download(const Tensor& t, float* host) {
+    if (t.empty() || !host) throw Error(PK_ERR_ARGUMENT, "download: empty tensor or null host pointer");
+    Tensor f = t;
+    if (t.dtype != PK_F32) {
+        f = Tensor::make(t.rows, t.cols, PK_F32);
+        k_cast(t, f);
+    }
+    hip_check(hipMemcpyAsync(host, f.ptr(), sizeof(float) * t.rows * t.cols, hipMemcpyDeviceToHost, tape_stream()),
+              "hipMemcpyAsync");
+    hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+}
+
 TapeContext& tape_context() { return g_context ? *g_context : g_own_context; }
 ContextScope::ContextScope(TapeContext& c) : prev_(g_context) { g_context = &c; }
 ContextScope::~ContextScope() { g_context = prev_; }

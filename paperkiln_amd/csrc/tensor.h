@@ -1,126 +1,14 @@
-// Device tensors, the caching allocator and the kernel launchers used by the
-// host-side tape (tape.h). Everything here lives in HBM; there is no host copy
-// of an activation and no CPU code path.
+// Internal side of the device tensors: the kernel launchers used by the
+// host-side tape. The types themselves (Tensor, Buffer, the allocator, the
+// tape context) are public and live in include/paperkiln_amd.hpp.
 #pragma once
 #include <hip/hip_runtime.h>
-#include <stdint.h>
 
-#include <memory>
-#include <stdexcept>
-#include <string>
-
-#include "paperkiln_amd.h"
+#include "paperkiln_amd.hpp"
 
 namespace pk {
 
-// What the host side throws. It is a std::runtime_error, as every failure of the reference is (shape faults,
-// src/ops.cpp:866-870; runtime-API faults, src/cuda_ops.cu:34-38), and carries the status the C ABI returns.
-struct Error : std::runtime_error {
-    int code;
-    Error(int c, const std::string& msg) : std::runtime_error(msg), code(c) {}
-};
-[[noreturn]] inline void shape_fail(const std::string& msg) { throw Error(PK_ERR_SHAPE, msg); }
-// The status of an exception caught at the C ABI: an Error's own code, PK_ERR_OOM for bad_alloc, else PK_ERR_ARGUMENT.
-int status_of(const std::exception& e);
-
-// ---- allocator -------------------------------------------------------------
-// Caching device allocator with a byte-level high-water mark. It replaces the
-// per-call cudaMalloc / cudaFree of the reference's device seam (paperkiln
-// src/cuda_resident.cu:226-263, src/cuda_ops.cu:63-72) and supplies the memory
-// receipt the reference can only give as a node count (live_variables(),
-// include/microtorch/autograd.hpp:61-64). Blocks are recycled in stream order:
-// a freed block remembers the stream of the thread that freed it (tape_stream())
-// and is handed out again at once, but only to a request made for that same
-// stream, whose later work is ordered after the work that last used the block.
-void* dev_alloc(size_t bytes);
-bool dev_free(void* p);       // false: not a block this allocator has handed out (nothing is done then)
-bool dev_owns(const void* p);  // a block this allocator handed out and has not been given back
-size_t dev_live_bytes();
-size_t dev_peak_bytes();
-void dev_reset_peak();
-void dev_trim();  // return cached blocks to the driver
-
-struct Buffer {
-    void* p = nullptr;
-    size_t bytes = 0;
-    bool owned = true;
-    explicit Buffer(size_t n) : p(dev_alloc(n)), bytes(n) {}
-    Buffer(void* caller_memory, size_t n) : p(caller_memory), bytes(n), owned(false) {}  // a view of caller memory
-    ~Buffer() {
-        if (owned) (void)dev_free(p);
-    }
-    Buffer(const Buffer&) = delete;
-    Buffer& operator=(const Buffer&) = delete;
-};
-
-// Row-major [rows, cols] matrix, the reference's Matrix
-// (third_party/transformer_cpp/include/matrix.hpp:32-43) moved to the device.
-struct Tensor {
-    std::shared_ptr<Buffer> buf;
-    int64_t rows = 0, cols = 0;
-    int dtype = PK_F32;
-    int64_t off_bytes = 0;  // a row-range view shares the buffer of the whole matrix
-    bool empty() const { return !buf; }
-    void* ptr() const { return buf ? static_cast<char*>(buf->p) + off_bytes : nullptr; }
-    int64_t numel() const { return rows * cols; }
-    size_t esize() const { return dtype == PK_F32 ? 4 : 2; }
-    static Tensor make(int64_t r, int64_t c, int dt) {
-        if (r <= 0 || c <= 0) shape_fail("Matrix: zero dimension");  // components.cpp:29-58
-        Tensor t;
-        t.rows = r;
-        t.cols = c;
-        t.dtype = dt;
-        t.buf = std::make_shared<Buffer>(static_cast<size_t>(r) * c * (dt == PK_F32 ? 4 : 2));
-        return t;
-    }
-    static Tensor borrow(const void* p, int64_t r, int64_t c, int dt) {  // caller-owned device memory, never freed here
-        if (!p) throw std::runtime_error("null device pointer");
-        if (r <= 0 || c <= 0) shape_fail("Matrix: zero dimension");
-        if (dt != PK_F32 && dt != PK_BF16) throw std::runtime_error("unknown element type");
-        Tensor t;
-        t.rows = r;
-        t.cols = c;
-        t.dtype = dt;
-        t.buf = std::make_shared<Buffer>(const_cast<void*>(p), static_cast<size_t>(r) * c * (dt == PK_F32 ? 4 : 2));
-        return t;
-    }
-    Tensor row_range(int64_t r0, int64_t n) const {  // rows [r0, r0+n) of this matrix, no copy
-        Tensor t = *this;
-        t.rows = n;
-        t.off_bytes = off_bytes + r0 * cols * static_cast<int64_t>(esize());
-        return t;
-    }
-};
-
 void hip_check(hipError_t e, const char* what);  // throws Error(PK_ERR_HIP), as cuda_check throws (cuda_ops.cu:34-38)
-
-// ---- per-tape state ---------------------------------------------------------
-// Everything a tape needs besides its Variables: the stream its kernels are
-// enqueued on and the element type activations and GEMM operands are held in.
-// The reference keeps the like in process-wide globals (device::set,
-// src/device.cpp:22,41-46); here a model owns one, and the C ABI makes it the
-// calling thread's current context for the length of each call, so two models
-// of different element types, or on different streams, do not see each other.
-// A thread that never entered a scope works on a context of its own.
-struct TapeContext {
-    hipStream_t stream = nullptr;
-    int compute = PK_F32;
-    struct Shadows;  // compute-dtype copies of fp32 parameters (tape.hip)
-    std::shared_ptr<Shadows> shadows;
-};
-TapeContext& tape_context();
-class ContextScope {
-public:
-    explicit ContextScope(TapeContext& c);
-    ~ContextScope();
-    ContextScope(const ContextScope&) = delete;
-    ContextScope& operator=(const ContextScope&) = delete;
-
-private:
-    TapeContext* prev_;
-};
-inline hipStream_t tape_stream() { return tape_context().stream; }
-inline void set_tape_stream(hipStream_t s) { tape_context().stream = s; }
 
 // ---- kernel launchers (elementwise.hip) -----------------------------------
 // All take row-major contiguous tensors; T = fp32 or bf16 storage, fp32 math.
