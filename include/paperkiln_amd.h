@@ -241,6 +241,14 @@ int pk_op_sumsq(const float* g, int64_t n, double* host_out, void* stream);
  * op = transpose when the flag is set (A is [k,m] then, B is [n,k]); operands dtype, output c_dtype, fp32 accumulate. */
 int pk_op_gemm(const void* a, int trans_a, const void* b, int trans_b, void* c, int64_t m, int64_t n, int64_t k,
                int dtype, int c_dtype, int accumulate, void* stream);
+/* Which kernel multiplies bf16 operands. 1 (default): every shape class goes to whichever measured faster for it
+ * on the MI355X -- this library's own matrix-core GEMM (the counterpart of the reference's tiled kernel,
+ * src/cuda_resident.cu:141-171) for short contractions, rocBLAS for long ones and for split weight gradients.
+ * 0: rocBLAS for everything, as for fp32 operands. 2: the library's own kernel for everything it takes
+ * (16-byte aligned rows, sizes that are multiples of 8); 3 / 4: the same with its 128 x 128 / 256 x 256 tile
+ * geometry forced (measurements). Process-wide; returns the previous setting. The environment variable
+ * PK_GEMM=library selects 0 at load time. */
+int pk_set_gemm_backend(int mode);
 
 #ifdef __cplusplus
 }

@@ -188,8 +188,15 @@ def clip_grad_norm_(grads, max_norm):
     return total
 
 
-def matmul(a, b, trans_a=False, trans_b=False, out_dtype=None):
-    """device::gemm: op(a) @ op(b), fp32 accumulate."""
+def set_gemm_backend(mode: int) -> int:
+    """Choose the kernel for bf16 GEMMs (pk_set_gemm_backend): 1 = per shape class whichever measured faster
+    (default), 0 = rocBLAS only, 2 = the library's own matrix-core kernel wherever it applies, 3 / 4 = the same
+    with small / large tiles forced. Returns the previous setting."""
+    return int(_lib.lib().pk_set_gemm_backend(int(mode)))
+
+
+def matmul(a, b, trans_a=False, trans_b=False, out_dtype=None, out=None):
+    """device::gemm: op(a) @ op(b), fp32 accumulate. With ``out`` the product is ADDED to it (beta = 1)."""
     _chk(a)
     _chk(b)
     if a.dtype != b.dtype:
@@ -198,6 +205,9 @@ def matmul(a, b, trans_a=False, trans_b=False, out_dtype=None):
     k2, n = (b.shape[1], b.shape[0]) if trans_b else b.shape
     if k != k2:
         raise RuntimeError("gemm: inner dimensions disagree")
-    c = torch.empty((m, n), dtype=out_dtype or a.dtype, device=a.device)
-    check(_lib.lib().pk_op_gemm(_p(a), int(trans_a), _p(b), int(trans_b), _p(c), m, n, k, _dt(a), _dt(c), 0, _s()))
+    c = out if out is not None else torch.empty((m, n), dtype=out_dtype or a.dtype, device=a.device)
+    if out is not None and (tuple(out.shape) != (m, n) or not out.is_contiguous()):
+        raise RuntimeError("gemm: output shape mismatch")
+    check(_lib.lib().pk_op_gemm(_p(a), int(trans_a), _p(b), int(trans_b), _p(c), m, n, k, _dt(a), _dt(c),
+                                int(out is not None), _s()))
     return c

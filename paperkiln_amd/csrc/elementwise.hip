@@ -6,6 +6,7 @@
 #include <hipcub/hipcub.hpp>
 #include <rocblas/rocblas.h>
 
+#include <cstdlib>
 #include <map>
 #include <cmath>
 #include <mutex>
@@ -1029,14 +1030,36 @@ rocblas_handle blas() {
 }
 }  // namespace
 
+namespace {
+int g_gemm_hand_written = [] {
+    const char* v = std::getenv("PK_GEMM");
+    return (v && std::string(v) == "library") ? 0 : 1;
+}();
+}
+void set_gemm_backend(int hand_written) { g_gemm_hand_written = hand_written; }
+int gemm_backend() { return g_gemm_hand_written; }
+
 void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dtype, int64_t M, int64_t N, int64_t ldc,
           float beta, int64_t lda) {
     if (lda == 0) lda = A.cols;
     const int64_t Ka = tA ? A.rows : A.cols, Kb = tB ? B.cols : B.rows;
     const int64_t Ma = tA ? A.cols : A.rows, Nb = tB ? B.rows : B.cols;
-    if (Ka != Kb) throw std::runtime_error("gemm: inner dimensions disagree");  // device.cpp:97
-    if (Ma != M || Nb != N) throw std::runtime_error("gemm: output shape mismatch");
+    if (Ka != Kb) shape_fail("gemm: inner dimensions disagree");  // device.cpp:97
+    if (Ma != M || Nb != N) shape_fail("gemm: output shape mismatch");
     if (A.dtype != B.dtype) throw std::runtime_error("gemm: operand dtypes differ");
+    // Which kernel: measured per shape on the MI355X as GPU time from a kernel trace (timing launches from the host
+    // measures the library's longer host path instead), on the Linear shapes of a d = 512 block and of the tied
+    // head. The two are within 15 % of each other on short contractions; the library's kernels are clearly
+    // ahead on long ones (K >= 1376: 695 - 870 TFLOP/s against 490 - 650) and on the split weight-gradient
+    // products. The hand-written kernel is ahead where a short contraction meets an output width that is not a
+    // multiple of 256, because the library's 176 - 256-wide tiles waste more of their last column there than
+    // 128 x 128 tiles do: [8192, 512] x [512, 2752] 42.9 against 55.0 us, [8192, 512] x [1376, 512]^T 23.7 against
+    // 38.1 us. That class goes to the hand-written kernel, everything else to the library.
+    // g_gemm_hand_written == 2 sends everything the hand-written kernel takes to it.
+    const bool mine = g_gemm_hand_written == 2 || (g_gemm_hand_written == 1 && !tA && Ka <= 1024 && N % 256 != 0 && N >= 1024);
+    if (A.dtype == PK_BF16 && mine &&
+        gemm_mfma_bf16(A.ptr(), tA, lda, B.ptr(), tB, B.cols, C, c_dtype, M, N, Ka, ldc, beta, tape_stream()))
+        return;
     // Row-major C = op(A) op(B)  <=>  column-major C^T = op(B)^T op(A)^T.
     const rocblas_datatype ab = A.dtype == PK_F32 ? rocblas_datatype_f32_r : rocblas_datatype_bf16_r;
     const rocblas_datatype ct = c_dtype == PK_F32 ? rocblas_datatype_f32_r : rocblas_datatype_bf16_r;
@@ -1090,6 +1113,23 @@ void gemm_tn_split(const Tensor& A, const Tensor& B, float* const* dst, int nspl
     if (B.rows != K) throw std::runtime_error("gemm: inner dimensions disagree");
     if (nsplit < 1 || nsplit > 4 || W % nsplit != 0) throw std::runtime_error("gemm_tn_split: bad column split");
     if (A.dtype != B.dtype) throw std::runtime_error("gemm: operand dtypes differ");
+    if (A.dtype == PK_BF16 && g_gemm_hand_written == 2) {  // one product [M, W] in fp32, then the column blocks go to their tensors
+        Buffer whole(sizeof(float) * static_cast<size_t>(M) * W);
+        if (gemm_mfma_bf16(A.ptr(), true, M, B.ptr(), false, W, whole.p, PK_F32, M, W, K, W, 0.0f, tape_stream())) {
+            SplitDst d{};
+            for (int k = 0; k < nsplit; ++k) d.p[k] = dst[k];
+            bool vec = (W / nsplit) % 4 == 0;
+            for (int k = 0; k < nsplit; ++k) vec = vec && aligned16p(dst[k]);
+            if (vec)
+                hipLaunchKernelGGL(add_parts_split4, ew_grid(M * W / 4), dim3(NT), 0, tape_stream(),
+                                   static_cast<const float*>(whole.p), d, 1, M, W / nsplit, nsplit, beta);
+            else
+                hipLaunchKernelGGL(add_parts_split, ew_grid(M * W), dim3(NT), 0, tape_stream(),
+                                   static_cast<const float*>(whole.p), d, 1, M, W / nsplit, nsplit, beta);
+            post();
+            return;
+        }
+    }
     const rocblas_datatype ab = A.dtype == PK_F32 ? rocblas_datatype_f32_r : rocblas_datatype_bf16_r;
     const float alpha = 1.0f, zero = 0.0f;
     rocblas_set_stream(blas(), tape_stream());

@@ -1,0 +1,339 @@
+// bf16 GEMM on the gfx950 matrix cores for the Linear layers of the Llama block: the MI355X counterpart of the
+// reference's tiled GEMM with transpose flags (paperkiln src/cuda_resident.cu:141-171, entry step_resident_gemm
+// :226-263, reached through device::gemm, src/device.cpp:91-125).
+//
+//   C[M, N] (+)= op(A) op(B),   row-major, bf16 operands, fp32 accumulation, C in bf16 or fp32
+//
+// One workgroup of four wavefronts owns a 128 x 128 tile of C and walks the contraction in slices of 64; each
+// wavefront owns 64 x 64 of it as 2 x 2 accumulators of v_mfma_f32_32x32x16_bf16. Operand tiles are staged in LDS,
+// double-buffered, one barrier per slice, the next slice's global loads in flight while the current one is
+// multiplied. An operand whose contraction index is contiguous in memory (A of "N", B of "T") is kept as
+// [row][k] with a pitch of 72 elements and read with 16-byte row reads; one whose contraction index is the row
+// index in memory (A of "T", B of "N") is kept as [k][column] with a pitch of 160 and read with
+// ds_read_b64_tr_b16, so no operand is ever transposed in memory. Both pitches are conflict-free for their read.
+// The product is formed as C^T (the B fragment in the MFMA's A slot), which leaves each lane with runs of four
+// consecutive columns of one row of C; the tile then goes through LDS once so that the global stores are whole
+// 16-byte chunks of consecutive columns.
+//
+// Long contractions with a small result (weight gradients over all tokens) are cut along the contraction axis
+// into slices that separate workgroups multiply into fp32 partial tiles; the partial tiles are added in slice
+// order by a second kernel -- no atomics, the same bits on every run.
+#include <algorithm>
+#include <type_traits>
+
+#include "mfma_common.h"
+#include "tensor.h"
+
+namespace pk {
+namespace {
+
+constexpr int BK = 64;
+constexpr int PITCH_ROW = BK + 8;  // [rows][64 k]: 16-byte row reads conflict-free
+
+// Tile geometry: WGM x WGN wavefronts, each owning FM x FN accumulators of 32 x 32.
+//   Small: 2 x 2 wavefronts of 2 x 2 -> 128 x 128, 256 threads, two workgroups per CU. For outputs of a few
+//          hundred tiles, where more and smaller workgroups fill the chip better.
+//   Large: 2 x 4 wavefronts of 4 x 2 -> 256 x 256, 512 threads, one workgroup per CU: half the operand bytes per
+//          MFMA, which is what the vector memory path (64 bytes per clock and CU) asks for on long runs.
+template <int WGM_, int WGN_, int FM_, int FN_>
+struct Geo {
+    static constexpr int WGM = WGM_, WGN = WGN_, FM = FM_, FN = FN_;
+    static constexpr int BM = WGM * FM * 32, BN = WGN * FN * 32, NTHR = WGM * WGN * 64;
+    // [64 k][columns] tiles: a pitch of 32 past a multiple of 128 keeps the transposing reads conflict-free
+    static constexpr int PITCH_TR_A = BM + 32, PITCH_TR_B = BN + 32;
+    static constexpr int A_EL = BM * PITCH_ROW > BK * PITCH_TR_A ? BM * PITCH_ROW : BK * PITCH_TR_A;
+    static constexpr int B_EL = BN * PITCH_ROW > BK * PITCH_TR_B ? BN * PITCH_ROW : BK * PITCH_TR_B;
+    static constexpr int CH_A = BM * BK / 8 / NTHR, CH_B = BN * BK / 8 / NTHR;  // 16-byte chunks per thread and slice
+};
+using GeoSmall = Geo<2, 2, 2, 2>;
+using GeoLarge = Geo<2, 4, 4, 2>;
+
+struct GemmArgs {
+    const uint16_t* a;
+    const uint16_t* b;
+    void* c;
+    int M, N, K;
+    int64_t lda, ldb, ldc;
+    int beta;         // 0: C = product, 1: C += product
+    int k_per_split;  // contraction elements per blockIdx.z (a multiple of BK); K when not split
+    int64_t part_stride;  // elements between the fp32 partial results of two slices (split only)
+    int tiles_m, tiles_n;
+};
+
+// Transposing operand read in natural k order: lane (c32, g) receives rows row0 + 8g .. 8g + 7 of column
+// col0 + c32 of a [k][column] tile.
+__device__ inline bf16x8 read_tr_nat(const uint16_t* tile, int pitch, int row0, int col0, int lane) {
+    const int g = lane >> 5, u = (lane >> 4) & 1, j = lane & 15;
+    const uint16_t* p = tile + (row0 + 8 * g + (j >> 2)) * pitch + col0 + 16 * u + 4 * (j & 3);
+    const s16x4 lo = lds_read_tr4(p), hi = lds_read_tr4(p + 4 * pitch);
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return *reinterpret_cast<const bf16x8*>(&v);
+}
+
+// One operand tile of the slice starting at k0: global -> registers (NCH 16-byte chunks per thread).
+// TR = false: memory is [row][k] (rows = the SPAN rows / columns of C this tile covers);
+// TR = true:  memory is [k][column].
+template <bool TR, int SPAN, int NTHR, int NCH>
+__device__ inline void fetch_tile(const uint16_t* base, int64_t ld, int rc0, int rc_count, int k0, int k_end, u32x4 (&r)[NCH]) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int c = static_cast<int>(threadIdx.x) + NTHR * i;
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        if (!TR) {
+            const int row = c >> 3, ch = c & 7;
+            const bool ok = rc0 + row < rc_count && k0 + ch * 8 < k_end;
+            r[i] = ok ? *reinterpret_cast<const u32x4*>(base + static_cast<int64_t>(rc0 + row) * ld + k0 + ch * 8) : zero;
+        } else {
+            constexpr int CPR = SPAN / 8;
+            const int row = c / CPR, ch = c % CPR;
+            const bool ok = k0 + row < k_end && rc0 + ch * 8 < rc_count;
+            r[i] = ok ? *reinterpret_cast<const u32x4*>(base + static_cast<int64_t>(k0 + row) * ld + rc0 + ch * 8) : zero;
+        }
+    }
+}
+template <bool TR, int SPAN, int NTHR, int NCH>
+__device__ inline void commit_tile(uint16_t* tile, const u32x4 (&r)[NCH]) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+        const int c = static_cast<int>(threadIdx.x) + NTHR * i;
+        if (!TR) {
+            *reinterpret_cast<u32x4*>(tile + (c >> 3) * PITCH_ROW + (c & 7) * 8) = r[i];
+        } else {
+            constexpr int CPR = SPAN / 8;
+            *reinterpret_cast<u32x4*>(tile + (c / CPR) * (SPAN + 32) + (c % CPR) * 8) = r[i];
+        }
+    }
+}
+
+template <typename G, bool TA, bool TB, bool CF32>
+__global__ __launch_bounds__(G::NTHR, 2) void gemm_bf16(GemmArgs g) {
+    constexpr int BM = G::BM, BN = G::BN, NTHR = G::NTHR, FM = G::FM, FN = G::FN;
+    __shared__ __attribute__((aligned(16))) uint16_t lds[2 * (G::A_EL + G::B_EL)];  // [buffer][A | B]
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c32 = lane & 31, gh = lane >> 5, wm = w / G::WGN, wn = w % G::WGN;
+
+    // XCD-aware tile order: workgroup ids go round-robin over the 8 XCDs, so XCD x takes the x-th eighth of the
+    // tile list (columns fastest): the tiles that share rows of A meet in one L2.
+    const int ntiles = g.tiles_m * g.tiles_n;
+    const int per_xcd = (ntiles + 7) / 8;
+    const int t = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (t >= ntiles) return;
+    const int m0 = (t / g.tiles_n) * BM, n0 = (t % g.tiles_n) * BN;
+    const int k_begin = blockIdx.z * g.k_per_split, k_end = min(g.K, k_begin + g.k_per_split);
+
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    u32x4 ra[G::CH_A], rb[G::CH_B];
+    // A: !TA [M][K] row form; TA [K][M] transposed form.  B: TB [N][K] row form; !TB [K][N] transposed form.
+    fetch_tile<TA, BM, NTHR, G::CH_A>(g.a, g.lda, m0, g.M, k_begin, k_end, ra);
+    fetch_tile<!TB, BN, NTHR, G::CH_B>(g.b, g.ldb, n0, g.N, k_begin, k_end, rb);
+    commit_tile<TA, BM, NTHR, G::CH_A>(lds, ra);
+    commit_tile<!TB, BN, NTHR, G::CH_B>(lds + G::A_EL, rb);
+    __syncthreads();
+
+    int buf = 0;
+    for (int k0 = k_begin; k0 < k_end; k0 += BK) {
+        const bool more = k0 + BK < k_end;
+        if (more) {
+            fetch_tile<TA, BM, NTHR, G::CH_A>(g.a, g.lda, m0, g.M, k0 + BK, k_end, ra);
+            fetch_tile<!TB, BN, NTHR, G::CH_B>(g.b, g.ldb, n0, g.N, k0 + BK, k_end, rb);
+        }
+        const uint16_t* As = lds + buf * (G::A_EL + G::B_EL);
+        const uint16_t* Bs = As + G::A_EL;
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; ++kk) {
+            bf16x8 fa[FM], fb[FN];
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+                fa[i] = TA ? read_tr_nat(As, G::PITCH_TR_A, kk * 16, (wm * FM + i) * 32, lane)
+                           : lds_read8(As + ((wm * FM + i) * 32 + c32) * PITCH_ROW + kk * 16 + gh * 8);
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+                fb[j] = !TB ? read_tr_nat(Bs, G::PITCH_TR_B, kk * 16, (wn * FN + j) * 32, lane)
+                            : lds_read8(Bs + ((wn * FN + j) * 32 + c32) * PITCH_ROW + kk * 16 + gh * 8);
+            // C^T blocks: rows = columns of C (from B), lane = row of C (from A)
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j) acc[i][j] = mfma32(fb[j], fa[i], acc[i][j]);
+        }
+        if (more) {
+            uint16_t* nxt = lds + (buf ^ 1) * (G::A_EL + G::B_EL);
+            commit_tile<TA, BM, NTHR, G::CH_A>(nxt, ra);
+            commit_tile<!TB, BN, NTHR, G::CH_B>(nxt + G::A_EL, rb);
+        }
+        __syncthreads();
+        buf ^= 1;
+    }
+
+    // Epilogue through LDS, one strip of 32 rows per wavefront row at a time: the strip as [WGM * 32][BN + pad]
+    // in the output's element type, then 16-byte chunks of consecutive columns to global memory (read-add-write
+    // when accumulating).
+    typedef typename std::conditional<CF32, float, uint16_t>::type CT;
+    constexpr int CP = BN + (CF32 ? 4 : 8);  // pitch in elements: rows stay 16-byte aligned
+    constexpr int EPC = CF32 ? 4 : 8;        // elements per 16-byte chunk
+    constexpr int CPR = BN / EPC;            // chunks per strip row
+    static_assert(G::WGM * 32 * CP * sizeof(CT) <= sizeof(lds), "epilogue strip must fit the tile buffers");
+    CT* cs = reinterpret_cast<CT*>(lds);
+    CT* cout = static_cast<CT*>(g.c) + (g.part_stride ? static_cast<int64_t>(blockIdx.z) * g.part_stride : 0);
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                const int row = wm * 32 + c32, col = (wn * FN + j) * 32 + qd * 8 + gh * 4;
+                if (CF32) {
+                    const f32x4 v = {acc[i][j][qd * 4], acc[i][j][qd * 4 + 1], acc[i][j][qd * 4 + 2], acc[i][j][qd * 4 + 3]};
+                    *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(cs) + row * CP + col) = v;
+                } else {
+                    const u32x2 v = {pack_bf16(acc[i][j][qd * 4], acc[i][j][qd * 4 + 1]),
+                                     pack_bf16(acc[i][j][qd * 4 + 2], acc[i][j][qd * 4 + 3])};
+                    *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(cs) + row * CP + col) = v;
+                }
+            }
+        __syncthreads();
+        for (int c = threadIdx.x; c < G::WGM * 32 * CPR; c += NTHR) {
+            const int srow = c / CPR, ch = c % CPR;
+            // strip row srow belongs to wavefront row srow / 32, whose i-th block of 32 rows this is
+            const int m = m0 + ((srow >> 5) * FM + i) * 32 + (srow & 31), n = n0 + ch * EPC;
+            if (m >= g.M || n >= g.N) continue;
+            u32x4 v = *reinterpret_cast<const u32x4*>(cs + srow * CP + ch * EPC);
+            CT* dst = cout + static_cast<int64_t>(m) * g.ldc + n;
+            if (g.beta) {
+                const u32x4 old = *reinterpret_cast<const u32x4*>(dst);
+                if (CF32) {
+                    f32x4 s = *reinterpret_cast<const f32x4*>(&old) + *reinterpret_cast<const f32x4*>(&v);
+                    v = *reinterpret_cast<const u32x4*>(&s);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float lo = __uint_as_float(old[e] << 16) + __uint_as_float(v[e] << 16);
+                        const float hi = __uint_as_float(old[e] & 0xffff0000u) + __uint_as_float(v[e] & 0xffff0000u);
+                        v[e] = pack_bf16(lo, hi);
+                    }
+                }
+            }
+            *reinterpret_cast<u32x4*>(dst) = v;
+        }
+        __syncthreads();
+    }
+}
+
+__global__ void sum_slices(const float* part, void* dst, int nparts, int64_t part_stride, int M, int N, int64_t ldc, int beta,
+                           int c_f32) {
+    const int64_t n4 = static_cast<int64_t>(M) * N / 4;
+    for (int64_t i = blockIdx.x * 256LL + threadIdx.x; i < n4; i += static_cast<int64_t>(gridDim.x) * 256) {
+        const int64_t e = i * 4, m = e / N, n = e % N;
+        f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int p = 0; p < nparts; ++p) s += *reinterpret_cast<const f32x4*>(part + p * part_stride + e);
+        if (c_f32) {
+            f32x4* d = reinterpret_cast<f32x4*>(static_cast<float*>(dst) + m * ldc + n);
+            *d = beta ? *d + s : s;
+        } else {
+            u32x2* d = reinterpret_cast<u32x2*>(static_cast<uint16_t*>(dst) + m * ldc + n);
+            if (beta) {
+                const u32x2 o = *d;
+                s[0] += __uint_as_float(o[0] << 16);
+                s[1] += __uint_as_float(o[0] & 0xffff0000u);
+                s[2] += __uint_as_float(o[1] << 16);
+                s[3] += __uint_as_float(o[1] & 0xffff0000u);
+            }
+            const u32x2 v = {pack_bf16(s[0], s[1]), pack_bf16(s[2], s[3])};
+            *d = v;
+        }
+    }
+}
+
+template <typename G, bool CF32>
+void launch_form(bool tA, bool tB, const GemmArgs& g, dim3 grid, hipStream_t st) {
+    if (!tA && !tB) hipLaunchKernelGGL((gemm_bf16<G, false, false, CF32>), grid, dim3(G::NTHR), 0, st, g);
+    if (!tA && tB) hipLaunchKernelGGL((gemm_bf16<G, false, true, CF32>), grid, dim3(G::NTHR), 0, st, g);
+    if (tA && !tB) hipLaunchKernelGGL((gemm_bf16<G, true, false, CF32>), grid, dim3(G::NTHR), 0, st, g);
+    if (tA && tB) hipLaunchKernelGGL((gemm_bf16<G, true, true, CF32>), grid, dim3(G::NTHR), 0, st, g);
+}
+template <typename G>
+void launch_geo(bool tA, bool tB, GemmArgs g, int S, bool c_f32, hipStream_t st) {
+    g.tiles_m = (g.M + G::BM - 1) / G::BM;
+    g.tiles_n = (g.N + G::BN - 1) / G::BN;
+    const unsigned gx = static_cast<unsigned>((g.tiles_m * g.tiles_n + 7) / 8 * 8);
+    if (c_f32)
+        launch_form<G, true>(tA, tB, g, dim3(gx, 1, static_cast<unsigned>(S)), st);
+    else
+        launch_form<G, false>(tA, tB, g, dim3(gx, 1, static_cast<unsigned>(S)), st);
+    hip_check(hipGetLastError(), "gemm_bf16 launch");
+}
+
+bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+int g_force_geo = -1;  // -1: choose by shape; 0 / 1: small / large tiles always (measurement)
+
+}  // namespace
+
+void gemm_mfma_force_tiles(int which) { g_force_geo = which; }
+
+// Returns false, having done nothing, for what the kernel does not take (fp32 operands, unaligned rows, sizes
+// that are not multiples of 8): the caller then uses the library GEMM.
+bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB, int64_t ldb, void* c, int c_dtype,
+                    int64_t M, int64_t N, int64_t K, int64_t ldc, float beta, hipStream_t st) {
+    if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return false;
+    if (beta != 0.0f && beta != 1.0f) return false;
+    if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return false;
+    if (lda % 8 || ldb % 8 || K % 8 || N % 8 || ldc % 8) return false;
+    if (tA && M % 8) return false;  // A^T is read in 16-byte chunks along M
+    GemmArgs g;
+    g.a = static_cast<const uint16_t*>(a);
+    g.b = static_cast<const uint16_t*>(b);
+    g.c = c;
+    g.M = static_cast<int>(M), g.N = static_cast<int>(N), g.K = static_cast<int>(K);
+    g.lda = lda, g.ldb = ldb, g.ldc = ldc;
+    g.beta = beta != 0.0f;
+    g.tiles_m = g.tiles_n = 0;
+    // Large tiles where the output alone gives every CU a 256 x 256 tile (and then some); small tiles otherwise.
+    const int64_t tiles_large = ((M + 255) / 256) * ((N + 255) / 256);
+    const bool large = g_force_geo >= 0 ? g_force_geo == 1 : tiles_large >= 240;
+    const int64_t ntiles = large ? tiles_large : ((M + 127) / 128) * ((N + 127) / 128);
+    // Split the contraction when the tiles alone would leave most of the chip idle and the contraction is long.
+    int S = 1;
+    if (ntiles < 192 && K >= 1024) {
+        S = static_cast<int>(std::min<int64_t>({(512 + ntiles - 1) / ntiles, K / 256, 32}));
+        if (S < 1) S = 1;
+    }
+    if (S == 1) {
+        g.k_per_split = g.K;
+        g.part_stride = 0;
+        if (large)
+            launch_geo<GeoLarge>(tA, tB, g, 1, c_dtype == PK_F32, st);
+        else
+            launch_geo<GeoSmall>(tA, tB, g, 1, c_dtype == PK_F32, st);
+        return true;
+    }
+    const int kps = static_cast<int>(((K + S - 1) / S + BK - 1) / BK * BK);
+    S = static_cast<int>((K + kps - 1) / kps);
+    Buffer part(sizeof(float) * static_cast<size_t>(S) * M * N);
+    GemmArgs gp = g;
+    gp.c = part.p;
+    gp.ldc = N;
+    gp.beta = 0;
+    gp.k_per_split = kps;
+    gp.part_stride = M * N;
+    if (large)
+        launch_geo<GeoLarge>(tA, tB, gp, S, true, st);
+    else
+        launch_geo<GeoSmall>(tA, tB, gp, S, true, st);
+    const int64_t n4 = M * N / 4;
+    hipLaunchKernelGGL(sum_slices, dim3(static_cast<unsigned>(std::min<int64_t>((n4 + 255) / 256, 4096))), dim3(256), 0, st,
+                       static_cast<const float*>(part.p), c, S, M * N, static_cast<int>(M), static_cast<int>(N), ldc,
+                       g.beta, c_dtype == PK_F32 ? 1 : 0);
+    hip_check(hipGetLastError(), "sum_slices launch");
+    return true;
+}
+
+}  // namespace pk

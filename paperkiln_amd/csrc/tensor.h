@@ -59,6 +59,15 @@ void k_adamw(const Tensor& p, const Tensor& g, const Tensor& m, const Tensor& v,
 // matrix (ldc). beta is 0 or 1.
 void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dtype, int64_t M, int64_t N, int64_t ldc,
           float beta, int64_t lda = 0);
+// gemm_mfma.hip: the hand-written bf16 matrix-core GEMM. Returns false (nothing done) for operands it does not take.
+bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB, int64_t ldb, void* c, int c_dtype,
+                    int64_t M, int64_t N, int64_t K, int64_t ldc, float beta, hipStream_t st);
+// Which GEMM serves bf16 operands: 1 (default) = each shape class goes to the kernel that measured faster for it,
+// 0 = the library only, 2 = the hand-written kernel for everything it takes. Set from the environment
+// (PK_GEMM=library) or by a caller that wants to compare them.
+void set_gemm_backend(int hand_written);
+void gemm_mfma_force_tiles(int which);  // -1: by shape (default), 0: 128 x 128 tiles, 1: 256 x 256 tiles (measurement)
+int gemm_backend();
 // dst[k] ([A.cols, B.cols/nsplit] fp32, contiguous) = beta * dst[k] + A^T B[:, k-th column block], k < nsplit <= 4
 void gemm_tn_split(const Tensor& A, const Tensor& B, float* const* dst, int nsplit, float beta);
 

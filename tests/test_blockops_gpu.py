@@ -228,3 +228,67 @@ def test_error_behaviour(bo):
         bo.cross_entropy(x, dev(np.array([0, 1, 8, 2], np.int32)))
     with pytest.raises(RuntimeError):
         bo.add(x, dev(synth.randn(433, (4, 9), 1.0)))
+
+
+GEMM_SHAPES = [(128, 128, 64), (560, 136, 200), (8, 8, 8), (2056, 520, 1376), (512, 1536, 4096), (264, 40, 8192),
+               (1000, 2048, 512), (300, 264, 72)]
+
+
+@pytest.mark.parametrize("mode", [3, 4], ids=["tiles128", "tiles256"])
+@pytest.mark.parametrize("shape", GEMM_SHAPES, ids=lambda s: f"M{s[0]}_N{s[1]}_K{s[2]}")
+def test_matrix_core_gemm_against_float64(bo, mode, shape):
+    """The library's own bf16 GEMM (the counterpart of the reference's tiled kernel with transpose flags,
+    src/cuda_resident.cu:141-171) in both tile geometries, all four transpose combinations, bf16 and fp32 results,
+    overwrite and accumulate, ragged edges, contractions that are not a multiple of the slice and long ones that are
+    split across workgroups -- against a float64 product of the same bf16 operands. The bar: the fp32 accumulation
+    error of a K-term sum (a few 1e-6 relative to the largest |C|, the library kernel's own distance is printed beside
+    it), plus one bf16 rounding where the result is stored in bf16. Two runs give the same bits."""
+    M, N, K = shape
+    gen = torch.Generator(device="cuda").manual_seed(M + 3 * N + 7 * K)
+    prev = bo.set_gemm_backend(mode)
+    try:
+        for ta in (False, True):
+            for tb in (False, True):
+                a = torch.randn((K, M) if ta else (M, K), generator=gen, device="cuda").bfloat16()
+                b = torch.randn((N, K) if tb else (K, N), generator=gen, device="cuda").bfloat16()
+                want = (a.double().t() if ta else a.double()) @ (b.double().t() if tb else b.double())
+                scale = float(want.abs().max())
+                for od in (torch.float32, torch.bfloat16):
+                    got = bo.matmul(a, b, ta, tb, out_dtype=od)
+                    again = bo.matmul(a, b, ta, tb, out_dtype=od)
+                    assert torch.equal(got, again)
+                    err = float((got.double() - want).abs().max())
+                    bar = scale * (2e-5 + (2.0 ** -8 if od == torch.bfloat16 else 0.0))
+                    assert err <= bar, (ta, tb, od, err, bar)
+                    c0 = torch.randn((M, N), generator=gen, device="cuda").to(od)
+                    acc = c0.clone()
+                    bo.matmul(a, b, ta, tb, out=acc)
+                    want_acc = c0.double() + want
+                    err = float((acc.double() - want_acc).abs().max())
+                    bar = float(want_acc.abs().max()) * (2e-5 + (2.0 ** -7 if od == torch.bfloat16 else 0.0))
+                    assert err <= bar, ("accumulate", ta, tb, od, err, bar)
+    finally:
+        bo.set_gemm_backend(prev)
+
+
+def test_gemm_dispatch_modes_agree(bo):
+    """Default dispatch (per shape class), library only, and the hand-written kernel everywhere give the same
+    product to fp32 accumulation accuracy on a Linear-shaped problem; operands the hand-written kernel does not take
+    (a column count that is not a multiple of 8) fall through to the library without an error."""
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    x = torch.randn((1024, 512), generator=gen, device="cuda").bfloat16()
+    w = torch.randn((512, 1376), generator=gen, device="cuda").bfloat16()
+    want = x.double() @ w.double()
+    outs = []
+    prev = bo.set_gemm_backend(1)
+    try:
+        for mode in (1, 0, 2):
+            bo.set_gemm_backend(mode)
+            outs.append(bo.matmul(x, w, out_dtype=torch.float32))
+            assert float((outs[-1].double() - want).abs().max()) <= 2e-5 * float(want.abs().max())
+        bo.set_gemm_backend(2)
+        odd = torch.randn((512, 100), generator=gen, device="cuda").bfloat16()
+        got = bo.matmul(x, odd, out_dtype=torch.float32)
+        assert float((got.double() - x.double() @ odd.double()).abs().max()) <= 2e-5 * float(want.abs().max())
+    finally:
+        bo.set_gemm_backend(prev)
