@@ -145,7 +145,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
             if (threadIdx.x < BMQ) {
                 const int t = min(q0 + static_cast<int>(threadIdx.x), a.T - 1);
                 const int64_t lrow = (static_cast<int64_t>(b) * a.Hq + h) * a.T + t;
-                lse_r = -a.lse[lrow] * LOG2E;
+                lse_r = a.lse[lrow];  // scaled when it is stored: arithmetic on it here would wait for every load just issued
                 dl_r = a.delta[lrow];
             }
         };
@@ -163,7 +163,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
                 *reinterpret_cast<u32x4*>(dOs[slot] + row * S + ch * 8) = gr[i];
             }
             if (tid < BMQ) {
-                nlse_s[slot][tid] = lse_r;
+                nlse_s[slot][tid] = -lse_r * LOG2E;
                 dl_s[slot][tid] = dl_r;
             }
         };

@@ -473,7 +473,7 @@ __global__ __launch_bounds__(512, 1) void f32_dkdv(AttnArgs a) {
         if (threadIdx.x < BQ) {
             const int t = min(q0 + static_cast<int>(threadIdx.x), a.T - 1);
             const int64_t lrow = (static_cast<int64_t>(b) * a.Hq + h) * a.T + t;
-            lse_r = -a.lse[lrow] * LOG2E;
+            lse_r = a.lse[lrow];  // scaled when it is stored: arithmetic on it here would wait for every load just issued
             dl_r = a.delta[lrow];
         }
     };
@@ -488,7 +488,7 @@ __global__ __launch_bounds__(512, 1) void f32_dkdv(AttnArgs a) {
             }
         }
         if (threadIdx.x < BQ) {
-            nlse_s[slot][threadIdx.x] = lse_r;
+            nlse_s[slot][threadIdx.x] = -lse_r * LOG2E;
             dl_s[slot][threadIdx.x] = dl_r;
         }
     };
