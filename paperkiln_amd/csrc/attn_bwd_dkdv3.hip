@@ -27,6 +27,19 @@
 // read of them (passes + 3 = 11 issue slots for the 8-pass 32x32x16) are the program's to
 // provide -- by the software pipeline's own distances on the fast path, by s_nop on the
 // edge path and before the epilogue.
+//
+// What a wavefront that has its SIMD to itself pays for (measured with a stream of
+// independent matrix instructions and N other instructions between each pair): the matrix
+// instruction occupies the pipe for 32 clocks and the issue port for about 8; an ordinary
+// vector instruction takes about 5 clocks of issue (8 when it reads the result of the one
+// before, 8.6 for v_exp_f32), a scalar one about the same. So a matrix instruction hides
+// five vector instructions and not one more, and nothing here is free: the loop below is
+// written to issue as few instructions as possible. LDS addresses are a per-lane register
+// plus an immediate, positions in memory are pointers that are advanced rather than
+// recomputed, -delta enters the dP tile as the matrix instruction's own C operand, and
+// what must run between two phases is kept to the eight pack instructions the next phase
+// needs at once. LDS reads, LDS writes and global loads cost their issue slot and no more
+// when the matrix pipe is the bound (one per four matrix instructions measured free).
 #include <type_traits>
 
 #include "mfma_common.h"
@@ -39,10 +52,16 @@ constexpr float LOG2E = 1.4426950408889634f;
 constexpr int BMQ = 64;   // queries per step
 constexpr int BNK = 128;  // keys per workgroup (4 blocks of 32)
 typedef __fp16 h16x2 __attribute__((ext_vector_type(2)));
+// typed LDS pointer from a 32-bit LDS byte address
+#define LDSP(T, addr) (reinterpret_cast<PK_LDS T*>(static_cast<uintptr_t>(addr)))
 
 // t = a . b            (fresh score tile in ordinary registers)
 __device__ __forceinline__ void mma_v0(f32x16& t, bf16x8 a, bf16x8 b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(t) : "v"(a), "v"(b));
+}
+// t = a . b + c        (fresh score tile started from a tile of constants)
+__device__ __forceinline__ void mma_vc(f32x16& t, bf16x8 a, bf16x8 b, const f32x16& c) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %3" : "=&v"(t) : "v"(a), "v"(b), "v"(c));
 }
 // t += a . b           (score tile, ordinary registers)
 __device__ __forceinline__ void mma_v(f32x16& t, bf16x8 a, bf16x8 b) {
@@ -74,7 +93,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
     constexpr int CPT = BMQ * NCH / 256;  // chunks per thread per tensor per step
     __shared__ __attribute__((aligned(16))) uint16_t Qs[3][BMQ * S];
     __shared__ __attribute__((aligned(16))) uint16_t dOs[3][BMQ * S];
-    __shared__ __attribute__((aligned(16))) uint16_t Pbuf[2][2][4][64 * 16];  // [step parity][query block][key block][lane][16]
+    __shared__ __attribute__((aligned(16))) uint16_t Pbuf[2][2][4][64 * 16];  // [step parity][query block][key block][half][lane][8]
     __shared__ __attribute__((aligned(16))) float nlse_s[3][BMQ];            // -LSE * log2(e)
     __shared__ __attribute__((aligned(16))) float dl_s[3][BMQ];
 
@@ -148,41 +167,54 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
             offq[i] = static_cast<uint32_t>(frow + RPI * i) * q_st2 + fch16;
             offg[i] = static_cast<uint32_t>(frow + RPI * i) * do_st2 + fch16;
         }
-        int f_h = 0, f_qt = 0;  // head inside the group and query tile of the next fetch
         // A tile is fetched and committed in CPT pieces (one 16-byte chunk of Q and one of dO per thread each), so
         // that the step loop can drop one piece into the shadow of a matrix instruction. The pieces have no
         // branch: rows past the end of the sequence re-read the last row (their P is masked to zero), a fetch
         // past the last step re-reads the last tile, and a commit past it fills a slot nobody reads.
-        const char *f_qb = nullptr, *f_gb = nullptr;  // scalar bases of the tile being fetched
-        uint32_t f_limq = 0, f_limg = 0;              // offsets of this thread's chunk in the last row that exists
+        //
+        // The position of the next fetch is kept as pointers that are advanced, not recomputed: one wavefront
+        // per SIMD issues every instruction of its own, scalar ones included, at about five clocks each.
+        int f_h = 0, f_qt = 0;       // head inside the group and query tile of the next fetch
+        int f_q0 = qt_lo * BMQ;      // first query row of that tile
+        const int h0 = hk * rep;
+        const char* f_qb = reinterpret_cast<const char*>(a.q) + (b * a.q_sb + h0 * a.q_sh + f_q0 * a.q_st) * 2;
+        const char* f_gb = reinterpret_cast<const char*>(a.d_o) + (b * a.do_sb + h0 * a.do_sh + f_q0 * a.do_st) * 2;
         // per-row scalars: wavefronts 0 and 1 carry LSE of rows 32w + lane (lanes 0-31), wavefronts 2 and 3 delta
         const float* const r_arr = w < 2 ? a.lse : a.delta;
-        const float r_mul = w < 2 ? -LOG2E : 1.0f;
+        const float r_mul = w < 2 ? -LOG2E : -1.0f;  // what the LDS holds: -LSE log2(e) and -delta
         const int rrow = (w & 1) * 32 + (lane & 31);
-        const float* f_rb = nullptr;  // row 0 of the tile in that array
+        const char* f_rb = reinterpret_cast<const char*>(r_arr + ((static_cast<int64_t>(b) * a.Hq + h0) * a.T + f_q0));
+        // steps from one tile to the next: inside a head, and from the last tile of a head to the first of the next
+        const int64_t qd_tile = BMQ * a.q_st * 2, qd_head = a.q_sh * 2 - (nqt - 1) * qd_tile;
+        const int64_t gd_tile = BMQ * a.do_st * 2, gd_head = a.do_sh * 2 - (nqt - 1) * gd_tile;
+        const int64_t rd_tile = BMQ * 4, rd_head = static_cast<int64_t>(a.T) * 4 - (nqt - 1) * rd_tile;
+        uint32_t f_limq = 0, f_limg = 0;  // offsets of this thread's chunk in the last row that exists
         uint32_t f_roff = 0;
         float row_r = 0.0f;
+        const char *c_qb = f_qb, *c_gb = f_gb, *c_rb = f_rb;  // the tile being fetched
         auto fetch_setup = [&]() {  // steps are fetched in order
-            const int h = hk * rep + f_h, q0 = (qt_lo + f_qt) * BMQ;
-            if (f_qt + 1 < nqt)
-                ++f_qt;
-            else if (f_h + 1 < rep)
-                f_qt = 0, ++f_h;
-            const int last = min(BMQ - 1, a.T - 1 - q0);
+            c_qb = f_qb, c_gb = f_gb, c_rb = f_rb;
+            const int last = min(BMQ - 1, a.T - 1 - f_q0);
             f_limq = static_cast<uint32_t>(last) * q_st2 + fch16;
             f_limg = static_cast<uint32_t>(last) * do_st2 + fch16;
             f_roff = static_cast<uint32_t>(min(rrow, last)) * 4u;
-            f_qb = reinterpret_cast<const char*>(a.q) + (b * a.q_sb + h * a.q_sh + q0 * a.q_st) * 2;
-            f_gb = reinterpret_cast<const char*>(a.d_o) + (b * a.do_sb + h * a.do_sh + q0 * a.do_st) * 2;
-            f_rb = r_arr + ((static_cast<int64_t>(b) * a.Hq + h) * a.T + q0);
+            // masks instead of selects: a nested select becomes a branch, and a taken branch costs the most of all
+            const int64_t in_head = -static_cast<int64_t>(f_qt + 1 < nqt);
+            const int64_t next_head = ~in_head & -static_cast<int64_t>(f_h + 1 < rep);
+            f_qb += (qd_tile & in_head) | (qd_head & next_head);
+            f_gb += (gd_tile & in_head) | (gd_head & next_head);
+            f_rb += (rd_tile & in_head) | (rd_head & next_head);
+            f_q0 += (BMQ & static_cast<int>(in_head)) | (-(nqt - 1) * BMQ & static_cast<int>(next_head));
+            f_qt = (f_qt + 1) & static_cast<int>(in_head) | f_qt & static_cast<int>(~(in_head | next_head));
+            f_h -= static_cast<int>(next_head);
         };
         auto fetch_q = [&](int i) {  // global -> registers
-            qr[i] = *reinterpret_cast<const u32x4*>(f_qb + min(offq[i], f_limq));
+            qr[i] = *reinterpret_cast<const u32x4*>(c_qb + min(offq[i], f_limq));
             // scaled when it is stored: arithmetic on it here would wait for every load just issued
-            if (i == 0 && lane < 32) row_r = *reinterpret_cast<const float*>(reinterpret_cast<const char*>(f_rb) + f_roff);
+            if (i == 0 && lane < 32) row_r = *reinterpret_cast<const float*>(c_rb + f_roff);
         };
         auto fetch_g = [&](int i) {
-            gr[i] = *reinterpret_cast<const u32x4*>(f_gb + min(offg[i], f_limg));
+            gr[i] = *reinterpret_cast<const u32x4*>(c_gb + min(offg[i], f_limg));
         };
         auto fetch_piece = [&](int i) {
             fetch_q(i);
@@ -254,11 +286,21 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
             fetch();
             __syncthreads();
         }
+        // LDS positions as 32-bit byte addresses: a lane's own part is formed once, the ring slot is added once a
+        // step, and every read below is that register plus a constant the instruction carries.
+        auto lds32 = [](const void* p) { return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p)); };
+        constexpr uint32_t SLOTB = BMQ * S * 2;
+        const uint32_t x_slot0 = lds32(rl == 0 ? Qs[0] : dOs[0]), y_slot0 = lds32(rl == 0 ? dOs[0] : Qs[0]);
+        const uint32_t x_lane = static_cast<uint32_t>(c32 * S + g * 8) * 2u;  // GEMM1: row c32, 8 elements from 8g
+        const int tj = lane & 15, tu = (lane >> 4) & 1;
+        const uint32_t y_lane = static_cast<uint32_t>((4 * g + (tj >> 2)) * S + TrMap<D>::src_col(0, tu, tj & 3)) * 2u;
+        const uint32_t rc_lane = lds32(rl == 0 ? nlse_s[0] : dl_s[0]) + g * 16u;
+        const uint32_t p_lane = lds32(Pbuf) + khalf * 2u * 2048u + lane * 16u;  // [parity][qb][khalf*2+kb][half][lane][8]
+        static_assert(TrMap<D>::src_col(1, 0, 0) - TrMap<D>::src_col(0, 0, 0) == 8, "block db starts 8 columns on");
+        int c_qt = 0, slot3 = 0, cslot = (rl + 1) % 3;  // query tile of this step, its ring slot, the slot staged into
         for (int stp = 0; stp < steps; ++stp) {
-            const int cslot = (stp + rl + 1) % 3;
             {
-  // role 1 runs one step behind
-                const int qbase = (qt_lo + stp % nqt) * BMQ;
+                const int qbase = (qt_lo + c_qt) * BMQ;
                 bool full[2];
 #pragma unroll
                 for (int qb = 0; qb < 2; ++qb) {
@@ -266,20 +308,26 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     full[qb] = qhi < a.T && kw0 + 63 < a.T && (!a.causal || kw0 + 63 <= qlo);
                 }
                 constexpr int PF = 3, NS = 2 * KK;  // fragments in flight; slots (= MFMAs) per GEMM
-                const int slot3 = stp % 3;
-                const uint16_t* X = (rl == 0 ? Qs[slot3] : dOs[slot3]) + c32 * S + g * 8;  // GEMM1 rows
-                const uint16_t* Y = rl == 0 ? dOs[slot3] : Qs[slot3];                       // GEMM2, transposed
-                const float* rowc = (rl == 0 ? nlse_s[slot3] : dl_s[slot3]) + g * 4;
-                auto xfrag = [&](int qb, int j) { return lds_read8(X + qb * 32 * S + j * 16); };
+                const uint32_t xa = x_slot0 + slot3 * SLOTB + x_lane;
+                const uint32_t ya = y_slot0 + slot3 * SLOTB + y_lane;
+                const uint32_t rca = rc_lane + slot3 * (BMQ * 4u);
+                const uint32_t pa = p_lane + (stp & 1) * (2u * 4u * 2048u);
+                auto xfrag = [&](int qb, int j) { return *LDSP(const bf16x8, xa + (qb * 32 * S + j * 16) * 2); };
                 auto yfrag = [&](int qb, int j) {
-                    return lds_read_tr_operand_perm<D>(Y, S, qb * 32 + (j / DB) * 16, j % DB, lane);
+                    const uint32_t at = ya + ((qb * 32 + (j / DB) * 16) * S + 8 * (j % DB)) * 2;
+                    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDSP(s16x4, at));
+                    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDSP(s16x4, at + 8 * S * 2));
+                    typedef short s16x8 __attribute__((ext_vector_type(8)));
+                    const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    return *reinterpret_cast<const bf16x8*>(&v);
                 };
                 f32x16 t0[2], t1[2];          // S or dP of query block 0 / 1, [sub-block], as the matrix pipe leaves them
                 // The elementwise results live in scalars of their own: written back into the 16-register tuples
                 // under the role branch they would make every slot copy whole tuples at the join.
                 float e0[2][16], e1[2][16];   // P or dS of query block 0 / 1
                 bf16x8 op0[2][2], op1[2][2];  // packed P or dS, [sub-block][16-query half]
-                f32x4 rc[4];                  // per-row constants of the block being worked on
+                f32x4 rc[4];                  // role 0: -LSE log2(e) of the rows of the block being worked on
+                f32x16 nd0, nd1;              // role 1: -delta of the rows of query block 0 / 1, laid out like a score tile
                 u32x4 pr[2][2];               // role 1: P handed over, [sub-block][half]
                 bf16x8 fr[NS / 2 + PF];       // fragment window of the running GEMM
                 // elementwise work on elements [lo, hi) of a query block: sub-block e/16, register e%16
@@ -295,19 +343,26 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                         for (int e = lo; e < hi; ++e) {
                             const int kb = e >> 4, r = e & 15;
                             const h16x2* ph = reinterpret_cast<const h16x2*>(&pr[kb][0]);
-                            y[kb][r] = static_cast<float>(ph[r >> 1][r & 1]) * (t[kb][r] - rc[r >> 2][r & 3]);
+                            y[kb][r] = static_cast<float>(ph[r >> 1][r & 1]) * t[kb][r];  // t is dP - delta already
                         }
                     }
                 };
+                auto row_consts = [&](int qb, int qd) { return *LDSP(const f32x4, rca + (qb * 32 + qd * 8) * 4); };
+                auto minus_delta = [&](int qb) {  // role 1, before GEMM1 of the block: its accumulators start from -delta
+                    const f32x4 c0 = row_consts(qb, 0), c1 = row_consts(qb, 1), c2 = row_consts(qb, 2), c3 = row_consts(qb, 3);
+                    const f32x16 v = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3],
+                                      c2[0], c2[1], c2[2], c2[3], c3[0], c3[1], c3[2], c3[3]};
+                    return v;
+                };
                 auto side_loads = [&](int qb) {
+                    if (rl == 0) {
 #pragma unroll
-                    for (int qd = 0; qd < 4; ++qd) rc[qd] = *reinterpret_cast<const f32x4*>(rowc + qb * 32 + qd * 8);
-                    if (rl == 1) {
+                        for (int qd = 0; qd < 4; ++qd) rc[qd] = row_consts(qb, qd);
+                    } else {
 #pragma unroll
                         for (int kb = 0; kb < 2; ++kb) {
-                            const uint16_t* pb = Pbuf[stp & 1][qb][khalf * 2 + kb] + lane * 16;
-                            pr[kb][0] = *reinterpret_cast<const u32x4*>(pb);
-                            pr[kb][1] = *reinterpret_cast<const u32x4*>(pb + 8);
+                            pr[kb][0] = *LDSP(const u32x4, pa + qb * 8192 + kb * 2048);
+                            pr[kb][1] = *LDSP(const u32x4, pa + qb * 8192 + kb * 2048 + 1024);
                         }
                     }
                 };
@@ -316,8 +371,14 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                                pack_bf16(y[8 * h + 4], y[8 * h + 5]), pack_bf16(y[8 * h + 6], y[8 * h + 7])};
                     return *reinterpret_cast<bf16x8*>(&u);
                 };
-                auto finish = [&](int qb, float(&y)[2][16], bf16x8(&op)[2][2]) {
-                    if (rl == 0 && !full[qb]) {  // diagonal / ragged block: zero what the mask hides (role 1 inherits the zeros)
+                // What follows the elementwise work of a block -- masking on the diagonal, packing to bf16, handing P
+                // over -- would leave the matrix pipe idle if it ran between two phases. Only what the next phase
+                // needs at once stays there (finish_head: the first k-half of the packed operand); the rest rides in
+                // the first slots of that phase (finish_slot).
+                auto finish_head = [&](int qb, float(&y)[2][16], bf16x8(&op)[2][2]) {
+                    // diagonal / ragged block: zero what the mask hides (role 1 inherits the zeros). Marked unlikely so
+                    // that the common case falls through: jumping over the masking code is a taken branch
+                    if (__builtin_expect(rl == 0 && !full[qb], 0)) {
                         const int qlo = qbase + qb * 32;
 #pragma unroll
                         for (int kb = 0; kb < 2; ++kb)
@@ -325,29 +386,24 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                             for (int r = 0; r < 16; ++r)
                                 y[kb][r] = kvis[kb](qlo + (r >> 2) * 8 + g * 4 + (r & 3)) ? y[kb][r] : 0.0f;
                     }
+                    op[0][0] = pack8(y[0], 0);
+                    op[1][0] = pack8(y[1], 0);
+                };
+                auto finish_slot = [&](int qb, float(&y)[2][16], bf16x8(&op)[2][2], int sl) {
+                    if (sl < 2) op[sl][1] = pack8(y[sl], 1);  // first used in slot 8 + sl
+                    if (rl == 0 && sl >= 2 && sl < 6) {  // hand P over in fp16 (11 significant bits in [0, 1])
+                        const int kb = (sl - 2) >> 1, hf = (sl - 2) & 1;
+                        h16x2 ph[4];
 #pragma unroll
-                    for (int kb = 0; kb < 2; ++kb) {
-                        op[kb][0] = pack8(y[kb], 0);
-                        op[kb][1] = pack8(y[kb], 1);
-                    }
-                    if (rl == 0) {  // hand P over in fp16 (11 significant bits in [0, 1])
-#pragma unroll
-                        for (int kb = 0; kb < 2; ++kb) {
-                            uint16_t* pb = Pbuf[stp & 1][qb][khalf * 2 + kb] + lane * 16;
-                            h16x2 ph[8];
-#pragma unroll
-                            for (int i = 0; i < 8; ++i) {
-                                const f32x2 p2 = {y[kb][2 * i], y[kb][2 * i + 1]};
-                                ph[i] = __builtin_convertvector(p2, h16x2);
-                            }
-                            *reinterpret_cast<u32x4*>(pb) = *reinterpret_cast<u32x4*>(&ph[0]);
-                            *reinterpret_cast<u32x4*>(pb + 8) = *reinterpret_cast<u32x4*>(&ph[4]);
+                        for (int i = 0; i < 4; ++i) {
+                            const f32x2 p2 = {y[kb][8 * hf + 2 * i], y[kb][8 * hf + 2 * i + 1]};
+                            ph[i] = __builtin_convertvector(p2, h16x2);
                         }
+                        *LDSP(u32x4, pa + qb * 8192 + kb * 2048 + hf * 1024) = *reinterpret_cast<u32x4*>(&ph[0]);
                     }
                 };
                 // staging piece p rides in phase p+1, the two roles in different slots: a wavefront whose load finds
                 // the address unit's queue full stalls, matrix instructions and all, so the loads are spread thin
-                static_assert(CPT == 4 && NS >= 14, "one staging piece per phase");
                 auto stage = [&](int piece, int sl) {
                     constexpr int first = rl * 8;
                     if (sl == first + 1) commit_piece(cslot, piece);
@@ -356,13 +412,16 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                 };
                 fetch_setup();
                 // ---- phase 1: GEMM1(block 0)
+                if (rl == 1) nd0 = minus_delta(0);
 #pragma unroll
                 for (int j = 0; j < PF; ++j) fr[j] = xfrag(0, j);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int sl = 0; sl < NS; ++sl) {
                     const int j = sl >> 1, kb = sl & 1;
-                    if (j == 0)
+                    if (j == 0 && rl == 1)
+                        mma_vc(t0[kb], fr[j], kv[kb][j], nd0);
+                    else if (j == 0)
                         mma_v0(t0[kb], fr[j], kv[kb][j]);
                     else
                         mma_v(t0[kb], fr[j], kv[kb][j]);
@@ -372,13 +431,16 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                 }
                 // ---- phase 2: GEMM1(block 1) || elementwise(block 0)
                 side_loads(0);
+                if (rl == 1) nd1 = minus_delta(1);
 #pragma unroll
                 for (int j = 0; j < PF; ++j) fr[j] = xfrag(1, j);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int sl = 0; sl < NS; ++sl) {
                     const int j = sl >> 1, kb = sl & 1;
-                    if (j == 0)
+                    if (j == 0 && rl == 1)
+                        mma_vc(t1[kb], fr[j], kv[kb][j], nd1);
+                    else if (j == 0)
                         mma_v0(t1[kb], fr[j], kv[kb][j]);
                     else
                         mma_v(t1[kb], fr[j], kv[kb][j]);
@@ -389,7 +451,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     stage(1, sl);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                finish(0, e0, op0);
+                finish_head(0, e0, op0);
                 // ---- phase 3: GEMM2(block 0) || elementwise(block 1)
                 side_loads(1);
 #pragma unroll
@@ -401,10 +463,11 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     mma_a(acc[kb][j % DB], fr[j], op0[kb][j / DB]);
                     if (kb == 0 && j + PF < 2 * DB) fr[j + PF] = yfrag(0, j + PF);
                     elems(t1, e1, sl * 32 / NS, (sl + 1) * 32 / NS);
+                    finish_slot(0, e0, op0, sl);
                     stage(2, sl);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                finish(1, e1, op1);
+                finish_head(1, e1, op1);
                 // ---- phase 4: GEMM2(block 1) || staging, one piece per matrix instruction
 #pragma unroll
                 for (int j = 0; j < PF; ++j) fr[j] = yfrag(1, j);
@@ -414,10 +477,14 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     const int j = sl >> 1, kb = sl & 1;
                     mma_a(acc[kb][j % DB], fr[j], op1[kb][j / DB]);
                     if (kb == 0 && j + PF < 2 * DB) fr[j + PF] = yfrag(1, j + PF);
+                    finish_slot(1, e1, op1, sl);
                     stage(3, sl);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
+            c_qt = c_qt + 1 == nqt ? 0 : c_qt + 1;
+            slot3 = slot3 == 2 ? 0 : slot3 + 1;
+            cslot = cslot == 2 ? 0 : cslot + 1;
             __syncthreads();
         }
         if (rl == 0) __syncthreads();

@@ -99,13 +99,13 @@ template <int D>
 struct TrMap;
 template <>
 struct TrMap<128> {
-    __device__ static int src_col(int db, int u, int a) { return 4 * (8 * a + u + 2 * db); }
-    __device__ static int col0(int db, int qd, int g) { return 32 * (2 * (qd & 1) + g) + 4 * (qd >> 1) + 8 * db; }
+    __device__ static constexpr int src_col(int db, int u, int a) { return 4 * (8 * a + u + 2 * db); }
+    __device__ static constexpr int col0(int db, int qd, int g) { return 32 * (2 * (qd & 1) + g) + 4 * (qd >> 1) + 8 * db; }
 };
 template <>
 struct TrMap<64> {  // natural order
-    __device__ static int src_col(int db, int u, int a) { return 32 * db + 16 * u + 4 * a; }
-    __device__ static int col0(int db, int qd, int g) { return 32 * db + 8 * qd + 4 * g; }
+    __device__ static constexpr int src_col(int db, int u, int a) { return 32 * db + 16 * u + 4 * a; }
+    __device__ static constexpr int col0(int db, int qd, int g) { return 32 * db + 8 * qd + 4 * g; }
 };
 template <int D>
 __device__ inline bf16x8 lds_read_tr_operand_perm(const uint16_t* tile, int stride, int row0, int db,
