@@ -90,7 +90,10 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
     constexpr int KK = D / 16, DB = D / 32;
     constexpr int S = D + 8;            // tile row pitch (elements): 16-byte row reads conflict-free
     constexpr int NCH = D / 8;          // 16-byte chunks per row
-    constexpr int CPT = BMQ * NCH / 256;  // chunks per thread per tensor per step
+    // Threads that stage tiles: the two wavefronts of role 1. Role 0 carries the exponentials and is the longer
+    // of the two; with all four wavefronts staging (NSTG = 256) the step is 4 % slower.
+    constexpr int NSTG = 128;
+    constexpr int CPT = BMQ * NCH / NSTG;  // chunks per staging thread per tensor per step
     __shared__ __attribute__((aligned(16))) uint16_t Qs[3][BMQ * S];
     __shared__ __attribute__((aligned(16))) uint16_t dOs[3][BMQ * S];
     __shared__ __attribute__((aligned(16))) uint16_t Pbuf[2][2][4][64 * 16];  // [step parity][query block][key block][half][lane][8]
@@ -154,11 +157,12 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
         // themselves: a thread's position inside a tile is fixed (row tid / 16 + 16 i, chunk tid % 16), its byte
         // offsets are formed once, the tile's position is a scalar base, and the (head, query tile) of the next
         // fetch is counted up instead of divided out.
-        const int frow = static_cast<int>(threadIdx.x) / NCH, fch = static_cast<int>(threadIdx.x) % NCH;
+        const int stid = static_cast<int>(threadIdx.x) - (256 - NSTG);  // negative: this thread stages nothing
+        const int frow = stid / NCH, fch = stid % NCH;
         const uint32_t q_st2 = static_cast<uint32_t>(a.q_st) * 2u, do_st2 = static_cast<uint32_t>(a.do_st) * 2u;
         const uint32_t fch16 = static_cast<uint32_t>(fch) * 16u;
         const int lds_off = frow * S + fch * 8;
-        constexpr int RPI = 256 / NCH;  // tile rows between a thread's consecutive chunks
+        constexpr int RPI = NSTG / NCH;  // tile rows between a thread's consecutive chunks
         // byte offsets of this thread's chunks inside a tile; a row past the end of the sequence is clamped to
         // the last one by clamping the offset (offsets grow with the row: the chunk offset is below the pitch)
         uint32_t offq[CPT], offg[CPT];
@@ -180,9 +184,12 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
         const char* f_qb = reinterpret_cast<const char*>(a.q) + (b * a.q_sb + h0 * a.q_sh + f_q0 * a.q_st) * 2;
         const char* f_gb = reinterpret_cast<const char*>(a.d_o) + (b * a.do_sb + h0 * a.do_sh + f_q0 * a.do_st) * 2;
         // per-row scalars: wavefronts 0 and 1 carry LSE of rows 32w + lane (lanes 0-31), wavefronts 2 and 3 delta
-        const float* const r_arr = w < 2 ? a.lse : a.delta;
-        const float r_mul = w < 2 ? -LOG2E : -1.0f;  // what the LDS holds: -LSE log2(e) and -delta
-        const int rrow = (w & 1) * 32 + (lane & 31);
+        // (with role 1 alone staging: wavefront 2 all of LSE, wavefront 3 all of delta)
+        const bool r_lse = NSTG == 256 ? w < 2 : w == 2;
+        const int r_lanes = NSTG == 256 ? 32 : 64;
+        const float* const r_arr = r_lse ? a.lse : a.delta;
+        const float r_mul = r_lse ? -LOG2E : -1.0f;  // what the LDS holds: -LSE log2(e) and -delta
+        const int rrow = NSTG == 256 ? (w & 1) * 32 + (lane & 31) : lane;
         const char* f_rb = reinterpret_cast<const char*>(r_arr + ((static_cast<int64_t>(b) * a.Hq + h0) * a.T + f_q0));
         // steps from one tile to the next: inside a head, and from the last tile of a head to the first of the next
         const int64_t qd_tile = BMQ * a.q_st * 2, qd_head = a.q_sh * 2 - (nqt - 1) * qd_tile;
@@ -211,7 +218,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
         auto fetch_q = [&](int i) {  // global -> registers
             qr[i] = *reinterpret_cast<const u32x4*>(c_qb + min(offq[i], f_limq));
             // scaled when it is stored: arithmetic on it here would wait for every load just issued
-            if (i == 0 && lane < 32) row_r = *reinterpret_cast<const float*>(c_rb + f_roff);
+            if (i == 0 && lane < r_lanes) row_r = *reinterpret_cast<const float*>(c_rb + f_roff);
         };
         auto fetch_g = [&](int i) {
             gr[i] = *reinterpret_cast<const u32x4*>(c_gb + min(offg[i], f_limg));
@@ -223,7 +230,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
         auto commit_piece = [&](int slot, int i) {  // registers -> LDS ring slot
             *reinterpret_cast<u32x4*>(Qs[slot] + lds_off + i * RPI * S) = qr[i];
             *reinterpret_cast<u32x4*>(dOs[slot] + lds_off + i * RPI * S) = gr[i];
-            if (i == 0 && lane < 32) (w < 2 ? nlse_s[slot] : dl_s[slot])[rrow] = row_r * r_mul;
+            if (i == 0 && lane < r_lanes) (r_lse ? nlse_s[slot] : dl_s[slot])[rrow] = row_r * r_mul;
         };
         auto fetch = [&]() {
             fetch_setup();
@@ -234,9 +241,11 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
 #pragma unroll
             for (int i = 0; i < CPT; ++i) commit_piece(slot, i);
         };
-        fetch();
-        commit(0);
-        fetch();
+        if (NSTG == 256 || role == 1) {
+            fetch();
+            commit(0);
+            fetch();
+        }
         // every load issued so far (the resident K / V rows above all) has landed: otherwise the wait-count
         // bookkeeping carries "kv may be in flight" around the loop and makes each step wait for its own prefetch
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
@@ -404,13 +413,22 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                 };
                 // staging piece p rides in phase p+1, the two roles in different slots: a wavefront whose load finds
                 // the address unit's queue full stalls, matrix instructions and all, so the loads are spread thin
-                auto stage = [&](int piece, int sl) {
-                    constexpr int first = rl * 8;
-                    if (sl == first + 1) commit_piece(cslot, piece);
-                    if (sl == first + 3) fetch_q(piece);
-                    if (sl == first + 5) fetch_g(piece);
+                auto stage = [&](int phase, int sl) {
+                    if (NSTG == 256) {
+                        constexpr int first = rl * 8;
+                        if (sl == first + 1) commit_piece(cslot, phase);
+                        if (sl == first + 3) fetch_q(phase);
+                        if (sl == first + 5) fetch_g(phase);
+                    } else if (rl == 1) {  // two pieces a phase
+                        if (sl == 1) commit_piece(cslot, 2 * phase);
+                        if (sl == 3) fetch_q(2 * phase);
+                        if (sl == 5) fetch_g(2 * phase);
+                        if (sl == 9) commit_piece(cslot, 2 * phase + 1);
+                        if (sl == 11) fetch_q(2 * phase + 1);
+                        if (sl == 13) fetch_g(2 * phase + 1);
+                    }
                 };
-                fetch_setup();
+                if (NSTG == 256 || rl == 1) fetch_setup();
                 // ---- phase 1: GEMM1(block 0)
                 if (rl == 1) nd0 = minus_delta(0);
 #pragma unroll
