@@ -336,17 +336,17 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                 // under the role branch they would make every slot copy whole tuples at the join.
                 float e0[2][16], e1[2][16];   // P or dS of query block 0 / 1
                 bf16x8 op0[2][2], op1[2][2];  // packed P or dS, [sub-block][16-query half]
-                f32x4 rc[4];                  // role 0: -LSE log2(e) of the rows of the block being worked on
+                f32x4 rc[2][4];               // role 0: -LSE log2(e) of the rows of query block 0 / 1
                 f32x16 nd0, nd1;              // role 1: -delta of the rows of query block 0 / 1, laid out like a score tile
-                u32x4 pr[2][2];               // role 1: P handed over, [sub-block][half]
+                u32x4 pr[2][2][2];            // role 1: P handed over, [query block][sub-block][half]
                 bf16x8 fr[NS / 2 + PF];       // fragment window of the running GEMM
                 // elementwise work on elements [lo, hi) of a query block: sub-block e/16, register e%16
-                auto elems = [&](const f32x16(&t)[2], float(&y)[2][16], int lo, int hi) {
+                auto elems = [&](int qb, const f32x16(&t)[2], float(&y)[2][16], int lo, int hi) {
                     if (rl == 0) {
 #pragma unroll
                         for (int e = lo; e < hi; ++e) {
                             const int kb = e >> 4, r = e & 15;
-                            y[kb][r] = __builtin_amdgcn_exp2f(fmaf(t[kb][r], cexp, rc[r >> 2][r & 3]));
+                            y[kb][r] = __builtin_amdgcn_exp2f(fmaf(t[kb][r], cexp, rc[qb][r >> 2][r & 3]));
                         }
                     } else {
 #pragma unroll
@@ -354,7 +354,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                             const int kb = e >> 4, r = e & 15;
                             // dS = P (dP - delta): t holds dP - delta already, P is one half of a packed fp16 pair and
                             // is widened by the instruction itself
-                            const uint32_t pw = pr[kb][r >> 3][(r >> 1) & 3];
+                            const uint32_t pw = pr[qb][kb][r >> 3][(r >> 1) & 3];
                             if (r & 1)
                                 asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(y[kb][r]) : "v"(pw), "v"(t[kb][r]));
                             else
@@ -369,15 +369,17 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                                       c2[0], c2[1], c2[2], c2[3], c3[0], c3[1], c3[2], c3[3]};
                     return v;
                 };
+                // Row constants (role 0) and the P handed over (role 1) of a block are asked for half a phase before the
+                // first slot that uses them: asked for at the phase's start, the lone wavefront sits out the LDS latency.
                 auto side_loads = [&](int qb) {
                     if (rl == 0) {
 #pragma unroll
-                        for (int qd = 0; qd < 4; ++qd) rc[qd] = row_consts(qb, qd);
+                        for (int qd = 0; qd < 4; ++qd) rc[qb][qd] = row_consts(qb, qd);
                     } else {
 #pragma unroll
                         for (int kb = 0; kb < 2; ++kb) {
-                            pr[kb][0] = *LDSP(const u32x4, pa + qb * 8192 + kb * 2048);
-                            pr[kb][1] = *LDSP(const u32x4, pa + qb * 8192 + kb * 2048 + 1024);
+                            pr[qb][kb][0] = *LDSP(const u32x4, pa + qb * 8192 + kb * 2048);
+                            pr[qb][kb][1] = *LDSP(const u32x4, pa + qb * 8192 + kb * 2048 + 1024);
                         }
                     }
                 };
@@ -450,12 +452,12 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     else
                         mma_v(t0[kb], fr[j], kv[kb][j]);
                     if (kb == 0 && j + PF < KK) fr[j + PF] = xfrag(0, j + PF);
+                    if (sl == 8) side_loads(0);
+                    if (sl == 10 && rl == 1) nd1 = minus_delta(1);
                     stage(0, sl);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 // ---- phase 2: GEMM1(block 1) || elementwise(block 0)
-                side_loads(0);
-                if (rl == 1) nd1 = minus_delta(1);
 #pragma unroll
                 for (int j = 0; j < PF; ++j) fr[j] = xfrag(1, j);
                 __builtin_amdgcn_sched_barrier(0);
@@ -471,13 +473,13 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     if (kb == 0 && j + PF < KK) fr[j + PF] = xfrag(1, j + PF);
                     // t0[0] was finished two matrix instructions before the first slot, t0[1] one before: the
                     // first half of the slots works on t0[0] only
-                    elems(t0, e0, sl * 32 / NS, (sl + 1) * 32 / NS);
+                    elems(0, t0, e0, sl * 32 / NS, (sl + 1) * 32 / NS);
+                    if (sl == 8) side_loads(1);
                     stage(1, sl);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 finish_head(0, e0, op0);
                 // ---- phase 3: GEMM2(block 0) || elementwise(block 1)
-                side_loads(1);
 #pragma unroll
                 for (int j = 0; j < PF; ++j) fr[j] = yfrag(0, j);
                 __builtin_amdgcn_sched_barrier(0);
@@ -486,7 +488,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     const int j = sl >> 1, kb = sl & 1;
                     mma_a(acc[kb][j % DB], fr[j], op0[kb][j / DB]);
                     if (kb == 0 && j + PF < 2 * DB) fr[j + PF] = yfrag(0, j + PF);
-                    elems(t1, e1, sl * 32 / NS, (sl + 1) * 32 / NS);
+                    elems(1, t1, e1, sl * 32 / NS, (sl + 1) * 32 / NS);
                     finish_slot(0, e0, op0, sl);
                     stage(2, sl);
                     __builtin_amdgcn_sched_barrier(0);

@@ -123,11 +123,20 @@ __device__ inline bf16x8 lds_read_tr_operand_perm(const uint16_t* tile, int stri
 // buffer resource over what is left of the matrix from row r0 on. Tile loads then take a per-thread byte
 // offset (row_in_tile * st + column) * 2 that never changes, the tile's position sits in the scalar
 // resource, and rows past the end read as zero without a branch (offsets beyond num_records).
+//
+// This runs once per tile in loops where every scalar instruction is issue time, so it is written for few
+// of them: the stride is below 2^22 and the row numbers below 2^24 (checked on the host before these kernels are
+// chosen), hence 32 x 32 -> 64-bit products (two scalar instructions each) and a clamp without a 64-bit compare.
 __device__ inline __amdgpu_buffer_rsrc_t tile_rsrc(const void* base, int64_t elem_off, int64_t st, int r0, int T, int D) {
-    const int64_t left = r0 < T ? (static_cast<int64_t>(T - r0 - 1) * st + D) * 2 : 0;
-    const uint16_t* p = static_cast<const uint16_t*>(base) + elem_off + static_cast<int64_t>(min(r0, T)) * st;
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, static_cast<int>(left < 0x7fffffff ? left : 0x7fffffff),
-                                             0x00020000);
+    const uint32_t st32 = static_cast<uint32_t>(st);
+    const uint32_t first = static_cast<uint32_t>(min(r0, T));
+    const uint32_t rows = static_cast<uint32_t>(T) - first;  // rows left from r0 on
+    const uint32_t some = rows != 0;
+    const uint64_t left = (static_cast<uint64_t>(rows - some) * st32 + (some ? D : 0)) * 2;  // bytes up to the last row's end
+    const uint32_t lo = static_cast<uint32_t>(left), hi = static_cast<uint32_t>(left >> 32);
+    const uint32_t records = hi ? 0x7fffffffu : min(lo, 0x7fffffffu);
+    const uint16_t* p = static_cast<const uint16_t*>(base) + elem_off + static_cast<uint64_t>(first) * st32;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, static_cast<int>(records), 0x00020000);
 }
 __device__ inline u32x4 tile_load16(__amdgpu_buffer_rsrc_t rsrc, int byte_off) {
     return __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, 0, 0);
