@@ -408,16 +408,19 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                 };
                 auto finish_slot = [&](int qb, float(&y)[2][16], bf16x8(&op)[2][2], int sl) {
                     if (sl < 2) op[sl][1] = pack8(y[sl], 1);  // first used in slot 8 + sl
-                    if (rl == 0 && sl >= 2 && sl < 6) {  // hand P over in fp16 (11 significant bits in [0, 1])
-                        const int kb = (sl - 2) >> 1, hf = (sl - 2) & 1;
-                        h16x2 ph[4];
+                };
+                // P goes to role 1 in fp16 (11 significant bits in [0, 1]), a quarter of a block per slot. Both blocks
+                // are handed over in phase 4, the phase with the least other work for role 0 (phase 3 carries the
+                // exponentials of block 1).
+                auto hand_over = [&](int qb, const float(&y)[2][16], int quarter) {
+                    const int kb = quarter >> 1, hf = quarter & 1;
+                    h16x2 ph[4];
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const f32x2 p2 = {y[kb][8 * hf + 2 * i], y[kb][8 * hf + 2 * i + 1]};
-                            ph[i] = __builtin_convertvector(p2, h16x2);
-                        }
-                        *LDSP(u32x4, pa + qb * 8192 + kb * 2048 + hf * 1024) = *reinterpret_cast<u32x4*>(&ph[0]);
+                    for (int i = 0; i < 4; ++i) {
+                        const f32x2 p2 = {y[kb][8 * hf + 2 * i], y[kb][8 * hf + 2 * i + 1]};
+                        ph[i] = __builtin_convertvector(p2, h16x2);
                     }
+                    *LDSP(u32x4, pa + qb * 8192 + kb * 2048 + hf * 1024) = *reinterpret_cast<u32x4*>(&ph[0]);
                 };
                 // staging piece p rides in phase p+1, the two roles in different slots: a wavefront whose load finds
                 // the address unit's queue full stalls, matrix instructions and all, so the loads are spread thin
@@ -504,6 +507,8 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     mma_a(acc[kb][j % DB], fr[j], op1[kb][j / DB]);
                     if (kb == 0 && j + PF < 2 * DB) fr[j + PF] = yfrag(1, j + PF);
                     finish_slot(1, e1, op1, sl);
+                    if (rl == 0 && sl >= 2 && sl < 6) hand_over(1, e1, sl - 2);
+                    if (rl == 0 && sl >= 8 && sl < 12) hand_over(0, e0, sl - 8);
                     stage(3, sl);
                     __builtin_amdgcn_sched_barrier(0);
                 }
