@@ -65,8 +65,8 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
     const int g = lane >> 5, c32 = lane & 31;
     // Lane parts of the two LDS operand addresses (elements): a 16-byte row read at
     // (row c32, column 8g) and a transposing read as lds_read_tr_operand_perm lays it out.
-    const int row_lane = c32 * S + g * 8;
-    const int tr_lane = (4 * g + ((lane & 15) >> 2)) * S + TrMap<D>::src_col(0, (lane >> 4) & 1, lane & 3);
+    const int row_lane = lds_row<D>(c32) * S + g * 8;
+    const int tr_lane = lds_row<D>(4 * g + ((lane & 15) >> 2)) * S + TrMap<D>::src_col(0, (lane >> 4) & 1, lane & 3);
     const int nkb = (a.T + BNK - 1) / BNK, rep = a.Hq / a.Hkv;
     // Full-causal: key block i is seen by T - 128i queries; blocks i and nkb-1-i
     // are taken back to back so that every workgroup carries the same work.
@@ -159,8 +159,8 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
             for (int i = 0; i < CPT; ++i) {
                 const int c = tid + 512 * i;
                 const int row = c / NCH, ch = c % NCH;
-                *reinterpret_cast<u32x4*>(Qs[slot] + row * S + ch * 8) = qr[i];
-                *reinterpret_cast<u32x4*>(dOs[slot] + row * S + ch * 8) = gr[i];
+                *reinterpret_cast<u32x4*>(Qs[slot] + lds_row<D>(row) * S + ch * 8) = qr[i];
+                *reinterpret_cast<u32x4*>(dOs[slot] + lds_row<D>(row) * S + ch * 8) = gr[i];
             }
             if (tid < BMQ) {
                 nlse_s[slot][tid] = -lse_r * LOG2E;
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
         // pointer that already carries the lane part
         auto tr_operand = [&](const uint16_t* p, int row0, int db) {
             p += row0 * S + TrMap<D>::src_col(db, 0, 0);
-            const s16x4 lo = lds_read_tr4(p), hi = lds_read_tr4(p + 8 * S);
+            const s16x4 lo = lds_read_tr4(p), hi = lds_read_tr4(p + TR_HI_ROWS<D> * S);
             typedef short s16x8 __attribute__((ext_vector_type(8)));
             const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             return *reinterpret_cast<const bf16x8*>(&v);

@@ -82,7 +82,7 @@ struct Tile {
         for (int i = 0; i < CPT; ++i) {
             const int c = threadIdx.x + 64 * NW * i;
             const int row = c / NCH, ch = c % NCH;
-            *reinterpret_cast<u32x4*>(lds + row * S + ch * 8) = r[i];
+            *reinterpret_cast<u32x4*>(lds + lds_row<D>(row) * S + ch * 8) = r[i];
         }
     }
 };
@@ -211,9 +211,9 @@ __global__ __launch_bounds__(64 * NW, 2) void mfma_dq(AttnArgs a) {
                 __builtin_amdgcn_s_setprio(1);
 #pragma unroll
                 for (int kk = 0; kk < KK; ++kk) {
-                    const bf16x8 kf = lds_read8(Ks + (nb * 32 + c32) * KT::S + kk * 16 + g * 8);
+                    const bf16x8 kf = lds_read8(Ks + (nb * 32 + lds_row<D>(c32)) * KT::S + kk * 16 + g * 8);
                     s = mfma32(kf, qreg[kk], s);
-                    const bf16x8 vf = lds_read8(Vs + (nb * 32 + c32) * KT::S + kk * 16 + g * 8);
+                    const bf16x8 vf = lds_read8(Vs + (nb * 32 + lds_row<D>(c32)) * KT::S + kk * 16 + g * 8);
                     dp = mfma32(vf, greg[kk], dp);
                 }
                 __builtin_amdgcn_s_setprio(0);

@@ -107,13 +107,30 @@ struct TrMap<64> {  // natural order
     __device__ static constexpr int src_col(int db, int u, int a) { return 32 * db + 16 * u + 4 * a; }
     __device__ static constexpr int col0(int db, int qd, int g) { return 32 * db + 8 * qd + 4 * g; }
 };
+// Where row r of a tile sits in LDS when the tile serves both 16-byte row reads and transposing reads at a pitch
+// 4 banks past a multiple of 64. For head_dim 128 rows keep their order (the column permutation above does the
+// work). For head_dim 64 a row is only 32 banks wide and no column order makes the four rows of a transposing
+// read (r, r+1, r+2, r+3 of a 16-row group, 16 banks each) miss each other at that pitch; instead the rows of each
+// 16-row group are stored in the order (4 (q % 4) + 9 (q / 4)) % 16, which puts rows 4i .. 4i+3 at bank offsets
+// 16 apart and still gives the sixteen rows of a row read sixteen distinct 4-bank windows.
+template <int D>
+__device__ constexpr int lds_row(int r) {
+    return D == 64 ? (r & ~15) | ((4 * (r & 3) + 9 * ((r >> 2) & 3)) & 15) : r;
+}
+// In that order the second four rows of a transposed operand (8 query rows on) always sit TR_HI_ROWS<D> LDS rows
+// past the first four: (4t + 9g + 18) % 16 = (4t + 9g) % 16 + 2 for every t < 4, g < 2.
+template <int D>
+constexpr int TR_HI_ROWS = D == 64 ? 2 : 8;
+static_assert(lds_row<64>(8 + 4 * 1 + 3) == lds_row<64>(4 * 1 + 3) + 2 && lds_row<64>(8 + 3) == lds_row<64>(3) + 2 &&
+              lds_row<64>(8) == lds_row<64>(0) + 2 && lds_row<64>(12) == lds_row<64>(4) + 2, "second half two rows on");
 template <int D>
 __device__ inline bf16x8 lds_read_tr_operand_perm(const uint16_t* tile, int stride, int row0, int db,
-                                                  int lane) {
+                                                  int lane) {  // row0: a multiple of 16
     const int g = lane >> 5, u = (lane >> 4) & 1, j = lane & 15;
-    const uint16_t* p = tile + (row0 + 4 * g + (j >> 2)) * stride + TrMap<D>::src_col(db, u, j & 3);
+    const int col = TrMap<D>::src_col(db, u, j & 3);
+    const uint16_t* p = tile + (row0 + lds_row<D>(4 * g + (j >> 2))) * stride + col;
     s16x4 lo = lds_read_tr4(p);
-    s16x4 hi = lds_read_tr4(p + 8 * stride);
+    s16x4 hi = lds_read_tr4(p + TR_HI_ROWS<D> * stride);
     typedef short s16x8 __attribute__((ext_vector_type(8)));
     s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     return *reinterpret_cast<bf16x8*>(&v);
