@@ -7,7 +7,7 @@
 // as the matrix pipe and neither passes half. Here a wavefront owns 64 keys: two
 // resident operand sets (K or V of two 32-key blocks), two accumulator sets, and
 // every Q / dO fragment read from the LDS feeds TWO matrix instructions. That is
-// 192 persistent registers, so one wavefront per SIMD, four per workgroup:
+// 192 persistent registers at head_dim 128 (96 at 64), so one wavefront per SIMD, four per workgroup:
 //
 //   role 0 (wavefronts 0-1, keys 0-63 / 64-127):  S -> P = exp2(S*c - LSE) -> dV^T += dO^T P
 //   role 1 (wavefronts 2-3, keys 0-63 / 64-127):  dP -> dS = P .* (dP - delta) -> dK^T += Q^T dS
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
         const int frow = stid / NCH, fch = stid % NCH;
         const uint32_t q_st2 = static_cast<uint32_t>(a.q_st) * 2u, do_st2 = static_cast<uint32_t>(a.do_st) * 2u;
         const uint32_t fch16 = static_cast<uint32_t>(fch) * 16u;
-        const int lds_off = frow * S + fch * 8;
+        const int lds_off = lds_row<D>(frow) * S + fch * 8;  // rows frow + RPI i: RPI is 8 (head_dim 128, natural order) or 16 (a whole row group)
         constexpr int RPI = NSTG / NCH;  // tile rows between a thread's consecutive chunks
         // byte offsets of this thread's chunks inside a tile; a row past the end of the sequence is clamped to
         // the last one by clamping the offset (offsets grow with the row: the chunk offset is below the pitch)
@@ -300,12 +300,11 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
         auto lds32 = [](const void* p) { return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(p)); };
         constexpr uint32_t SLOTB = BMQ * S * 2;
         const uint32_t x_slot0 = lds32(rl == 0 ? Qs[0] : dOs[0]), y_slot0 = lds32(rl == 0 ? dOs[0] : Qs[0]);
-        const uint32_t x_lane = static_cast<uint32_t>(c32 * S + g * 8) * 2u;  // GEMM1: row c32, 8 elements from 8g
+        const uint32_t x_lane = static_cast<uint32_t>(lds_row<D>(c32) * S + g * 8) * 2u;  // GEMM1: row c32, 8 elements from 8g
         const int tj = lane & 15, tu = (lane >> 4) & 1;
-        const uint32_t y_lane = static_cast<uint32_t>((4 * g + (tj >> 2)) * S + TrMap<D>::src_col(0, tu, tj & 3)) * 2u;
+        const uint32_t y_lane = static_cast<uint32_t>(lds_row<D>(4 * g + (tj >> 2)) * S + TrMap<D>::src_col(0, tu, tj & 3)) * 2u;
         const uint32_t rc_lane = lds32(rl == 0 ? nlse_s[0] : dl_s[0]) + g * 16u;
         const uint32_t p_lane = lds32(Pbuf) + khalf * 2u * 2048u + lane * 16u;  // [parity][qb][khalf*2+kb][half][lane][8]
-        static_assert(TrMap<D>::src_col(1, 0, 0) - TrMap<D>::src_col(0, 0, 0) == 8, "block db starts 8 columns on");
         int c_qt = 0, slot3 = 0, cslot = (rl + 1) % 3;  // query tile of this step, its ring slot, the slot staged into
         for (int stp = 0; stp < steps; ++stp) {
             {
@@ -324,9 +323,9 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                 const uint32_t pa = p_lane + (stp & 1) * (2u * 4u * 2048u);
                 auto xfrag = [&](int qb, int j) { return *LDSP(const bf16x8, xa + (qb * 32 * S + j * 16) * 2); };
                 auto yfrag = [&](int qb, int j) {
-                    const uint32_t at = ya + ((qb * 32 + (j / DB) * 16) * S + 8 * (j % DB)) * 2;
+                    const uint32_t at = ya + ((qb * 32 + (j / DB) * 16) * S + TrMap<D>::src_col(j % DB, 0, 0) - TrMap<D>::src_col(0, 0, 0)) * 2;
                     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDSP(s16x4, at));
-                    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDSP(s16x4, at + 8 * S * 2));
+                    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDSP(s16x4, at + TR_HI_ROWS<D> * S * 2));
                     typedef short s16x8 __attribute__((ext_vector_type(8)));
                     const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                     return *reinterpret_cast<const bf16x8*>(&v);
@@ -431,12 +430,14 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                         if (sl == first + 3) fetch_q(phase);
                         if (sl == first + 5) fetch_g(phase);
                     } else if (rl == 1) {  // two pieces a phase
-                        if (sl == 1) commit_piece(cslot, 2 * phase);
-                        if (sl == 3) fetch_q(2 * phase);
-                        if (sl == 5) fetch_g(2 * phase);
-                        if (sl == 9) commit_piece(cslot, 2 * phase + 1);
-                        if (sl == 11) fetch_q(2 * phase + 1);
-                        if (sl == 13) fetch_g(2 * phase + 1);
+                        static_assert(CPT == 4 || (CPT == 8 && NS >= 14), "one or two pieces a phase");
+                        constexpr int PPP = CPT / 4;  // pieces per phase
+                        if (sl == 1) commit_piece(cslot, PPP * phase);
+                        if (sl == 3) fetch_q(PPP * phase);
+                        if (sl == 5) fetch_g(PPP * phase);
+                        if (PPP == 2 && sl == 9) commit_piece(cslot, 2 * phase + 1);
+                        if (PPP == 2 && sl == 11) fetch_q(2 * phase + 1);
+                        if (PPP == 2 && sl == 13) fetch_g(2 * phase + 1);
                     }
                 };
                 if (NSTG == 256 || rl == 1) fetch_setup();
@@ -455,8 +456,8 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     else
                         mma_v(t0[kb], fr[j], kv[kb][j]);
                     if (kb == 0 && j + PF < KK) fr[j + PF] = xfrag(0, j + PF);
-                    if (sl == 8) side_loads(0);
-                    if (sl == 10 && rl == 1) nd1 = minus_delta(1);
+                    if (sl == NS / 2) side_loads(0);
+                    if (sl == NS / 2 + 2 && rl == 1) nd1 = minus_delta(1);
                     stage(0, sl);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -477,7 +478,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     // t0[0] was finished two matrix instructions before the first slot, t0[1] one before: the
                     // first half of the slots works on t0[0] only
                     elems(0, t0, e0, sl * 32 / NS, (sl + 1) * 32 / NS);
-                    if (sl == 8) side_loads(1);
+                    if (sl == NS / 2) side_loads(1);
                     stage(1, sl);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -493,6 +494,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     if (kb == 0 && j + PF < 2 * DB) fr[j + PF] = yfrag(0, j + PF);
                     elems(1, t1, e1, sl * 32 / NS, (sl + 1) * 32 / NS);
                     finish_slot(0, e0, op0, sl);
+                    if (rl == 0 && NS < 12 && sl >= 2 && sl < 6) hand_over(0, e0, sl - 2);  // phase 4 is too short to take both
                     stage(2, sl);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -508,7 +510,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     if (kb == 0 && j + PF < 2 * DB) fr[j + PF] = yfrag(1, j + PF);
                     finish_slot(1, e1, op1, sl);
                     if (rl == 0 && sl >= 2 && sl < 6) hand_over(1, e1, sl - 2);
-                    if (rl == 0 && sl >= 8 && sl < 12) hand_over(0, e0, sl - 8);
+                    if (rl == 0 && NS >= 12 && sl >= 8 && sl < 12) hand_over(0, e0, sl - 8);
                     stage(3, sl);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -565,12 +567,14 @@ int launch(const AttnArgs& a, hipStream_t st) {
 bool mfma_dkdv3_takes(const AttnArgs& a) {
     // a thread's byte offset inside a 64-row tile of Q / dO is kept in 32 bits
     const int64_t reach = 2 * BMQ * (a.q_st > a.do_st ? a.q_st : a.do_st);
-    // with a band the 32-key kernel is ahead (0.22 against 0.24 ms at window 256 + 4 sinks, T 4096): the steps are
+    // head_dim 64 (phases of 8 matrix instructions instead of 16) or 128; with a band the 32-key kernel is ahead
+    // (0.22 against 0.24 ms at head_dim 128, window 256 + 4 sinks, T 4096): the steps are
     // few, most of them masked, and the workgroup that owns the sink keys alone walks every query tile
-    return a.dk_dim == 128 && a.window == 0 && reach < (int64_t{1} << 31);
+    return (a.dk_dim == 128 || a.dk_dim == 64) && a.window == 0 && reach < (int64_t{1} << 31);
 }
 
 int launch_mfma_dkdv3(const AttnArgs& a, hipStream_t st) {
+    if (a.dk_dim == 64) return a.grad_f32 ? launch<64, true>(a, st) : launch<64, false>(a, st);
     return a.grad_f32 ? launch<128, true>(a, st) : launch<128, false>(a, st);
 }
 

@@ -284,7 +284,7 @@ int launch(const AttnArgs& a, int stages, hipStream_t st) {
         PK_HIP(hipGetLastError());
     }
     if (stages & PK_BWD_DKDV) {
-        // head_dim 128 without a band: 64 keys per wavefront, one wavefront per SIMD; otherwise 32 keys, two
+        // without a band: 64 keys per wavefront, one wavefront per SIMD; with one: 32 keys, two per SIMD
         if (int rc = mfma_dkdv3_takes(a) ? launch_mfma_dkdv3(a, st) : launch_mfma_dkdv2(a, st)) return rc;
     }
     if (!fused && (stages & PK_BWD_DQ)) {

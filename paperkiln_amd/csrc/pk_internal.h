@@ -118,7 +118,7 @@ bool mfma_supported(const AttnArgs& a);
 int launch_mfma_fwd(const AttnArgs& a, hipStream_t st);
 int launch_mfma_bwd(const AttnArgs& a, int stages, hipStream_t st);
 int launch_mfma_dkdv2(const AttnArgs& a, hipStream_t st);
-// attn_bwd_dkdv3.hip: dK / dV with 64 keys per wavefront and hand-fixed register classes (head_dim 128, no band)
+// attn_bwd_dkdv3.hip: dK / dV with 64 keys per wavefront and hand-fixed register classes (head_dim 64 or 128, no band)
 bool mfma_dkdv3_takes(const AttnArgs& a);
 int launch_mfma_dkdv3(const AttnArgs& a, hipStream_t st);
 

@@ -186,24 +186,25 @@ def test_bf16_sweep_against_oracle(oracle, case):
     assert max(errs[0], errs[2], errs[3], errs[4]) < BF16_TOL and errs[1] < BF16_LSE_TOL
 
 
-# head_dim 128 without a band has a dK/dV kernel of its own (64 keys per wavefront, two roles, a ring of 64-query
+# head_dim 64 / 128 without a band has a dK/dV kernel of its own (64 keys per wavefront, two roles, a ring of 64-query
 # tiles): lengths on every side of its 64-query tile and 128-key block, one to four query heads per KV head
 # (the workgroup walks them in turn), both mask kinds, both gradient element types.
-D128_CASES = [(B, T, rep, Hkv, causal, (T % 2) == 1)
+D128_CASES = [(B, T, rep, Hkv, causal, (T % 2) == 1, dk)
+              for dk in (128, 64)
               for (B, T, rep, Hkv) in [(1, 63, 1, 1), (2, 64, 2, 1), (1, 65, 1, 2), (1, 127, 3, 1), (2, 129, 1, 1), (1, 191, 4, 1),
                                        (1, 257, 2, 2), (1, 449, 1, 1), (1, 700, 3, 1), (1, 1025, 2, 1)]
               for causal in (True, False)]
 
 
-@pytest.mark.parametrize("case", D128_CASES, ids=lambda c: f"B{c[0]}_T{c[1]}_r{c[2]}_kv{c[3]}_c{int(c[4])}_g32{int(c[5])}")
-def test_bf16_head_dim_128_no_band_against_oracle(oracle, case):
-    B, T, rep, Hkv, causal, g32 = case
-    q, k, v, d_o = make(B, T, rep * Hkv, Hkv, 128, 1.0, 9100 + T)
-    scale = float(np.float32(1.0 / np.sqrt(128)))
+@pytest.mark.parametrize("case", D128_CASES, ids=lambda c: f"d{c[6]}_B{c[0]}_T{c[1]}_r{c[2]}_kv{c[3]}_c{int(c[4])}_g32{int(c[5])}")
+def test_bf16_no_band_dkdv_kernel_against_oracle(oracle, case):
+    B, T, rep, Hkv, causal, g32, dk = case
+    q, k, v, d_o = make(B, T, rep * Hkv, Hkv, dk, 1.0, 9100 + T)
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
     want_o, want_lse = oracle.attn_fwd(q, k, v, scale, causal, 0, 0)
     want = (want_o, want_lse) + oracle.attn_bwd(q, k, v, d_o, scale, causal, 0, 0)
     got = run_gpu(q, k, v, d_o, scale, causal, 0, 0, torch.bfloat16, torch.float32 if g32 else torch.bfloat16)
-    errs = report(f"d128 T{T} rep{rep}", got, want)
+    errs = report(f"d{dk} T{T} rep{rep}", got, want)
     assert max(errs[0], errs[2], errs[3], errs[4]) < BF16_TOL and errs[1] < BF16_LSE_TOL
 
 
