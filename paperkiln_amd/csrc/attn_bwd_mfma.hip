@@ -273,8 +273,11 @@ int launch(const AttnArgs& a, int stages, hipStream_t st) {
     const dim3 dq_grid(xcd_grid(paired ? (nbq + 1) / 2 : nbq, a.Hq / a.Hkv, a.Hkv * a.B));
     // delta and dQ asked for together: dQ forms delta itself and runs first, dK/dV reads what it wrote
     const bool fused = (stages & PK_BWD_DELTA) && (stages & PK_BWD_DQ);
+    const bool dq3 = D == 128 && mfma_dq3_takes(a);  // 64 queries per wavefront, one wavefront per SIMD
     if (fused) {
-        if (wide)
+        if (dq3) {
+            if (int rc = launch_mfma_dq3(a, true, st)) return rc;
+        } else if (wide)
             hipLaunchKernelGGL((mfma_dq<D, GF32, true, 8>), dq_grid, dim3(512), 0, st, a);
         else
             hipLaunchKernelGGL((mfma_dq<D, GF32, true, 4>), dq_grid, dim3(256), 0, st, a);
@@ -288,7 +291,9 @@ int launch(const AttnArgs& a, int stages, hipStream_t st) {
         if (int rc = mfma_dkdv3_takes(a) ? launch_mfma_dkdv3(a, st) : launch_mfma_dkdv2(a, st)) return rc;
     }
     if (!fused && (stages & PK_BWD_DQ)) {
-        if (wide)
+        if (dq3) {
+            if (int rc = launch_mfma_dq3(a, false, st)) return rc;
+        } else if (wide)
             hipLaunchKernelGGL((mfma_dq<D, GF32, false, 8>), dq_grid, dim3(512), 0, st, a);
         else
             hipLaunchKernelGGL((mfma_dq<D, GF32, false, 4>), dq_grid, dim3(256), 0, st, a);
