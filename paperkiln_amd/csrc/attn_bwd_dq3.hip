@@ -168,20 +168,18 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
 #pragma unroll
             for (int k = 0; k < NPIECE; ++k) dma_piece(k);
         };
-        dma_tile(0);
-        dma_tile(1);
-
         // Resident operands: Q and dO of the two 32-query blocks (B operands, lane = query), the per-query scalars.
         // A lane's operand chunks are 16 bytes out of every 32 of its own row, so loading them straight from memory
-        // touches a cache line per lane and instruction (18 000 cycles per pass, measured). Instead the wavefront's 64
-        // rows of each tensor go through a region of LDS of its own -- one tile's worth, taken from the two ring slots
-        // that are still empty -- with the same row-filling loads as the tiles, and are read from there as operands.
+        // touches a cache line per lane and instruction (18 000 cycles per pass, measured). The rows therefore go
+        // through LDS: a wavefront fills tile-sized regions of its own in the still empty ring with the same
+        // row-filling loads as the tiles and reads its operands from there. Nobody else reads these rows, so each
+        // round trip goes to memory (about 5000 cycles): Q and dO together in the first, O (for delta) together with
+        // the first two K / V tiles in the second.
         bf16x8 qreg[2][KK], greg[2][KK];
         float nlse[2], dl[2];
         {
-            const uint32_t region = ((w & 1) ? v_lds : k_lds) + static_cast<uint32_t>(2 + (w >> 1)) * SLOTB;
             const int last_row = max(min(BMW - 1, a.T - 1 - qw), 0);  // rows past the end repeat the last one (never stored)
-            auto stage_rows = [&](const void* base, int64_t off, int64_t st_t) {
+            auto stage_rows = [&](uint32_t region, const void* base, int64_t off, int64_t st_t) {
                 const char* src = reinterpret_cast<const char*>(base) + (off + static_cast<int64_t>(min(qw, a.T - 1)) * st_t) * 2;
                 const uint32_t st2 = static_cast<uint32_t>(st_t) * 2u;
                 int row = lane / UPR, ch = lane % UPR;  // unit 64 i + lane of the padded tile
@@ -192,23 +190,31 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
                     row += 64 / UPR, ch += 64 % UPR;
                     if (ch >= UPR) ch -= UPR, ++row;
                 }
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             };
-            auto staged = [&](int qb, int kk) { return *LDSP(const bf16x8, region + x_lane + (qb * 32 * S + kk * 16) * 2); };
             static_assert(UNITS % 64 == 0, "whole load instructions per wavefront");
-            stage_rows(a.q, b * a.q_sb + h * a.q_sh, a.q_st);
+            auto staged = [&](uint32_t region, int qb, int kk) {
+                return *LDSP(const bf16x8, region + x_lane + (qb * 32 * S + kk * 16) * 2);
+            };
+            // first round trip: Q into the K half of ring slot w, dO into its V half
+            const uint32_t region_q = k_lds + static_cast<uint32_t>(w) * SLOTB, region_g = v_lds + static_cast<uint32_t>(w) * SLOTB;
+            stage_rows(region_q, a.q, b * a.q_sb + h * a.q_sh, a.q_st);
+            stage_rows(region_g, a.d_o, b * a.do_sb + h * a.do_sh, a.do_st);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) qreg[qb][kk] = staged(qb, kk);
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // read before the region is filled again
-            stage_rows(a.d_o, b * a.do_sb + h * a.do_sh, a.do_st);
-#pragma unroll
-            for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-                for (int kk = 0; kk < KK; ++kk) greg[qb][kk] = staged(qb, kk);
+                for (int kk = 0; kk < KK; ++kk) {
+                    qreg[qb][kk] = staged(region_q, qb, kk);
+                    greg[qb][kk] = staged(region_g, qb, kk);
+                }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            if (FUSE_DELTA) stage_rows(a.o, b * a.o_sb + h * a.o_sh, a.o_st);
+            __syncthreads();  // every wavefront has read its regions: slots 0 and 1 may take their tiles
+            // second round trip: the first two tiles, and O into a region of slots 2 / 3
+            dma_tile(0);
+            dma_tile(1);
+            const uint32_t region_o = ((w & 1) ? v_lds : k_lds) + static_cast<uint32_t>(2 + (w >> 1)) * SLOTB;
+            if (FUSE_DELTA) stage_rows(region_o, a.o, b * a.o_sb + h * a.o_sh, a.o_st);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb) {
                 const int qi = qw + qb * 32 + c32;
@@ -220,7 +226,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
                     float part = 0.0f;  // this lane's half of the row: d = 16kk + 8g .. +7
 #pragma unroll
                     for (int kk = 0; kk < KK; ++kk) {
-                        const bf16x8 o8 = staged(qb, kk);
+                        const bf16x8 o8 = staged(region_o, qb, kk);
                         const u32x4 ov = *reinterpret_cast<const u32x4*>(&o8);
                         const u32x4 gv = *reinterpret_cast<const u32x4*>(&greg[qb][kk]);
 #pragma unroll
@@ -237,8 +243,8 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         }
-        __syncthreads();  // every wavefront is done with its region: the third tile may land there
-        dma_tile(2);
+        __syncthreads();  // every wavefront has read its O region: the third tile may land there; tiles 0 and 1 are in
+        dma_tile(2);      // waited for at the end of the first iteration
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
@@ -264,9 +270,6 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
                 asm volatile("" : "+a"(acc[qb][db]));
             }
 
-        // every load so far has landed (the tiles in LDS, the rows in registers) before the loop is entered
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
 
         constexpr int PF = 3;              // fragments in flight
         constexpr int N1 = 4 * KK;         // matrix instructions of a G1 phase: (K, V) x kk x two query blocks
@@ -331,14 +334,23 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
         };
         // Elementwise work of one element e (query block e / 16, register e % 16) of the unit whose scores are in
         // (s_, d_); after the 8th and 16th element of a block its packed half is formed.
-        auto elem = [&](const f32x16(&s_)[2], const f32x16(&d_)[2], int e) {
-            const int qb = e >> 4, r = e & 15;
-            const float p = __builtin_amdgcn_exp2f(fmaf(s_[qb][r], cexp, nlse[qb]));
-            y[r & 7] = p * d_[qb][r];  // d_ holds dP - delta
-            if ((r & 7) == 7) {
-                u32x4 u = {pack_bf16(y[0], y[1]), pack_bf16(y[2], y[3]), pack_bf16(y[4], y[5]), pack_bf16(y[6], y[7])};
-                dsp[qb][r >> 3] = *reinterpret_cast<bf16x8*>(&u);
+        // Three instructions per element -- x = S c - LSE, p = exp2(x), dS = p (dP - delta) -- each the input of the next:
+        // issued back to back they wait for one another (a dependent vector instruction issues after 8 clocks, an
+        // independent one after 5), so they are staggered over three slots. Slot sl forms x of element sl, p of
+        // element sl - 1 and dS of element sl - 2; the last two elements finish in the first two slots of the G2 phase
+        // that follows. After the 8th and 16th element of a block its packed half is formed.
+        float xq = 0.0f, pq = 0.0f;
+        auto elem = [&](const f32x16(&s_)[2], const f32x16(&d_)[2], int sl) {
+            if (sl >= 2 && sl < 34) {
+                const int e = sl - 2, qb = e >> 4, r = e & 15;
+                y[r & 7] = pq * d_[qb][r];  // d_ holds dP - delta
+                if ((r & 7) == 7) {
+                    u32x4 u = {pack_bf16(y[0], y[1]), pack_bf16(y[2], y[3]), pack_bf16(y[4], y[5]), pack_bf16(y[6], y[7])};
+                    dsp[qb][r >> 3] = *reinterpret_cast<bf16x8*>(&u);
+                }
             }
+            if (sl >= 1 && sl < 33) pq = __builtin_amdgcn_exp2f(xq);
+            if (sl < 32) xq = fmaf(s_[sl >> 4][sl & 15], cexp, nlse[sl >> 4]);
         };
         // A unit on the diagonal or past the end of the keys: what the mask hides becomes -inf before the exponentials
         // (p = 0, dS = 0). Off the common path; tiles away from the diagonal carry no mask arithmetic at all.
@@ -370,12 +382,18 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
                 if (__builtin_expect(!unit_full(n0), 0)) mask_unit(sc[0], n0);
                 g1(ka, va, 1, sc[1], dp[1], [&](int sl) { elem(sc[0], dp[0], sl); });
                 // ---- G2(t, 0)
-                g2(ya, 0, [&](int sl) { stage(0, sl); });
+                g2(ya, 0, [&](int sl) {
+                    if (sl < 2) elem(sc[0], dp[0], N1 + sl);
+                    stage(0, sl);
+                });
                 // ---- G1(t+1, 0) || E(t, 1)
                 if (__builtin_expect(!unit_full(n0 + 32), 0)) mask_unit(sc[1], n0 + 32);
                 g1(k_lds + slot1 + x_lane, v_lds + slot1 + x_lane, 0, sc[0], dp[0], [&](int sl) { elem(sc[1], dp[1], sl); });
                 // ---- G2(t, 1)
-                g2(ya, 1, [&](int sl) { stage(NPIECE / 2, sl); });
+                g2(ya, 1, [&](int sl) {
+                    if (sl < 2) elem(sc[1], dp[1], N1 + sl);
+                    stage(NPIECE / 2, sl);
+                });
             }
             if (t > hi_w) {  // past this wavefront's diagonal: only the staging (a second skip, not an else: see dK / dV)
 #pragma unroll
