@@ -25,8 +25,11 @@
 // assembly is that the compiler no longer knows these are matrix instructions: the wait
 // states between a matrix instruction writing ordinary registers and the first VALU
 // read of them (passes + 3 = 11 issue slots for the 8-pass 32x32x16) are the program's to
-// provide -- by the software pipeline's own distances on the fast path, by s_nop on the
-// edge path and before the epilogue.
+// provide -- by the software pipeline's own distances inside the loop (a phase of matrix
+// instructions lies between a score tile and its first reader) and by s_nop before the
+// epilogue. Likewise a matrix instruction must not read, as A or B, a register that the
+// vector instruction just before it wrote: it would see the old contents. Both distances
+// are checked on the compiled assembly by tests/test_asm_hazards.py.
 //
 // What a wavefront that has its SIMD to itself pays for (measured with a stream of
 // independent matrix instructions and N other instructions between each pair): the matrix
@@ -71,8 +74,6 @@ __device__ __forceinline__ void mma_v(f32x16& t, bf16x8 a, bf16x8 b) {
 __device__ __forceinline__ void mma_a(f32x16& acc, bf16x8 a, bf16x8 b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
-// wait states for a matrix result in ordinary registers before the VALU may read it
-__device__ __forceinline__ void mma_settle() { asm volatile("s_nop 7\n\ts_nop 7" ::: "memory"); }
 
 template <bool F32>
 __device__ inline void store4g(void* base, int64_t idx, float x0, float x1, float x2, float x3) {

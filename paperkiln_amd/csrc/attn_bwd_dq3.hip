@@ -14,6 +14,7 @@
 //   G1   S^T = K Q^T and dP^T = V dO^T   32 matrix instructions (16 fragments, two blocks each)
 //   E    dS = exp2(S c - LSE) (dP - delta), packed to bf16         (lane = query: all in-lane)
 //   G2   dQ^T += K^T dS^T                16 matrix instructions (8 transposed fragments)
+// at head_dim 128, half as many matrix instructions (and the same E) at head_dim 64.
 // With nobody else on its SIMD the wavefront overlaps these by hand: E of a unit rides in the
 // shadows of G1 of the next one, one element per matrix instruction,
 //   per tile t:   G1(t, 1) || E(t, 0)  .  G2(t, 0)  .  G1(t+1, 0) || E(t, 1)  .  G2(t, 1)
@@ -24,7 +25,9 @@
 //
 // All matrix instructions are inline assembly with fixed register classes, as in the dK / dV
 // kernel; the wait states between a matrix instruction and the first VALU read of its result
-// are provided by the pipeline's own distances (a whole phase) and by s_nop before the epilogue.
+// are provided by the pipeline's own distances (a whole phase) and by s_nop before the epilogue,
+// and a packed dS operand is formed at least two issue slots before the matrix instruction that
+// reads it (tests/test_asm_hazards.py checks both on the compiled assembly).
 #include <type_traits>
 
 #include "mfma_common.h"
@@ -54,6 +57,12 @@ __device__ __forceinline__ void mma_sc(f32x16& t, bf16x8 a, const bf16x8& b, con
 // acc += a . b                    dQ^T accumulator in accumulation registers, B operand (packed dS) in ordinary ones
 __device__ __forceinline__ void mma_q(f32x16& acc, bf16x8 a, bf16x8 b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+// The same for the first use of a packed dS operand: a matrix instruction that reads a register written by the vector
+// instruction just before it gets the old contents (the compiler spaces the two apart only for matrix instructions it
+// emits itself), so two idle states go first.
+__device__ __forceinline__ void mma_q_fresh(f32x16& acc, bf16x8 a, bf16x8 b) {
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
 
 template <bool F32>
@@ -108,10 +117,15 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
     const uint32_t k_lds = lds32(Kt[0]), v_lds = lds32(Vt[0]);
     // lane parts of the LDS read addresses: a 16-byte row read at (row c32, 8 elements from 8g), and the
     // transposing read of K^T as lds_read_tr_operand_perm lays it out
-    const uint32_t x_lane = static_cast<uint32_t>(c32 * S + g * 8) * 2u;
+    const uint32_t x_lane = static_cast<uint32_t>(lds_row<D>(c32) * S + g * 8) * 2u;
     const int tj = lane & 15, tu = (lane >> 4) & 1;
     const uint32_t y_lane = static_cast<uint32_t>(lds_row<D>(4 * g + (tj >> 2)) * S + TrMap<D>::src_col(0, tu, tj & 3)) * 2u;
-    static_assert(D == 128, "row order and column blocks below are those of head_dim 128");
+    // Which memory row a load puts into LDS row R of a tile: the inverse of lds_row (R = 4a + 9b mod 16 inside a group
+    // of 16 with b = R % 4 at head_dim 64; the identity at 128).
+    auto mem_row = [](int R) {
+        const int r = R & 15, bq = r & 3, aq = ((r - 9 * bq) & 15) >> 2;
+        return D == 64 ? (R & ~15) | (4 * bq + aq) : R;
+    };
 
     // Tile staging: which 16 bytes of a tile this lane fetches with its i-th load (the LDS side is lane after lane).
     const uint32_t k_st2 = static_cast<uint32_t>(a.k_st) * 2u, v_st2 = static_cast<uint32_t>(a.v_st) * 2u;
@@ -119,7 +133,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
 #pragma unroll
     for (int i = 0; i <= NI; ++i) {
         const int u = i < NI ? 256 * i + static_cast<int>(threadIdx.x) : 256 * NI + 16 * w + (lane & 15);
-        const uint32_t row = u / UPR, ch = min(u % UPR, NCH - 1);  // the padding unit repeats the last chunk
+        const uint32_t row = mem_row(u / UPR), ch = min(u % UPR, NCH - 1);  // the padding unit repeats the last chunk
         offk[i] = row * k_st2 + ch * 16u;
         offv[i] = row * v_st2 + ch * 16u;
     }
@@ -186,7 +200,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
 #pragma unroll
                 for (int i = 0; i < UNITS / 64; ++i) {
                     dma16(region + static_cast<uint32_t>(i) * 1024u,
-                          static_cast<uint32_t>(min(row, last_row)) * st2 + static_cast<uint32_t>(min(ch, NCH - 1)) * 16u, src);
+                          static_cast<uint32_t>(min(mem_row(row), last_row)) * st2 + static_cast<uint32_t>(min(ch, NCH - 1)) * 16u, src);
                     row += 64 / UPR, ch += 64 % UPR;
                     if (ch >= UPR) ch -= UPR, ++row;
                 }
@@ -284,7 +298,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
         };
         // G2 fragment fi of a unit: K^T, 16-key half kc = fi / DB, column block db = fi % DB
         auto g2frag = [&](uint32_t ya, int nb, int fi) {
-            const uint32_t at = ya + ((nb * 32 + (fi / DB) * 16) * S + 8 * (fi % DB)) * 2;
+            const uint32_t at = ya + ((nb * 32 + (fi / DB) * 16) * S + TrMap<D>::src_col(fi % DB, 0, 0) - TrMap<D>::src_col(0, 0, 0)) * 2;
             const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDSP(s16x4, at));
             const s16x4 hi2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDSP(s16x4, at + TR_HI_ROWS<D> * S * 2));
             typedef short s16x8 __attribute__((ext_vector_type(8)));
@@ -326,7 +340,10 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
 #pragma unroll
             for (int sl = 0; sl < N2; ++sl) {
                 const int fi = sl >> 1, qb = sl & 1;
-                mma_q(acc[qb][fi % DB], f[fi], dsp[qb][fi / DB]);
+                if (fi % DB == 0)
+                    mma_q_fresh(acc[qb][0], f[fi], dsp[qb][fi / DB]);
+                else
+                    mma_q(acc[qb][fi % DB], f[fi], dsp[qb][fi / DB]);
                 if (qb == 0 && fi + PF < N2 / 2) f[fi + PF] = g2frag(ya, nb, fi + PF);
                 shadow(sl);
                 __builtin_amdgcn_sched_barrier(0);
@@ -336,21 +353,35 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
         // (s_, d_); after the 8th and 16th element of a block its packed half is formed.
         // Three instructions per element -- x = S c - LSE, p = exp2(x), dS = p (dP - delta) -- each the input of the next:
         // issued back to back they wait for one another (a dependent vector instruction issues after 8 clocks, an
-        // independent one after 5), so they are staggered over three slots. Slot sl forms x of element sl, p of
-        // element sl - 1 and dS of element sl - 2; the last two elements finish in the first two slots of the G2 phase
+        // independent one after 5), so they are staggered over three slots. Slot sl forms x of element sl (of the pair 2 sl, 2 sl + 1
+        // at head_dim 64, where a phase has half the slots), p of element sl - 1 and dS of element sl - 2; the last two elements finish in the first two slots of the G2 phase
         // that follows. After the 8th and 16th element of a block its packed half is formed.
-        float xq = 0.0f, pq = 0.0f;
+        constexpr int EPS = 32 / N1;  // elements per slot: 1 at head_dim 128, 2 at 64
+        float xq[EPS] = {}, pq[EPS] = {};
         auto elem = [&](const f32x16(&s_)[2], const f32x16(&d_)[2], int sl) {
-            if (sl >= 2 && sl < 34) {
-                const int e = sl - 2, qb = e >> 4, r = e & 15;
-                y[r & 7] = pq * d_[qb][r];  // d_ holds dP - delta
-                if ((r & 7) == 7) {
-                    u32x4 u = {pack_bf16(y[0], y[1]), pack_bf16(y[2], y[3]), pack_bf16(y[4], y[5]), pack_bf16(y[6], y[7])};
-                    dsp[qb][r >> 3] = *reinterpret_cast<bf16x8*>(&u);
+#pragma unroll
+            for (int i = 0; i < EPS; ++i) {
+                if (sl >= 2 && sl < N1 + 2) {
+                    const int e = (sl - 2) * EPS + i, qb = e >> 4, r = e & 15;
+                    y[r & 7] = pq[i] * d_[qb][r];  // d_ holds dP - delta
+                    if ((r & 7) == 7) {
+                        u32x4 u = {pack_bf16(y[0], y[1]), pack_bf16(y[2], y[3]), pack_bf16(y[4], y[5]), pack_bf16(y[6], y[7])};
+                        dsp[qb][r >> 3] = *reinterpret_cast<bf16x8*>(&u);
+                        // formed here, in this slot: without the pin the compiler may sink the whole chain of the half
+                        // to just before the matrix instruction that reads it, which then reads a register written one
+                        // instruction earlier -- inside an asm statement the compiler keeps no distance for that
+                        asm volatile("" : "+v"(dsp[qb][r >> 3]));
+                    }
                 }
             }
-            if (sl >= 1 && sl < 33) pq = __builtin_amdgcn_exp2f(xq);
-            if (sl < 32) xq = fmaf(s_[sl >> 4][sl & 15], cexp, nlse[sl >> 4]);
+#pragma unroll
+            for (int i = 0; i < EPS; ++i)
+                if (sl >= 1 && sl < N1 + 1) pq[i] = __builtin_amdgcn_exp2f(xq[i]);
+#pragma unroll
+            for (int i = 0; i < EPS; ++i) {
+                const int e = sl * EPS + i;
+                if (sl < N1) xq[i] = fmaf(s_[e >> 4][e & 15], cexp, nlse[e >> 4]);
+            }
         };
         // A unit on the diagonal or past the end of the keys: what the mask hides becomes -inf before the exponentials
         // (p = 0, dS = 0). Off the common path; tiles away from the diagonal carry no mask arithmetic at all.
@@ -402,8 +433,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
             // Tile t+2 (asked for one iteration ago) has landed; the NPIECE loads of tile t+3 issued in this iteration
             // may stay in flight (loads complete in order). Every wavefront issues exactly NPIECE load instructions
             // per iteration, on either path.
-            static_assert(NPIECE == 10, "the wait below counts the loads of one tile");
-            asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NPIECE) : "memory");
             __syncthreads();
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may land in the ring after the pass
@@ -449,10 +479,11 @@ int launch(const AttnArgs& a, bool fuse_delta, hipStream_t st) {
 bool mfma_dq3_takes(const AttnArgs& a) {
     // a lane's byte offset inside a 64-row tile of K / V is kept in 32 bits
     const int64_t reach = 2 * BN * (a.k_st > a.v_st ? a.k_st : a.v_st);
-    return a.dk_dim == 128 && a.window == 0 && reach < (int64_t{1} << 31);
+    return (a.dk_dim == 128 || a.dk_dim == 64) && a.window == 0 && reach < (int64_t{1} << 31);
 }
 
 int launch_mfma_dq3(const AttnArgs& a, bool fuse_delta, hipStream_t st) {
+    if (a.dk_dim == 64) return a.grad_f32 ? launch<64, true>(a, fuse_delta, st) : launch<64, false>(a, fuse_delta, st);
     return a.grad_f32 ? launch<128, true>(a, fuse_delta, st) : launch<128, false>(a, fuse_delta, st);
 }
 

@@ -273,7 +273,7 @@ int launch(const AttnArgs& a, int stages, hipStream_t st) {
     const dim3 dq_grid(xcd_grid(paired ? (nbq + 1) / 2 : nbq, a.Hq / a.Hkv, a.Hkv * a.B));
     // delta and dQ asked for together: dQ forms delta itself and runs first, dK/dV reads what it wrote
     const bool fused = (stages & PK_BWD_DELTA) && (stages & PK_BWD_DQ);
-    const bool dq3 = D == 128 && mfma_dq3_takes(a);  // 64 queries per wavefront, one wavefront per SIMD
+    const bool dq3 = mfma_dq3_takes(a);  // 64 queries per wavefront, one wavefront per SIMD
     if (fused) {
         if (dq3) {
             if (int rc = launch_mfma_dq3(a, true, st)) return rc;

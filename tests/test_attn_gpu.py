@@ -18,7 +18,9 @@ BF16_TOL, BF16_LSE_TOL = 2e-2, 1e-3
 
 
 def maxabs(a, b):
-    return float(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64)).max())
+    # NaN anywhere counts as an infinite error: Python's max() over a list of errors drops a NaN that is not first
+    e = float(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64)).max())
+    return e if np.isfinite(e) else float("inf")
 
 
 def dev(x, dtype):

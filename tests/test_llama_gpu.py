@@ -24,7 +24,8 @@ def load(name):
 
 
 def maxdiff(a, b):
-    return max(float(np.abs(a[k].astype(np.float64) - b[k]).max()) for k in a)
+    errs = [float(np.abs(a[k].astype(np.float64) - b[k]).max()) for k in a]
+    return max(errs) if np.all(np.isfinite(errs)) else float("inf")  # max() drops a NaN that is not first
 
 
 @pytest.mark.parametrize("name", ["llama_T16_single", "llama_T16x2_stacked"])
@@ -141,7 +142,8 @@ def test_errors():
 
 def reldiff(a, b):
     """Largest |a - b| over all parameters, relative to the largest |b| of the same parameter."""
-    return max(float(np.abs(a[k].astype(np.float64) - b[k]).max() / max(float(np.abs(b[k]).max()), 1e-30)) for k in a)
+    errs = [float(np.abs(a[k].astype(np.float64) - b[k]).max() / max(float(np.abs(b[k]).max()), 1e-30)) for k in a]
+    return max(errs) if np.all(np.isfinite(errs)) else float("inf")
 
 
 # (dtype, vocab, tokens, seq_len, rows per head chunk or None = the library's default of 2048)
