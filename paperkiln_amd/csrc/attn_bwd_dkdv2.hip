@@ -330,11 +330,16 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
                                          : b * a.dk_sb + hk * a.dk_sh + kj * a.dk_st;
             const float sc = role == 0 ? 1.0f : a.scale;
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
+            for (int db = 0; db < DB; ++db) {
+                if (!GF32) {
+                    store_acc_bf16<D>(static_cast<uint16_t*>(dst) + ob, db, g, acc[db], sc);
+                    continue;
+                }
 #pragma unroll
                 for (int qd = 0; qd < 4; ++qd)
                     store4g<GF32>(dst, ob + TrMap<D>::col0(db, qd, g), acc[db][qd * 4] * sc, acc[db][qd * 4 + 1] * sc,
                                   acc[db][qd * 4 + 2] * sc, acc[db][qd * 4 + 3] * sc);
+            }
         }
         __syncthreads();  // the next pass refills the ring
     }

@@ -538,18 +538,25 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                                        : b * a.dk_sb + hk * a.dk_sh + kj * a.dk_st;
             const float sc = rl == 0 ? 1.0f : a.scale;
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
+            for (int db = 0; db < DB; ++db) {
+                if (!GF32) {
+                    store_acc_bf16<D>(static_cast<uint16_t*>(dst) + ob, db, g, acc[kb][db], sc);
+                    continue;
+                }
 #pragma unroll
                 for (int qd = 0; qd < 4; ++qd)
                     store4g<GF32>(dst, ob + TrMap<D>::col0(db, qd, g), acc[kb][db][qd * 4] * sc, acc[kb][db][qd * 4 + 1] * sc,
                                   acc[kb][db][qd * 4 + 2] * sc, acc[kb][db][qd * 4 + 3] * sc);
+            }
         }
         };  // run_role
         if (role == 0)
             run_role(std::integral_constant<int, 0>{});
         else
             run_role(std::integral_constant<int, 1>{});
-        __syncthreads();  // the next pass refills the ring
+        // No barrier here: after the last barrier of the step loop nobody reads the rings any more, the stores above
+        // touch no LDS, and a barrier would make every wavefront wait for its stores to be acknowledged before the
+        // next pass may ask for its rows.
     }
 }
 

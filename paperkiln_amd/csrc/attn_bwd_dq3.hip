@@ -307,10 +307,13 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
         };
         // one G1 phase: unit (tile slot addresses ka / va, half nb) into score set `into`; `shadow(sl)` is the
         // other work of slot sl
-        auto g1 = [&](uint32_t ka, uint32_t va, int nb, f32x16(&s_)[2], f32x16(&d_)[2], auto shadow) {
+        // `have`: the first PF fragments were asked for in the last slots of the phase before (nx); `next(j)` asks for
+        // fragment j of the phase that follows, in this phase's last slots, so that no phase opens with an LDS round trip
+        bf16x8 nx[PF];
+        auto g1 = [&](uint32_t ka, uint32_t va, int nb, f32x16(&s_)[2], f32x16(&d_)[2], auto shadow, auto have, auto next) {
             bf16x8 f[N1 / 2];
 #pragma unroll
-            for (int j = 0; j < PF; ++j) f[j] = g1frag(ka, va, nb, j);
+            for (int j = 0; j < PF; ++j) f[j] = decltype(have)::value ? nx[j] : g1frag(ka, va, nb, j);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int sl = 0; sl < N1; ++sl) {
@@ -326,16 +329,21 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
                     else
                         mma_s(s_[qb], f[fi], qreg[qb][kk]);
                 }
-                if (qb == 0 && fi + PF < N1 / 2) f[fi + PF] = g1frag(ka, va, nb, fi + PF);
+                if (qb == 0) {
+                    if (fi + PF < N1 / 2)
+                        f[fi + PF] = g1frag(ka, va, nb, fi + PF);
+                    else
+                        nx[fi + PF - N1 / 2] = next(fi + PF - N1 / 2);
+                }
                 shadow(sl);
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
         // one G2 phase: dQ^T += K^T dS^T of the unit in hand
-        auto g2 = [&](uint32_t ya, int nb, auto shadow) {
+        auto g2 = [&](uint32_t ya, int nb, auto shadow, auto next) {
             bf16x8 f[N2 / 2];
 #pragma unroll
-            for (int j = 0; j < PF; ++j) f[j] = g2frag(ya, nb, j);
+            for (int j = 0; j < PF; ++j) f[j] = nx[j];
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int sl = 0; sl < N2; ++sl) {
@@ -344,7 +352,12 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
                     mma_q_fresh(acc[qb][0], f[fi], dsp[qb][fi / DB]);
                 else
                     mma_q(acc[qb][fi % DB], f[fi], dsp[qb][fi / DB]);
-                if (qb == 0 && fi + PF < N2 / 2) f[fi + PF] = g2frag(ya, nb, fi + PF);
+                if (qb == 0) {
+                    if (fi + PF < N2 / 2)
+                        f[fi + PF] = g2frag(ya, nb, fi + PF);
+                    else
+                        nx[fi + PF - N2 / 2] = next(fi + PF - N2 / 2);
+                }
                 shadow(sl);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -396,7 +409,9 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
             return n0u + 31 < a.T && (!a.causal || n0u + 31 <= qw);
         };
 
-        if (hi_w >= 0) g1(k_lds + x_lane, v_lds + x_lane, 0, sc[0], dp[0], [](int) {});
+        if (hi_w >= 0)
+            g1(k_lds + x_lane, v_lds + x_lane, 0, sc[0], dp[0], [](int) {}, std::false_type{},
+               [&](int j) { return g1frag(k_lds + x_lane, v_lds + x_lane, 1, j); });
         // the first elementwise slots follow at once here (in the loop a whole G2 phase lies between): let the last
         // matrix instructions of this prologue write their results first
         asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7\n\ts_nop 7" ::: "memory");
@@ -411,20 +426,28 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
                 const uint32_t ka = k_lds + slot + x_lane, va = v_lds + slot + x_lane, ya = k_lds + slot + y_lane;
                 // ---- G1(t, 1) || E(t, 0)
                 if (__builtin_expect(!unit_full(n0), 0)) mask_unit(sc[0], n0);
-                g1(ka, va, 1, sc[1], dp[1], [&](int sl) { elem(sc[0], dp[0], sl); });
+                const uint32_t ka1 = k_lds + slot1 + x_lane, va1 = v_lds + slot1 + x_lane;
+                g1(ka, va, 1, sc[1], dp[1], [&](int sl) { elem(sc[0], dp[0], sl); }, std::true_type{},
+                   [&](int j) { return g2frag(ya, 0, j); });
                 // ---- G2(t, 0)
-                g2(ya, 0, [&](int sl) {
-                    if (sl < 2) elem(sc[0], dp[0], N1 + sl);
-                    stage(0, sl);
-                });
+                g2(ya, 0,
+                   [&](int sl) {
+                       if (sl < 2) elem(sc[0], dp[0], N1 + sl);
+                       stage(0, sl);
+                   },
+                   [&](int j) { return g1frag(ka1, va1, 0, j); });
                 // ---- G1(t+1, 0) || E(t, 1)
                 if (__builtin_expect(!unit_full(n0 + 32), 0)) mask_unit(sc[1], n0 + 32);
-                g1(k_lds + slot1 + x_lane, v_lds + slot1 + x_lane, 0, sc[0], dp[0], [&](int sl) { elem(sc[1], dp[1], sl); });
-                // ---- G2(t, 1)
-                g2(ya, 1, [&](int sl) {
-                    if (sl < 2) elem(sc[1], dp[1], N1 + sl);
-                    stage(NPIECE / 2, sl);
-                });
+                g1(ka1, va1, 0, sc[0], dp[0], [&](int sl) { elem(sc[1], dp[1], sl); }, std::true_type{},
+                   [&](int j) { return g2frag(ya, 1, j); });
+                // ---- G2(t, 1); its last slots ask for the first fragments of the next iteration's G1(t+1, 1): that tile
+                // has been readable since the barrier before this iteration
+                g2(ya, 1,
+                   [&](int sl) {
+                       if (sl < 2) elem(sc[1], dp[1], N1 + sl);
+                       stage(NPIECE / 2, sl);
+                   },
+                   [&](int j) { return g1frag(ka1, va1, 1, j); });
             }
             if (t > hi_w) {  // past this wavefront's diagonal: only the staging (a second skip, not an else: see dK / dV)
 #pragma unroll
@@ -450,14 +473,22 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
             if (qi >= a.T) continue;
             const int64_t ob = b * a.dq_sb + h * a.dq_sh + qi * a.dq_st;
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
+            for (int db = 0; db < DB; ++db) {
+                if (!GF32) {
+                    store_acc_bf16<D>(static_cast<uint16_t*>(a.dq) + ob, db, g, acc[qb][db], a.scale);
+                    continue;
+                }
 #pragma unroll
                 for (int qd = 0; qd < 4; ++qd)
                     store4q<GF32>(a.dq, ob + TrMap<D>::col0(db, qd, g), acc[qb][db][qd * 4] * a.scale,
                                   acc[qb][db][qd * 4 + 1] * a.scale, acc[qb][db][qd * 4 + 2] * a.scale,
                                   acc[qb][db][qd * 4 + 3] * a.scale);
+            }
         }
-        __syncthreads();  // the next pass refills the ring
+        // No barrier here: every wavefront passed the barrier of the last iteration after its last read of the ring,
+        // the stores above touch no LDS, and the next pass meets its own barriers before anybody reads what another
+        // wavefront wrote. A barrier would also make each wavefront wait for its dQ stores to be acknowledged before
+        // the next pass may ask for its rows.
     }
 }
 

@@ -249,12 +249,17 @@ __global__ __launch_bounds__(64 * NW, 2) void mfma_dq(AttnArgs a) {
     if (qi < a.T) {
         const int64_t ob = b * a.dq_sb + h * a.dq_sh + qi * a.dq_st;
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
+        for (int db = 0; db < DB; ++db) {
+            if (!GF32) {
+                store_acc_bf16<D>(static_cast<uint16_t*>(a.dq) + ob, db, g, dq_acc[db], a.scale);
+                continue;
+            }
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd)
                 store4<GF32>(a.dq, ob + TrMap<D>::col0(db, qd, g), dq_acc[db][qd * 4] * a.scale,
                              dq_acc[db][qd * 4 + 1] * a.scale, dq_acc[db][qd * 4 + 2] * a.scale,
                              dq_acc[db][qd * 4 + 3] * a.scale);
+        }
     }
     __syncthreads();  // the next pass refills the tile buffers
   }

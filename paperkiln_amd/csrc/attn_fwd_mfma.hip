@@ -251,13 +251,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void mfma_fwd(AttnArgs a) {
         const float inv = 1.0f / lt;
         uint16_t* orow = static_cast<uint16_t*>(a.o) + b * a.o_sb + h * a.o_sh + qi * a.o_st;
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int qd = 0; qd < 4; ++qd) {
-                u32x2 pk2 = {pack_bf16(acc_o[qb][db][qd * 4 + 0] * inv, acc_o[qb][db][qd * 4 + 1] * inv),
-                             pack_bf16(acc_o[qb][db][qd * 4 + 2] * inv, acc_o[qb][db][qd * 4 + 3] * inv)};
-                *reinterpret_cast<u32x2*>(orow + db * 32 + qd * 8 + g * 4) = pk2;
-            }
+        for (int db = 0; db < DB; ++db) store_acc_bf16_natural(orow, db, g, acc_o[qb][db], inv);
         if (g == 0)
             a.lse[(static_cast<int64_t>(b) * a.Hq + h) * a.T + qi] = m[qb] * a.scale + logf(lt);
     }

@@ -107,6 +107,43 @@ struct TrMap<64> {  // natural order
     __device__ static constexpr int src_col(int db, int u, int a) { return 32 * db + 16 * u + 4 * a; }
     __device__ static constexpr int col0(int db, int qd, int g) { return 32 * db + 8 * qd + 4 * g; }
 };
+// One 32 x 32 accumulator block (lane = row c32 of the output, elements 4qd .. 4qd+3 = four consecutive columns from
+// TrMap<D>::col0(db, qd, g)) scaled and written as bf16 in 16-byte pieces instead of 8-byte ones: a lane's store is one
+// request to the memory pipe whatever its size, and an epilogue of 8-byte pieces spends its time queueing requests.
+// At head_dim 128 the pieces qd and qd + 2 of a lane are neighbours (4 columns apart); in the natural order of
+// head_dim 64 a lane's neighbour piece sits in lane ^ 32, so pieces qd and qd + 1 trade halves first
+// (v_permlane32_swap) and lane half g writes the eight columns from 32 db + 8 (2 qp + g). Both lanes of a pair must
+// be active (they hold the same row, so a bound on the row keeps or drops them together).
+// natural column order: elements 4qd .. 4qd+3 of half g are columns 32 db + 8 qd + 4 g ..
+__device__ inline void store_acc_bf16_natural(uint16_t* row, int db, int g, const f32x16& acc, float sc) {
+#pragma unroll
+    for (int qp = 0; qp < 2; ++qp) {
+        const int lo = qp * 8, hi = qp * 8 + 4;
+        const uint32_t a0 = pack_bf16(acc[lo] * sc, acc[lo + 1] * sc), a1 = pack_bf16(acc[lo + 2] * sc, acc[lo + 3] * sc);
+        const uint32_t b0 = pack_bf16(acc[hi] * sc, acc[hi + 1] * sc), b1 = pack_bf16(acc[hi + 2] * sc, acc[hi + 3] * sc);
+        // (x, y) = swap(a, b): lanes 32..63 of a trade places with lanes 0..31 of b, so half 0 ends up with piece
+        // 2qp of both halves and half 1 with piece 2qp + 1 of both
+        const auto r0 = __builtin_amdgcn_permlane32_swap(a0, b0, false, false);
+        const auto r1 = __builtin_amdgcn_permlane32_swap(a1, b1, false, false);
+        u32x4 v = {r0[0], r1[0], r0[1], r1[1]};
+        *reinterpret_cast<u32x4*>(row + 32 * db + 8 * (2 * qp + g)) = v;
+    }
+}
+// column order of TrMap<D>
+static_assert(TrMap<64>::col0(1, 2, 1) == 32 + 16 + 4 && TrMap<128>::col0(1, 2, 0) == TrMap<128>::col0(1, 0, 0) + 4,
+              "head_dim 64 is in natural order; at 128 piece qd + 2 follows piece qd");
+template <int D>
+__device__ inline void store_acc_bf16(uint16_t* row, int db, int g, const f32x16& acc, float sc) {
+    if (D != 128) return store_acc_bf16_natural(row, db, g, acc, sc);
+#pragma unroll
+    for (int qp = 0; qp < 2; ++qp) {
+        const int lo = qp * 4, hi = (qp + 2) * 4;
+        u32x4 v = {pack_bf16(acc[lo] * sc, acc[lo + 1] * sc), pack_bf16(acc[lo + 2] * sc, acc[lo + 3] * sc),
+                   pack_bf16(acc[hi] * sc, acc[hi + 1] * sc), pack_bf16(acc[hi + 2] * sc, acc[hi + 3] * sc)};
+        *reinterpret_cast<u32x4*>(row + TrMap<128>::col0(db, qp, g)) = v;
+    }
+}
+
 // Where row r of a tile sits in LDS when the tile serves both 16-byte row reads and transposing reads at a pitch
 // 4 banks past a multiple of 64. For head_dim 128 rows keep their order (the column permutation above does the
 // work). For head_dim 64 a row is only 32 banks wide and no column order makes the four rows of a transposing
