@@ -191,7 +191,17 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
         // the first two K / V tiles in the second.
         bf16x8 qreg[2][KK], greg[2][KK];
         float nlse[2], dl[2];
+        f32x16 acc[2][DB];  // dQ^T of the two query blocks
         {
+            // asked for first, used after the second round trip
+            float lse_raw[2];
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+                const int qi = qw + qb * 32 + c32;
+                const int64_t lrow = (static_cast<int64_t>(b) * a.Hq + h) * a.T + qi;
+                lse_raw[qb] = qi < a.T ? a.lse[lrow] : 0.0f;
+                if (!FUSE_DELTA) dl[qb] = qi < a.T ? a.delta[lrow] : 0.0f;
+            }
             const int last_row = max(min(BMW - 1, a.T - 1 - qw), 0);  // rows past the end repeat the last one (never stored)
             auto stage_rows = [&](uint32_t region, const void* base, int64_t off, int64_t st_t) {
                 const char* src = reinterpret_cast<const char*>(base) + (off + static_cast<int64_t>(min(qw, a.T - 1)) * st_t) * 2;
@@ -213,6 +223,15 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
             const uint32_t region_q = k_lds + static_cast<uint32_t>(w) * SLOTB, region_g = v_lds + static_cast<uint32_t>(w) * SLOTB;
             stage_rows(region_q, a.q, b * a.q_sb + h * a.q_sh, a.q_st);
             stage_rows(region_g, a.d_o, b * a.do_sb + h * a.do_sh, a.do_st);
+            // the accumulators are cleared while the rows are on their way
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[qb][db][r] = 0.0f;
+                    asm volatile("" : "+a"(acc[qb][db]));
+                }
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb)
@@ -224,20 +243,24 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             __syncthreads();  // every wavefront has read its regions: slots 0 and 1 may take their tiles
             // second round trip: the first two tiles, and O into a region of slots 2 / 3
-            dma_tile(0);
-            dma_tile(1);
             const uint32_t region_o = ((w & 1) ? v_lds : k_lds) + static_cast<uint32_t>(2 + (w >> 1)) * SLOTB;
             if (FUSE_DELTA) stage_rows(region_o, a.o, b * a.o_sb + h * a.o_sh, a.o_st);
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            dma_tile(0);
+            dma_tile(1);
+            // loads complete in order: O is in when only the 2 NPIECE tile loads are left, and delta is formed while
+            // those are on their way
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NPIECE) : "memory");
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb) {
                 const int qi = qw + qb * 32 + c32;
-                const int64_t lrow = (static_cast<int64_t>(b) * a.Hq + h) * a.T + qi;
                 // a query past the end: p = exp2(-huge) = 0, so nothing it holds matters
-                nlse[qb] = -1e30f, dl[qb] = 0.0f;
-                if (qi < a.T) nlse[qb] = -a.lse[lrow] * LOG2E;
+                nlse[qb] = -1e30f;
+                if (FUSE_DELTA) dl[qb] = 0.0f;
+                if (qi < a.T) nlse[qb] = -lse_raw[qb] * LOG2E;
                 if (FUSE_DELTA) {
-                    float part = 0.0f;  // this lane's half of the row: d = 16kk + 8g .. +7
+                    // this lane's half of the row (d = 16kk + 8g .. +7), in four sums so that the additions do not
+                    // wait for one another
+                    float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                     for (int kk = 0; kk < KK; ++kk) {
                         const bf16x8 o8 = staged(region_o, qb, kk);
@@ -245,20 +268,24 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
                         const u32x4 gv = *reinterpret_cast<const u32x4*>(&greg[qb][kk]);
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
-                            part = fmaf(__uint_as_float(ov[i] << 16), __uint_as_float(gv[i] << 16), part);
-                            part = fmaf(__uint_as_float(ov[i] & 0xFFFF0000u), __uint_as_float(gv[i] & 0xFFFF0000u), part);
+                            part[i] = fmaf(__uint_as_float(ov[i] << 16), __uint_as_float(gv[i] << 16), part[i]);
+                            part[i] = fmaf(__uint_as_float(ov[i] & 0xFFFF0000u), __uint_as_float(gv[i] & 0xFFFF0000u), part[i]);
                         }
                     }
-                    dl[qb] = xhalf_sum(part);
-                    if (qi < a.T && g == 0) a.delta[lrow] = dl[qb];
-                } else if (qi < a.T) {
-                    dl[qb] = a.delta[lrow];
+                    dl[qb] = xhalf_sum((part[0] + part[1]) + (part[2] + part[3]));
                 }
             }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         }
         __syncthreads();  // every wavefront has read its O region: the third tile may land there; tiles 0 and 1 are in
         dma_tile(2);      // waited for at the end of the first iteration
+        if (FUSE_DELTA) {  // written after the barrier, which would otherwise wait for the store to be acknowledged
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+                const int qi = qw + qb * 32 + c32;
+                if (qi < a.T && g == 0) a.delta[(static_cast<int64_t>(b) * a.Hq + h) * a.T + qi] = dl[qb];
+            }
+        }
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
@@ -274,15 +301,6 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
             for (int r = 0; r < 16; ++r) ndl[qb][r] = -dl[qb];
         const QueryVis qvis[2] = {QueryVis(qw + c32, a.T, a.causal, a.window, a.sinks),
                                   QueryVis(qw + 32 + c32, a.T, a.causal, a.window, a.sinks)};
-        f32x16 acc[2][DB];  // dQ^T of the two query blocks
-#pragma unroll
-        for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[qb][db][r] = 0.0f;
-                asm volatile("" : "+a"(acc[qb][db]));
-            }
 
 
         constexpr int PF = 3;              // fragments in flight
