@@ -301,7 +301,6 @@ int launch_mfma_fwd(const AttnArgs& a, hipStream_t st) {
     // Eight wavefronts (256 queries) per K/V tile halve the tile traffic per MFMA (2.7 % faster at T = 4096, 6 % at
     // T = 16384; slower at head_dim 64 and with a window). One such workgroup fills a CU, so it is only used where the
     // paired causal grid still gives every CU at least two of them in turn.
-    if (mfma_fwd3_takes(a)) return launch_mfma_fwd3(a, st);
     const int nqb256 = (a.T + 255) / 256;
     const bool wide = a.dk_dim == 128 && a.causal && a.window == 0 &&
                       static_cast<int64_t>((nqb256 + 1) / 2) * a.Hq * a.B >= 512;

@@ -124,8 +124,5 @@ int launch_mfma_dkdv3(const AttnArgs& a, hipStream_t st);
 // attn_bwd_dq3.hip: dQ with 64 queries per wavefront, same construction (head_dim 64 or 128, no band)
 bool mfma_dq3_takes(const AttnArgs& a);
 int launch_mfma_dq3(const AttnArgs& a, bool fuse_delta, hipStream_t st);
-// attn_fwd3.hip: forward with 64 queries per wavefront, same construction (head_dim 128, no band)
-bool mfma_fwd3_takes(const AttnArgs& a);
-int launch_mfma_fwd3(const AttnArgs& a, hipStream_t st);
 
 }  // namespace pk

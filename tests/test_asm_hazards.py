@@ -1,6 +1,6 @@
 """Register hazards around hand-placed matrix instructions.
 
-The forward, dK/dV and dQ kernels with 64 keys / queries per wavefront issue their matrix instructions from asm statements, so
+The dK/dV and dQ kernels with 64 keys / queries per wavefront issue their matrix instructions from asm statements, so
 the compiler does not know which registers those read and write and keeps none of the distances gfx950 needs between
 them and the vector instructions around them. Two of those distances are not enforced by the hardware either:
 
@@ -10,7 +10,7 @@ them and the vector instructions around them. Two of those distances are not enf
     than its pass count + 3 issue slots earlier (8 passes for v_mfma_f32_32x32x16_bf16) sees the old contents. A
     matrix instruction in between counts as 8 slots: it cannot enter the pipe before the writer has left it.
 
-This test compiles the three kernels to assembly and checks both distances on every path the assembler text shows
+This test compiles the two kernels to assembly and checks both distances on every path the assembler text shows
 (straight-line windows; a label or branch ends a window, which errs on the side of missing a hazard across a jump, so
 the kernels keep their own s_nop where a phase starts)."""
 import os
@@ -84,7 +84,7 @@ def scan(path):
     return found
 
 
-@pytest.mark.parametrize("src", ["attn_fwd3.hip", "attn_bwd_dq3.hip", "attn_bwd_dkdv3.hip"])
+@pytest.mark.parametrize("src", ["attn_bwd_dq3.hip", "attn_bwd_dkdv3.hip"])
 def test_no_unspaced_register_hazard_around_asm_matrix_instructions(src, tmp_path):
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
