@@ -41,7 +41,8 @@ def measured_traffic_bytes():
         for line in open(PMC_SUMMARY):
             m = re.match(r"(mfma_\w+)<", line)
             if m:
-                kernel = {"mfma_fwd": "fwd", "mfma_dq": "dq", "mfma_dkdv2": "dkdv", "mfma_dkdv3": "dkdv"}.get(m.group(1))
+                kernel = {"mfma_fwd": "fwd", "mfma_dq": "dq", "mfma_dq3": "dq", "mfma_dkdv2": "dkdv",
+                          "mfma_dkdv3": "dkdv"}.get(m.group(1))
             m = re.search(r"HBM traffic per launch: .* total ([0-9.]+) MB", line)
             if m and kernel:
                 out[kernel] = float(m.group(1)) * 1e6
