@@ -6,8 +6,8 @@ them and the vector instructions around them. Two of those distances are not enf
 
   * a matrix instruction that reads, as A or B, a register written by the vector instruction just before it sees the
     old contents (measured: at distance 0 the packed dS operand still held the fp32 product; at distance 1 it was right);
-  * a vector instruction, LDS / global store or matrix operand read of a register that a matrix instruction wrote less
-    than its pass count + 3 issue slots earlier (8 passes for v_mfma_f32_32x32x16_bf16) sees the old contents. A
+  * a vector instruction (a move out of an accumulation register included), LDS / global store or matrix operand read of
+    a register that a matrix instruction wrote less than its pass count + 3 issue slots earlier (8 passes for v_mfma_f32_32x32x16_bf16) sees the old contents. A
     matrix instruction in between counts as 8 slots: it cannot enter the pipe before the writer has left it.
 
 This test compiles the two kernels to assembly and checks both distances on every path the assembler text shows
@@ -30,12 +30,13 @@ MFMA_SLOTS = 8          # a matrix instruction in between enters the pipe only w
 
 
 def _regs(tok):
+    """registers named by one operand, as (file, index) pairs: ordinary (v) and accumulation (a) registers"""
     tok = tok.strip().rstrip(",")
-    m = re.fullmatch(r"v\[(\d+):(\d+)\]", tok)
+    m = re.fullmatch(r"([va])\[(\d+):(\d+)\]", tok)
     if m:
-        return set(range(int(m.group(1)), int(m.group(2)) + 1))
-    m = re.fullmatch(r"v(\d+)", tok)
-    return {int(m.group(1))} if m else set()
+        return {(m.group(1), i) for i in range(int(m.group(2)), int(m.group(3)) + 1)}
+    m = re.fullmatch(r"([va])(\d+)", tok)
+    return {(m.group(1), int(m.group(2)))} if m else set()
 
 
 def scan(path):
