@@ -135,6 +135,65 @@ def window_variant(ops, q, k, v, d_o, out, scale, B, H, T, dk, warmup, steps):
                          "unit": "GB/s", "frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}}
 
 
+def other_config(ops, name, B, Hq, Hkv, T, dk, theta, bound, steps=400, warmup=50):
+    """BASELINE configs 2 and 3 at their full shapes (bf16, causal, RoPE pre-applied to Q and K on the host in
+    fp32 before rounding): forward + backward in one loop, with per-kernel HIP events on every 8th step."""
+    import numpy as np
+    import torch
+    from paperkiln_amd import synth
+    dev = torch.device("cuda:0")
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
+    q = synth.bf16_round(synth.rope_interleaved(synth.randn(21, (B, T, Hq, dk)), theta))
+    k = synth.bf16_round(synth.rope_interleaved(synth.randn(22, (B, T, Hkv, dk)), theta))
+    v = synth.bf16_round(synth.randn(23, (B, T, Hkv, dk)))
+    g = synth.bf16_round(synth.randn(24, (B, T, Hq, dk)))
+    q, k, v, g = (torch.from_numpy(x).to(dev).bfloat16() for x in (q, k, v, g))
+    out = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
+           torch.empty(max(ops.bwd_workspace_bytes(q, k), 16), dtype=torch.uint8, device=dev))
+
+    def step(events=None):
+        def mark(nm):
+            if events is not None:
+                e = torch.cuda.Event(enable_timing=True)
+                e.record()
+                events.append((nm, e))
+        mark("start")
+        o, lse = ops.attn_fwd(q, k, v, scale, True)
+        mark("fwd")
+        ops.attn_bwd(q, k, v, o, lse, g, scale, True, out=out)
+        mark("bwd")
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = []
+    t0 = time.perf_counter()
+    for i in range(steps):
+        if i % 8 == 0:
+            ev = []
+            step(ev)
+            evs.append(ev)
+        else:
+            step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    kern = {}
+    for ev in evs:
+        for (_, e0), (nm, e1) in zip(ev[:-1], ev[1:]):
+            kern[nm] = kern.get(nm, 0.0) + e0.elapsed_time(e1) / len(evs)
+    pairs = synth.visible_pairs(T, True, 0, 0)
+    flops = 14.0 * dk * pairs * B * Hq
+    nbytes = (6.0 * Hq + 6.0 * Hkv) * B * T * dk * 2 + 2.0 * B * Hq * T * 4
+    tf, gbs = flops / (ms * 1e-3) / 1e12, nbytes / (ms * 1e-3) / 1e9
+    roof = ({"bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+             "frac": round(tf / PEAK_BF16_TFLOPS, 4)} if bound == "mfma" else
+            {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+             "frac": round(gbs / PEAK_HBM_GBS, 4)})
+    return {"workload": name, "steps": steps, "ms_per_step": round(ms, 4), "tflops": round(tf, 2),
+            "hbm_gb_per_s_algorithmic": round(gbs, 1), "tokens_per_s": round(B * T / (ms * 1e-3), 1),
+            "kernel_ms": {n: round(t, 4) for n, t in kern.items()}, "roofline": roof}
+
+
 def fp32_variant(ops, q, k, v, d_o, scale, B, H, T, dk):
     """Same shape with fp32 tensors (the reference's own element type): the kernels built on the fp32
     matrix instruction, priced against the fp32 MFMA peak."""
@@ -214,8 +273,8 @@ def main():
                     help="untimed run of the same step for this long before the counted warm-up: the card leaves its "
                          "idle clock state only under sustained load, and --warmup counts steps, not time")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--sections", default="window,fp32,llama",
-                    help="extra measurements beside the headline: any of window,fp32,llama (empty = headline only, "
+    ap.add_argument("--sections", default="window,cfg2,cfg3,fp32,llama",
+                    help="extra measurements beside the headline: any of window,cfg2,cfg3,fp32,llama (empty = headline only, "
                          "which is what the profiles under profiles/ were taken with)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -316,12 +375,21 @@ def main():
         "kernel_ms": {n: round(t, 4) for n, t in kern_ms.items()}, "kernel_event_steps": len(all_events),
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-                     "traffic": measured_traffic_bytes().get(dominant)},
+                     "traffic": measured_traffic_bytes().get(dominant),
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel as committed under "
+                                       "profiles/ (a constant read from that summary, not a measurement of this run)"},
     }
     extras = [x for x in args.sections.split(",") if x]
     if "window" in extras:
         res["window_variant"] = window_variant(ops, q, k, v, d_o, out, scale, B, H, T, dk, args.warmup,
                                                max(args.steps // 2, 1))
+    if "cfg2" in extras:
+        # 15.1 GFLOP against 101 MB: about 6 us of matrix work and 13 us of HBM time at peak, so the HBM roofline
+        res["cfg2"] = other_config(ops, "BASELINE config 2: causal MHA B=16 H=8 T=512 head_dim=64, RoPE theta=1e4 "
+                                   "pre-applied, bf16", 16, 8, 8, 512, 64, 1e4, "hbm")
+    if "cfg3" in extras:
+        res["cfg3"] = other_config(ops, "BASELINE config 3: causal GQA B=4 Hq=14 Hkv=2 T=2048 head_dim=64, RoPE "
+                                   "theta=1e6 pre-applied, bf16", 4, 14, 2, 2048, 64, 1e6, "mfma")
     if "fp32" in extras:
         res["fp32_variant"] = fp32_variant(ops, q, k, v, d_o, scale, B, H, T, dk)
     if "llama" in extras:

@@ -456,6 +456,9 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                         mma_v0(t0[kb], fr[j], kv[kb][j]);
                     else
                         mma_v(t0[kb], fr[j], kv[kb][j]);
+                    // The matrix instruction reads its C operand over its passes and nothing interlocks a vector write
+                    // to those registers: -delta stays allocated until a further matrix instruction has been issued.
+                    if (sl == 2 && rl == 1) asm volatile("" ::"v"(nd0));
                     if (kb == 0 && j + PF < KK) fr[j + PF] = xfrag(0, j + PF);
                     if (sl == NS / 2) side_loads(0);
                     if (sl == NS / 2 + 2 && rl == 1) nd1 = minus_delta(1);
@@ -475,6 +478,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                         mma_v0(t1[kb], fr[j], kv[kb][j]);
                     else
                         mma_v(t1[kb], fr[j], kv[kb][j]);
+                    if (sl == 2 && rl == 1) asm volatile("" ::"v"(nd1));
                     if (kb == 0 && j + PF < KK) fr[j + PF] = xfrag(1, j + PF);
                     // t0[0] was finished two matrix instructions before the first slot, t0[1] one before: the
                     // first half of the slots works on t0[0] only

@@ -138,6 +138,9 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
         offv[i] = row * v_st2 + ch * 16u;
     }
     auto unit_base = [&](int i) { return static_cast<uint32_t>(i < NI ? 256 * i + 64 * w : 256 * NI + 16 * w) * 16u; };
+    // m0 is set and used inside the one statement. It is not on the clobber list: the compiler treats m0 as a reserved
+    // register (it rejects the clobber with a warning), never keeps a value in it across other code and writes it
+    // directly before each instruction of its own that reads it, so nothing of the compiler's can be live in m0 here.
     auto dma16 = [](uint32_t lds, uint32_t voff, const char* base) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds), "v"(voff), "s"(base) : "memory");
     };

@@ -72,6 +72,13 @@ def exact_grads(q, k, v, d_o, scale, causal, window, sinks):
     return dq, dk_, dv
 
 
+# fp32 cases whose gradient missed the absolute 1e-5 against the reference arithmetic and were decided by the
+# float64 value instead, filled in as the tests of this module run: "<tag> <dQ|dK|dV>" -> (|gpu - ref|, gpu's and
+# the reference's distance from float64). test_fp32_cases_decided_by_float64_are_the_known_ones (last in this
+# file) holds the set to KNOWN_ARBITRATED, so a change that pushes more cases over 1e-5 fails there.
+ARBITRATED = {}
+
+
 def check_fp32_grads(tag, got, want, inputs):
     """The fp32 bar for dQ, dK, dV: max-abs 1e-5 against the CPU reference arithmetic. Where a gradient misses that
     (large sums: a sink key's dK / dV adds a term per query of the sequence), the float64 value of the same formula
@@ -86,6 +93,7 @@ def check_fp32_grads(tag, got, want, inputs):
         if exact is None:
             exact = exact_grads(*inputs)
         e_gpu, e_ref = maxabs(g, exact[idx]), maxabs(w, exact[idx])
+        ARBITRATED[f"{tag} {name}"] = (err, e_gpu, e_ref)
         print(f"  {tag} {name}: |gpu - ref| {err:.2e} >= 1e-5; against float64: gpu {e_gpu:.2e}, reference {e_ref:.2e}",
               flush=True)
         assert e_gpu <= max(2.0 * e_ref, FP32_TOL), (tag, name)
@@ -750,3 +758,24 @@ def test_long_sequence_prefix_property():
     assert float(dk_[:, P:].abs().max()) == 0.0 and float(dv[:, P:].abs().max()) == 0.0
     assert float((dk_[:, :P] - dkp).abs().max()) < 1e-4 * float(dkp.abs().max()) + 1e-5
     assert float((dv[:, :P] - dvp).abs().max()) < 1e-4 * float(dvp.abs().max()) + 1e-5
+
+
+# Every one of these is a sum over hundreds of queries (sink keys, long sequences); listed when the suite was
+# last run in full on an MI355X.
+KNOWN_ARBITRATED = {
+    "split tail T1501 w16 s3 d128 dK",  # |gpu - ref| 1.34e-05; vs float64: gpu 1.06e-05, reference 1.25e-05
+    "split tail T1501 w16 s3 d128 dV",  # 1.38e-05; 1.11e-05, 1.40e-05
+    "split tail T1501 w16 s3 d32 dV",   # 1.65e-05; 6.44e-06, 1.68e-05
+    "sweep9 d32 dK",                    # 1.34e-05; 9.51e-06, 9.34e-06
+    "sweep9 d32 dV",                    # 1.53e-05; 1.68e-05, 1.08e-05
+}
+
+
+def test_fp32_cases_decided_by_float64_are_the_known_ones():
+    """Runs last in this module. The fp32 bar is max-abs 1e-5 against the reference arithmetic; check_fp32_grads lets
+    a gradient that misses it pass when float64 shows the gap to be summation-order rounding. Which cases needed that
+    is recorded, and any case outside the committed list fails here."""
+    for k, (err, e_gpu, e_ref) in sorted(ARBITRATED.items()):
+        print(f"  arbitrated: {k}: |gpu - ref| {err:.2e}, vs float64 gpu {e_gpu:.2e} / reference {e_ref:.2e}")
+    new = set(ARBITRATED) - KNOWN_ARBITRATED
+    assert not new, f"fp32 cases newly over the absolute 1e-5 bar: {sorted(new)}"

@@ -113,3 +113,24 @@ def test_llama_class_against_the_reference_vectors():
     assert max(maxabs(grads[k[2:]], z[k]) for k in z.files if k.startswith("g:")) < 1e-5
     assert stats["peak_activation_bytes"] > 0
     assert model.adamw_step(3e-3, max_norm=1.0) == pytest.approx(float(z["total_norm"]), abs=1e-4)
+
+
+@pytest.mark.gpu
+def test_bf16_llama_class_gradients_against_the_reference_vectors():
+    """The bf16 model through the pybind class: loss within 2e-2 of the reference, every gradient tensor (plain and
+    checkpointed) within 2e-2 of its largest reference entry."""
+    m = module()
+    m.init(0)
+    z = np.load(os.path.join(GOLDEN, "llama_T16x2_stacked.npz"))
+    vocab, d, L, H, dff = (int(x) for x in z["cfg"])
+    model = m.Llama(vocab, d, L, H, dff, compute_dtype="bf16")
+    model.load_state_dict({k[2:]: z[k] for k in z.files if k.startswith("p:")})
+    for ckpt in (False, True):
+        loss, _ = model.loss_backward([int(i) for i in z["ids"]], [int(t) for t in z["targets"]], int(z["seq_len"]),
+                                      checkpoint_blocks=ckpt)
+        assert abs(loss - float(z["loss"])) < 2e-2
+        grads = model.grads()
+        for k in z.files:
+            if k.startswith("g:"):
+                bar = 2e-2 * float(np.abs(z[k]).max())
+                assert maxabs(grads[k[2:]], z[k]) <= bar, (k, ckpt)

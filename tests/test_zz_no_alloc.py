@@ -19,6 +19,10 @@ def inputs(B, T, Hq, Hkv, dk, dtype, seed):
     return mk(Hq), mk(Hkv), mk(Hkv), mk(Hq)
 
 
+def torch_allocations():
+    return torch.cuda.memory_stats().get("allocation.all.allocated", 0)
+
+
 # (element type, head_dim, window, sinks, first shape (B, T, Hq, Hkv), second and smaller shape)
 CASES = [
     (torch.bfloat16, 128, 0, 0, (2, 1024, 4, 2), (1, 300, 2, 2)),     # matrix-core kernels, causal
@@ -38,8 +42,16 @@ def test_static_scratch_backward_equals_workspace_backward(case):
         want = ops.attn_bwd(q, k, v, o, lse, d_o, scale, True, window, sinks)
         out = tuple(torch.full_like(x, float("nan")) for x in (q, k, v))
         print(f"\n  static backward, call {n}: {dtype} B={B} T={T} Hq={Hq} Hkv={Hkv} dk={dk} w={window} s={sinks}", flush=True)
+        # the property the entry point exists for: nothing is allocated, neither from the library's own pool
+        # nor from the device (outputs are passed in, so torch allocates nothing either: its count of
+        # allocation requests, which only ever grows, stands still)
+        L = _lib.lib()
+        torch.cuda.synchronize()
+        before = (L.pk_live_bytes(), L.pk_peak_bytes(), torch.cuda.mem_get_info()[0], torch_allocations())
         got = ops.attn_bwd_static(q, k, v, o, lse, d_o, scale, True, window, sinks, out=out)
         torch.cuda.synchronize()
+        after = (L.pk_live_bytes(), L.pk_peak_bytes(), torch.cuda.mem_get_info()[0], torch_allocations())
+        assert after == before, f"call {n}: the static backward changed an allocation counter: {before} -> {after}"
         for name, a, b in zip(("dQ", "dK", "dV"), got, want):
             assert torch.isfinite(a.float()).all(), name
             assert torch.equal(a, b), f"call {n}: {name}"
