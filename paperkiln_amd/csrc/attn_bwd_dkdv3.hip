@@ -108,12 +108,16 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
     // Full-causal: key block i is seen by T - 128i queries; blocks i and nkb-1-i
     // are taken back to back so that every workgroup carries the same work.
     const bool paired = a.causal && a.window == 0;
-    int blk, rr, kvu;
+    // hs > 1: the query heads of the group are dealt to hs workgroups (gqa_head_split); this one takes heads
+    // [hfirst, hfirst + nh) of the group and leaves fp32 partial sums for launch_gqa_reduce
+    const int hs = a.head_split;
+    int blk, rr = 0, kvu;
     if (a.window > 0 && a.sinks > 0 && nkb > 1) {
         if (!xcd_map_block0_first(nkb, a.Hkv * a.B, blk, kvu)) return;
-    } else if (!xcd_map(paired ? (nkb + 1) / 2 : nkb, 1, a.Hkv * a.B, blk, rr, kvu)) {
+    } else if (!xcd_map(paired ? (nkb + 1) / 2 : nkb, hs, a.Hkv * a.B, blk, rr, kvu)) {
         return;
     }
+    const int hfirst = rr * rep / hs, nh = (rr + 1) * rep / hs - hfirst;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv;
     const float cexp = a.scale * LOG2E;
     const int npass = (paired && blk != nkb - 1 - blk) ? 2 : 1;
@@ -151,7 +155,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
         const int qt_lo = a.causal ? k0 / BMQ : 0;
         const int qt_hi = (a.window > 0 && k0 >= a.sinks) ? min(a.T - 1, khi + a.window - 1) / BMQ : (a.T - 1) / BMQ;
         const int nqt = qt_hi - qt_lo + 1;
-        const int steps = nqt * rep;
+        const int steps = nqt * nh;
 
         u32x4 qr[CPT], gr[CPT];
         // Staging is all this wavefront's own time (nobody shares its SIMD), so it is kept to the loads and stores
@@ -181,7 +185,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
         // per SIMD issues every instruction of its own, scalar ones included, at about five clocks each.
         int f_h = 0, f_qt = 0;       // head inside the group and query tile of the next fetch
         int f_q0 = qt_lo * BMQ;      // first query row of that tile
-        const int h0 = hk * rep;
+        const int h0 = hk * rep + hfirst;
         const char* f_qb = reinterpret_cast<const char*>(a.q) + (b * a.q_sb + h0 * a.q_sh + f_q0 * a.q_st) * 2;
         const char* f_gb = reinterpret_cast<const char*>(a.d_o) + (b * a.do_sb + h0 * a.do_sh + f_q0 * a.do_st) * 2;
         // per-row scalars: wavefronts 0 and 1 carry LSE of rows 32w + lane (lanes 0-31), wavefronts 2 and 3 delta
@@ -208,7 +212,7 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
             f_roff = static_cast<uint32_t>(min(rrow, last)) * 4u;
             // masks instead of selects: a nested select becomes a branch, and a taken branch costs the most of all
             const int64_t in_head = -static_cast<int64_t>(f_qt + 1 < nqt);
-            const int64_t next_head = ~in_head & -static_cast<int64_t>(f_h + 1 < rep);
+            const int64_t next_head = ~in_head & -static_cast<int64_t>(f_h + 1 < nh);
             f_qb += (qd_tile & in_head) | (qd_head & next_head);
             f_gb += (gd_tile & in_head) | (gd_head & next_head);
             f_rb += (rd_tile & in_head) | (rd_head & next_head);
@@ -488,6 +492,9 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 finish_head(0, e0, op0);
+                // the packs stay ahead of the fragment reads: a matrix instruction must not directly follow the
+                // vector instruction that writes one of its operands
+                __builtin_amdgcn_sched_barrier(0);
                 // ---- phase 3: GEMM2(block 0) || elementwise(block 1)
 #pragma unroll
                 for (int j = 0; j < PF; ++j) fr[j] = yfrag(0, j);
@@ -504,6 +511,9 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 finish_head(1, e1, op1);
+                // the packs stay ahead of the fragment reads: a matrix instruction must not directly follow the
+                // vector instruction that writes one of its operands
+                __builtin_amdgcn_sched_barrier(0);
                 // ---- phase 4: GEMM2(block 1) || staging, one piece per matrix instruction
 #pragma unroll
                 for (int j = 0; j < PF; ++j) fr[j] = yfrag(1, j);
@@ -537,10 +547,21 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
         for (int kb = 0; kb < 2; ++kb) {
             const int kj = kj0 + 32 * kb;
             if (kj >= a.T) continue;
+            const float sc = rl == 0 ? 1.0f : a.scale;
+            if (hs > 1) {  // fp32 partial sums of this split, rows of pitch D
+                float* prow = a.part + ((static_cast<size_t>(kvu) * hs + rr) * 2 + (rl == 0 ? 1 : 0)) * a.T * D +
+                              static_cast<size_t>(kj) * D;
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int qd = 0; qd < 4; ++qd)
+                        store4g<true>(prow, TrMap<D>::col0(db, qd, g), acc[kb][db][qd * 4] * sc, acc[kb][db][qd * 4 + 1] * sc,
+                                      acc[kb][db][qd * 4 + 2] * sc, acc[kb][db][qd * 4 + 3] * sc);
+                continue;
+            }
             void* dst = rl == 0 ? a.dv : a.dk;
             const int64_t ob = rl == 0 ? b * a.dv_sb + hk * a.dv_sh + kj * a.dv_st
                                        : b * a.dk_sb + hk * a.dk_sh + kj * a.dk_st;
-            const float sc = rl == 0 ? 1.0f : a.scale;
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 if (!GF32) {
@@ -564,14 +585,40 @@ __global__ __launch_bounds__(256, 1) void mfma_dkdv3(AttnArgs a) {
     }
 }
 
+// dK / dV = the splits' partial sums added in split order; four consecutive head_dim elements per thread
+template <bool GF32>
+__global__ __launch_bounds__(256) void gqa_reduce(AttnArgs a) {
+    const int D = a.dk_dim, hs = a.head_split;
+    const int64_t per_unit = static_cast<int64_t>(a.T) * D / 4;  // quads per (unit, tensor)
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= per_unit * 2 * a.Hkv * a.B) return;
+    const int64_t quad = idx % per_unit;
+    const int which = static_cast<int>((idx / per_unit) & 1), kvu = static_cast<int>(idx / (2 * per_unit));
+    const int hk = kvu % a.Hkv, b = kvu / a.Hkv;
+    const int t = static_cast<int>(quad / (D / 4)), d = static_cast<int>(quad % (D / 4)) * 4;
+    const size_t split_stride = static_cast<size_t>(2) * a.T * D;
+    const float* src = a.part + (static_cast<size_t>(kvu) * hs * 2 + which) * a.T * D + static_cast<size_t>(t) * D + d;
+    f32x4 sum = *reinterpret_cast<const f32x4*>(src);
+    for (int r = 1; r < hs; ++r) {
+        const f32x4 x = *reinterpret_cast<const f32x4*>(src + r * split_stride);
+        sum[0] += x[0], sum[1] += x[1], sum[2] += x[2], sum[3] += x[3];
+    }
+    void* dst = which == 0 ? a.dk : a.dv;
+    const int64_t at = which == 0 ? b * a.dk_sb + hk * a.dk_sh + t * a.dk_st + d : b * a.dv_sb + hk * a.dv_sh + t * a.dv_st + d;
+    store4g<GF32>(dst, at, sum[0], sum[1], sum[2], sum[3]);
+}
+
 template <int D, bool GF32>
 int launch(const AttnArgs& a, hipStream_t st) {
     const int nb128 = (a.T + 127) / 128;
     const bool paired = a.causal && a.window == 0;
-    hipLaunchKernelGGL((mfma_dkdv3<D, GF32>), dim3(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, 1, a.Hkv * a.B)),
-                       dim3(256), 0, st, a);
+    const int hs = a.part ? a.head_split : 1;
+    AttnArgs b = a;
+    b.head_split = hs;
+    hipLaunchKernelGGL((mfma_dkdv3<D, GF32>), dim3(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, hs, a.Hkv * a.B)),
+                       dim3(256), 0, st, b);
     PK_HIP(hipGetLastError());
-    return PK_OK;
+    return hs > 1 ? launch_gqa_reduce(b, st) : PK_OK;
 }
 
 }  // namespace
@@ -583,6 +630,17 @@ bool mfma_dkdv3_takes(const AttnArgs& a) {
     // (0.22 against 0.24 ms at head_dim 128, window 256 + 4 sinks, T 4096): the steps are
     // few, most of them masked, and the workgroup that owns the sink keys alone walks every query tile
     return (a.dk_dim == 128 || a.dk_dim == 64) && a.window == 0 && reach < (int64_t{1} << 31);
+}
+
+int launch_gqa_reduce(const AttnArgs& a, hipStream_t st) {
+    const int64_t quads = static_cast<int64_t>(a.T) * a.dk_dim / 4 * 2 * a.Hkv * a.B;
+    const dim3 grid(static_cast<unsigned>((quads + 255) / 256));
+    if (a.grad_f32)
+        hipLaunchKernelGGL(gqa_reduce<true>, grid, dim3(256), 0, st, a);
+    else
+        hipLaunchKernelGGL(gqa_reduce<false>, grid, dim3(256), 0, st, a);
+    PK_HIP(hipGetLastError());
+    return PK_OK;
 }
 
 int launch_mfma_dkdv3(const AttnArgs& a, hipStream_t st) {

@@ -101,6 +101,22 @@ size_t tail_bytes(const pk_attn_shape* s) {
     return pad + sink_tail_bytes(s->B * s->Hkv, t.nch, s->dk);
 }
 
+// (GQA, band-free bf16 only) the per-split partial dK / dV of the dK/dV launch, after delta and the sink tail
+int head_split_of(const pk_attn_shape* s) {
+    const Mask m = effective_mask(s);
+    return gqa_head_split(s->B, s->T, s->Hq, s->Hkv, s->dk, s->causal != 0, m.window, s->dtype == PK_BF16);
+}
+size_t part_bytes(const pk_attn_shape* s) {
+    const int hs = head_split_of(s);
+    if (hs <= 1) return 0;
+    const size_t before = delta_bytes(s) + tail_bytes(s);
+    return (256 - before % 256) % 256 + gqa_part_bytes(s->B * s->Hkv, hs, s->T, s->dk);
+}
+
+int bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k, const pk_tensor4* v,
+               const pk_tensor4* o, const float* lse, const pk_tensor4* d_o, const pk_tensor4* dq, const pk_tensor4* dk,
+               const pk_tensor4* dv, void* workspace, size_t workspace_bytes, int stages, bool split_heads, void* stream);
+
 void fill_common(AttnArgs& a, const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k,
                  const pk_tensor4* v, const pk_tensor4* o) {
     std::memset(&a, 0, sizeof a);
@@ -113,6 +129,7 @@ void fill_common(AttnArgs& a, const pk_attn_shape* s, const pk_tensor4* q, const
     a.causal = s->causal != 0; a.window = m.window; a.sinks = m.sinks;
     a.scale = s->scale;
     a.grad_f32 = s->grad_dtype == PK_F32;
+    a.head_split = 1;
 }
 
 }  // namespace
@@ -158,7 +175,7 @@ int pk_attn_fwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k
 
 size_t pk_attn_bwd_workspace_bytes(const pk_attn_shape* s) {
     if (check_shape(s, "pk_attn_bwd_workspace_bytes")) return 0;
-    return delta_bytes(s) + tail_bytes(s);
+    return delta_bytes(s) + tail_bytes(s) + part_bytes(s);
 }
 
 int pk_attn_bwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k, const pk_tensor4* v,
@@ -173,7 +190,11 @@ int pk_attn_bwd_static(const pk_attn_shape* s, const pk_tensor4* q, const pk_ten
                        const pk_tensor4* o, const float* lse, const pk_tensor4* d_o, const pk_tensor4* dq,
                        const pk_tensor4* dk, const pk_tensor4* dv, void* stream) {
     if (int rc = check_shape(s, "pk_attn_bwd_static")) return rc;
-    const size_t need = delta_bytes(s) + tail_bytes(s);
+    // The GQA head split of the dK/dV launch needs room for its partial sums; where that does not fit the array the
+    // heads of a group are walked by one workgroup as before (same results up to the order of summation).
+    size_t need = delta_bytes(s) + tail_bytes(s);
+    const bool split_heads = need + part_bytes(s) <= SCRATCH_BYTES;
+    if (split_heads) need += part_bytes(s);
     if (need > SCRATCH_BYTES)
         return fail(PK_ERR_WORKSPACE, "pk_attn_bwd_static: this shape needs " + std::to_string(need) +
                                           " bytes of scratch, the static array holds " + std::to_string(SCRATCH_BYTES) +
@@ -181,8 +202,9 @@ int pk_attn_bwd_static(const pk_attn_shape* s, const pk_tensor4* q, const pk_ten
     void* ws = nullptr;
     if (int rc = scratch_of_current_device(&ws)) return rc;
     // Every word of the workspace the kernels read they have written earlier in the same call (D_i by the dQ
-    // kernel, each piece's partial sink rows by its own workgroup), so nothing has to be cleared between calls.
-    return pk_attn_bwd_stages(s, q, k, v, o, lse, d_o, dq, dk, dv, ws, SCRATCH_BYTES, PK_BWD_ALL, stream);
+    // kernel, each piece's partial sink rows and each split's partial dK / dV by its own workgroup), so nothing has
+    // to be cleared between calls.
+    return bwd_stages(s, q, k, v, o, lse, d_o, dq, dk, dv, ws, SCRATCH_BYTES, PK_BWD_ALL, split_heads, stream);
 }
 
 int pk_attn_bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k,
@@ -190,12 +212,24 @@ int pk_attn_bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_ten
                        const pk_tensor4* d_o, const pk_tensor4* dq, const pk_tensor4* dk,
                        const pk_tensor4* dv, void* workspace, size_t workspace_bytes, int stages,
                        void* stream) {
+    return bwd_stages(s, q, k, v, o, lse, d_o, dq, dk, dv, workspace, workspace_bytes, stages, true, stream);
+}
+
+}  // extern "C"
+
+namespace pk {
+namespace {
+
+int bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k, const pk_tensor4* v,
+               const pk_tensor4* o, const float* lse, const pk_tensor4* d_o, const pk_tensor4* dq, const pk_tensor4* dk,
+               const pk_tensor4* dv, void* workspace, size_t workspace_bytes, int stages, bool split_heads, void* stream) {
     if (int rc = check_shape(s, "pk_attn_bwd")) return rc;
     if (stages <= 0 || (stages & ~PK_BWD_ALL))
         return fail(PK_ERR_ARGUMENT, "pk_attn_bwd_stages: stages must be a non-empty subset of PK_BWD_ALL");
     if (bad(q) || bad(k) || bad(v) || bad(o) || !lse || bad(d_o) || bad(dq) || bad(dk) || bad(dv))
         return fail(PK_ERR_ARGUMENT, "pk_attn_bwd: null tensor");
-    if (!workspace || workspace_bytes < pk_attn_bwd_workspace_bytes(s))
+    const size_t before_part = delta_bytes(s) + tail_bytes(s);
+    if (!workspace || workspace_bytes < before_part + (split_heads ? part_bytes(s) : 0))
         return fail(PK_ERR_WORKSPACE, "pk_attn_bwd: workspace smaller than pk_attn_bwd_workspace_bytes()");
     if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
         return fail(PK_ERR_ARGUMENT, "pk_attn_bwd: workspace must be 16-byte aligned");
@@ -211,10 +245,15 @@ int pk_attn_bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_ten
         const size_t db = delta_bytes(s);
         a.tail = reinterpret_cast<float*>(static_cast<char*>(workspace) + db + (256 - db % 256) % 256);
     }
+    if (split_heads && part_bytes(s)) {
+        a.head_split = head_split_of(s);
+        a.part = reinterpret_cast<float*>(static_cast<char*>(workspace) + before_part + (256 - before_part % 256) % 256);
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (s->dtype == PK_BF16 && mfma_supported(a)) return launch_mfma_bwd(a, stages, st);
     if (s->dtype == PK_F32 && f32_mfma_supported(a)) return launch_f32_mfma_bwd(a, stages, st);
     return launch_generic_bwd(a, s->dtype == PK_BF16, stages, st);
 }
 
-}  // extern "C"
+}  // namespace
+}  // namespace pk

@@ -34,6 +34,8 @@ struct AttnArgs {
     void* dv;
     float* delta;    // bwd scratch: rowsum(dO .* O)   [B,Hq,T]
     float* tail;     // bwd scratch: partial dK/dV rows of the sink keys (see sink_tail), or null
+    float* part;     // bwd scratch: per-split partial dK/dV of a GQA group (see gqa_head_split), or null
+    int head_split;  // number of workgroups that share the query heads of one KV head in the dK/dV launch (1 = no split)
     int64_t q_sb, q_st, q_sh;
     int64_t k_sb, k_st, k_sh;
     int64_t v_sb, v_st, v_sh;
@@ -100,6 +102,28 @@ __host__ inline bool sink_tail_pays(const SinkTail& t, int T, int window, int kv
                        ((128 + window) / step + prologue);
     return chain > rest;
 }
+// GQA head split. One dK/dV workgroup owns 128 keys of one (batch, KV head) and walks the query tiles of every
+// query head of the group in turn, so a launch has ceil(T/128) * B * Hkv workgroups (half that when causal
+// blocks are paired) however many query heads there are: 14 query heads on 2 KV heads at B = 4, T = 2048
+// fill 64 of 256 CUs. Where the launch would leave CUs idle, the heads of a group are dealt to `hs`
+// workgroups; split r takes heads [r rep / hs, (r + 1) rep / hs), writes its fp32 partial dK and dV to
+//   part[((unit * hs + r) * 2 + {0: dK, 1: dV}) * T + key][head_dim]
+// and a second kernel adds the splits in order (no atomics, repeatable). Band-free bf16 kernels only.
+__host__ __device__ inline int gqa_head_split(int B, int T, int Hq, int Hkv, int dk, int causal, int window, int bf16) {
+    const int rep = Hq / Hkv;
+    if (!bf16 || rep <= 1 || window != 0 || (dk != 64 && dk != 128)) return 1;
+    const int nkb = (T + 127) / 128;
+    const long long wgs = static_cast<long long>(causal ? (nkb + 1) / 2 : nkb) * B * Hkv;
+    if (wgs >= 384) return 1;  // at least one and a half workgroups per CU already
+    const int hs = static_cast<int>((512 + wgs - 1) / wgs);
+    return hs < rep ? hs : rep;
+}
+__host__ __device__ inline size_t gqa_part_bytes(int kv_units, int hs, int T, int dk) {
+    return hs > 1 ? sizeof(float) * 2 * static_cast<size_t>(kv_units) * hs * T * dk : 0;
+}
+// adds the splits into dK / dV; attn_bwd_dkdv3.hip
+int launch_gqa_reduce(const AttnArgs& a, hipStream_t st);
+
 // adds the pieces into dK/dV rows [0, sinks) of every (batch, KV head); attn_bwd_dkdv2.hip
 int launch_sink_tail_reduce(const AttnArgs& a, hipStream_t st);
 

@@ -760,6 +760,37 @@ def test_long_sequence_prefix_property():
     assert float((dv[:, :P] - dvp).abs().max()) < 1e-4 * float(dvp.abs().max()) + 1e-5
 
 
+@pytest.mark.parametrize("B,T,Hq,Hkv,dk", [(8, 2048, 14, 2, 64), (1, 1000, 6, 2, 128), (2, 640, 8, 1, 128)])
+def test_gqa_head_split_of_the_dkdv_launch(B, T, Hq, Hkv, dk):
+    """Few (batch, KV head) units: the query heads of a group are dealt to several dK/dV workgroups whose fp32 partial
+    sums a second kernel adds in a fixed order (7 heads over 4 workgroups in the first case, a ragged deal). Same
+    result as MHA over repeated KV heads with the group's dK / dV summed, bit-identical from call to call, and bit-identical
+    between the workspace entry point and the one with the library's own scratch where that holds the partial sums."""
+    q, k, v, d_o = make(B, T, Hq, Hkv, dk, 1.0, 4300 + T)
+    scale = float(np.float32(1.0 / np.sqrt(dk)))
+    tq, tk, tv, tg = (torch.from_numpy(x).cuda().bfloat16() for x in (q, k, v, d_o))
+    rep = Hq // Hkv
+    o, lse = ops.attn_fwd(tq, tk, tv, scale, True)
+    sh_one = ops.bwd_workspace_bytes(tq, tq)   # the same shape as MHA: delta only
+    assert ops.bwd_workspace_bytes(tq, tk) > sh_one, "this shape is expected to split the heads of a group"
+    dq, dk_, dv = ops.attn_bwd(tq, tk, tv, o, lse, tg, scale, True, grad_dtype=torch.float32)
+    again = ops.attn_bwd(tq, tk, tv, o, lse, tg, scale, True, grad_dtype=torch.float32)
+    assert all(torch.equal(a, b) for a, b in zip((dq, dk_, dv), again))
+    kr, vr = tk.repeat_interleave(rep, dim=2), tv.repeat_interleave(rep, dim=2)
+    dq2, dk2, dv2 = ops.attn_bwd(tq, kr, vr, o, lse, tg, scale, True, grad_dtype=torch.float32)
+    assert torch.equal(dq2, dq)
+    sk = dk2.view(B, T, Hkv, rep, dk).sum(dim=3)
+    sv = dv2.view(B, T, Hkv, rep, dk).sum(dim=3)
+    assert float((sk - dk_).abs().max()) < 1e-3 * float(dk_.abs().max()) + 1e-4  # fp32 sums in another order
+    assert float((sv - dv).abs().max()) < 1e-3 * float(dv.abs().max()) + 1e-4
+    # bf16 gradients through the same split, and the static-scratch entry point
+    b16 = ops.attn_bwd(tq, tk, tv, o, lse, tg, scale, True)
+    assert float((b16[1].float() - dk_).abs().max()) <= 2e-2 * max(1.0, float(dk_.abs().max()))
+    if ops.bwd_workspace_bytes(tq, tk) <= 32 << 20:
+        st = ops.attn_bwd_static(tq, tk, tv, o, lse, tg, scale, True)
+        assert all(torch.equal(a, b) for a, b in zip(b16, st))
+
+
 # Every one of these is a sum over hundreds of queries (sink keys, long sequences); listed when the suite was
 # last run in full on an MI355X.
 KNOWN_ARBITRATED = {
