@@ -28,8 +28,11 @@ namespace pk {
 namespace {
 
 constexpr float LOG2E = 1.4426950408889634f;
-constexpr int BMQ = 64;   // queries per step
-constexpr int BNK = 128;  // keys per workgroup (4 blocks of 32)
+// Two geometries. 128 keys per workgroup (8 wavefronts, 64-query steps, one workgroup per CU) is the general one.
+// With a narrow band a key block meets only a handful of query steps, and the fixed costs of a workgroup -- resident
+// rows, first tiles, pipeline fill, epilogue -- weigh as much as its steps; there a workgroup takes 64 keys with 4
+// wavefronts and 32-query steps, so that TWO workgroups fit a CU (registers: still two wavefronts per SIMD; LDS: 61 KB
+// each) and one's fixed costs run beside the other's steps. Finer tiles also waste less on the band's edges.
 typedef __fp16 h16x2 __attribute__((ext_vector_type(2)));
 
 template <bool F32>
@@ -45,23 +48,25 @@ __device__ inline void store4g(void* base, int64_t idx, float x0, float x1, floa
 
 // TAIL: the launch carries the extra workgroups of a split sink tail (a separate instantiation, so
 // that the plain causal kernel keeps its register budget)
-template <int D, bool GF32, bool TAIL>
-__global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
+template <int D, bool GF32, bool TAIL, int BNK, int BMQ>
+__global__ __launch_bounds__(4 * BNK, 2) void mfma_dkdv2(AttnArgs a) {
     constexpr int KK = D / 16, DB = D / 32;
+    constexpr int NTHR = 4 * BNK, NKB = BNK / 32, NQB = BMQ / 32;  // threads; 32-key blocks; 32-query blocks per step
     constexpr int S = D + 8;            // tile row pitch (elements): 16-byte row reads conflict-free
     constexpr int NCH = D / 8;          // 16-byte chunks per row
-    constexpr int CPT = BMQ * NCH / 512;  // chunks per thread per tensor per step
+    constexpr int CPT = BMQ * NCH / NTHR;  // chunks per thread per tensor per step
+    static_assert(CPT >= 1 && BMQ * NCH % NTHR == 0, "every thread stages the same number of chunks");
     __shared__ __attribute__((aligned(16))) uint16_t tiles[2][3][BMQ * S];  // [Q | dO][ring slot]
     uint16_t (*const Qs)[BMQ * S] = tiles[0];
     uint16_t (*const dOs)[BMQ * S] = tiles[1];
-    __shared__ __attribute__((aligned(16))) uint16_t Pbuf[2][2][4][2 * 64 * 8];  // [step parity][query block][key block][half][lane][8]
+    __shared__ __attribute__((aligned(16))) uint16_t Pbuf[2][NQB][NKB][2 * 64 * 8];  // [step parity][query block][key block][half][lane][8]
     __shared__ __attribute__((aligned(16))) float nlse_s[3][BMQ];            // -LSE * log2(e)
     __shared__ __attribute__((aligned(16))) float dl_s[3][BMQ];
 
     const int lane = threadIdx.x & 63;
     // the wavefront index as a scalar: every test on it becomes a scalar branch
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int role = w >> 2, kbw = w & 3;
+    const int role = w / NKB, kbw = w % NKB;
     const int g = lane >> 5, c32 = lane & 31;
     // Lane parts of the two LDS operand addresses (elements): a 16-byte row read at
     // (row c32, column 8g) and a transposing read as lds_read_tr_operand_perm lays it out.
@@ -124,6 +129,8 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
         if (TAIL && chunk >= 0) {
             qt_lo = (tl.q0 + chunk * TAIL_CHUNK) / BMQ;
             qt_hi = min(a.T - 1, tl.q0 + (chunk + 1) * TAIL_CHUNK - 1) / BMQ;
+        } else if (TAIL && kblk == 0) {
+            qt_hi = tl.q0 / BMQ - 1;  // the band part of block 0 ends where the chunks begin, whatever the block size
         }
         const int nqt = qt_hi - qt_lo + 1;
         const int steps = nqt * rep;
@@ -134,7 +141,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
             const int h = hk * rep + step / nqt, q0 = (qt_lo + step % nqt) * BMQ;
 #pragma unroll
             for (int i = 0; i < CPT; ++i) {
-                const int c = threadIdx.x + 512 * i;
+                const int c = threadIdx.x + NTHR * i;
                 const int row = c / NCH, ch = c % NCH;
                 const int t = min(q0 + row, a.T - 1);
                 qr[i] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.q) + b * a.q_sb + h * a.q_sh +
@@ -157,7 +164,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
             asm volatile("" : "+v"(tid));
 #pragma unroll
             for (int i = 0; i < CPT; ++i) {
-                const int c = tid + 512 * i;
+                const int c = tid + NTHR * i;
                 const int row = c / NCH, ch = c % NCH;
                 *reinterpret_cast<u32x4*>(Qs[slot] + lds_row<D>(row) * S + ch * 8) = qr[i];
                 *reinterpret_cast<u32x4*>(dOs[slot] + lds_row<D>(row) * S + ch * 8) = gr[i];
@@ -214,7 +221,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
                     asm volatile("" : "+v"(xrow), "+v"(ytr));
                     const uint16_t* flat = &tiles[0][0][0];
 #pragma unroll
-                    for (int qb = 0; qb < 2; ++qb) {
+                    for (int qb = 0; qb < NQB; ++qb) {
                         int qlo;
                         if (!block_live(s, qb, qlo)) continue;
                         // One accumulator chain: the other role's wavefront on this SIMD issues
@@ -274,7 +281,7 @@ __global__ __launch_bounds__(512, 2) void mfma_dkdv2(AttnArgs a) {
                     asm volatile("" : "+v"(xrow), "+v"(ytr));
                     const uint16_t* flat = &tiles[0][0][0];
 #pragma unroll
-                    for (int qb = 0; qb < 2; ++qb) {
+                    for (int qb = 0; qb < NQB; ++qb) {
                         int qlo;
                         if (!block_live(sp, qb, qlo)) continue;
                         f32x16 dp;
@@ -365,10 +372,10 @@ __global__ __launch_bounds__(256) void sink_tail_reduce(AttnArgs a, int nch) {
     }
 }
 
-template <int D, bool GF32>
-int launch(const AttnArgs& a_in, hipStream_t st) {
+template <int D, bool GF32, int BNK, int BMQ>
+int launch_geo(const AttnArgs& a_in, hipStream_t st) {
     AttnArgs a = a_in;
-    const int nb128 = (a.T + 127) / 128;
+    const int nkb = (a.T + BNK - 1) / BNK;
     const bool paired = a.causal && a.window == 0;
     SinkTail tl = a.tail ? sink_tail(a.T, a.window, a.sinks) : SinkTail{0, 0};
     // a tail step keeps two of the eight wavefronts busy but takes as long as a full one (measured)
@@ -377,14 +384,24 @@ int launch(const AttnArgs& a_in, hipStream_t st) {
         tl.nch = 0;
     }
     if (tl.nch > 0) {
-        hipLaunchKernelGGL((mfma_dkdv2<D, GF32, true>), dim3(xcd_grid(nb128 + tl.nch, 1, a.Hkv * a.B)), dim3(512), 0, st, a);
+        hipLaunchKernelGGL((mfma_dkdv2<D, GF32, true, BNK, BMQ>), dim3(xcd_grid(nkb + tl.nch, 1, a.Hkv * a.B)), dim3(4 * BNK), 0,
+                           st, a);
         PK_HIP(hipGetLastError());
         return launch_sink_tail_reduce(a, st);
     }
-    hipLaunchKernelGGL((mfma_dkdv2<D, GF32, false>), dim3(xcd_grid(paired ? (nb128 + 1) / 2 : nb128, 1, a.Hkv * a.B)),
-                       dim3(512), 0, st, a);
+    hipLaunchKernelGGL((mfma_dkdv2<D, GF32, false, BNK, BMQ>), dim3(xcd_grid(paired ? (nkb + 1) / 2 : nkb, 1, a.Hkv * a.B)),
+                       dim3(4 * BNK), 0, st, a);
     PK_HIP(hipGetLastError());
     return PK_OK;
+}
+
+template <int D, bool GF32>
+int launch(const AttnArgs& a, hipStream_t st) {
+    // A band of a few key blocks: the small geometry, two workgroups per CU. Measured at B=4 H=16 T=4096, head_dim 128,
+    // small against large: window 128 0.190 / 0.229 ms, 256 0.190 / 0.223, 512 0.264 / 0.276, 1024 0.404 / 0.387,
+    // 2048 0.623 / 0.565; at head_dim 64 (window 256) 0.142 / 0.134, so only head_dim 128 takes it.
+    if (D == 128 && a.window > 0 && a.window <= 512) return launch_geo<D, GF32, 64, 32>(a, st);
+    return launch_geo<D, GF32, 128, 64>(a, st);
 }
 
 }  // namespace
