@@ -70,7 +70,34 @@ __device__ inline void store_kv_lds(uint16_t* Ks, uint16_t* Vs, const u32x4* kr,
 // final O = acc / l and LSE = m*scale + ln(l) are exact for any reference m.
 constexpr float LAZY_T = 6.0f;
 
-template <int D, int NQ, int OCC, int NW>
+// A K or V tile's position as a scalar buffer resource that is ADVANCED from tile to tile instead of rebuilt: base
+// pointer plus the bytes left up to the end of the last row (the resource's num_records, so rows past the end read
+// as zero). For matrices below 2 GiB from the first row of the (batch, head) to the last, which the launcher checks.
+struct TileCursor {
+    const uint16_t* p;
+    int left;        // bytes from p to the end of row T - 1 (below 2^31)
+    int step;        // bytes per tile of BN rows
+    __device__ TileCursor(const void* base, int64_t elem_off, int64_t st, int r0, int T, int D) {
+        const uint32_t st32 = static_cast<uint32_t>(st), first = static_cast<uint32_t>(min(r0, T));
+        const uint32_t rows = static_cast<uint32_t>(T) - first;
+        p = static_cast<const uint16_t*>(base) + elem_off + static_cast<uint64_t>(first) * st32;
+        left = rows ? static_cast<int>(((rows - 1) * st32 + D) * 2u) : 0;
+        step = static_cast<int>(static_cast<uint32_t>(BN) * st32 * 2u);
+    }
+    __device__ __amdgpu_buffer_rsrc_t rsrc() const {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p), 0, left, 0x00020000);
+    }
+    __device__ void next() {
+        p = reinterpret_cast<const uint16_t*>(reinterpret_cast<const char*>(p) + step);
+        left = max(left - step, 0);  // signed on purpose: the unsigned form becomes a saturating subtraction, a vector instruction
+    }
+};
+
+// WIN = false: no band (plain causal or full attention). Key tiles are then walked in order from 0, so the tile
+// positions are cursors that advance, and which tiles a wavefront skips or masks is decided by comparing the tile
+// index with two numbers formed once per pass -- a lone scalar instruction costs a wavefront as much issue time as a
+// vector one, and the general form of these tests was 70 scalar instructions per tile.
+template <int D, int NQ, int OCC, int NW, bool WIN>
 __global__ __launch_bounds__(64 * NW, OCC) void mfma_fwd(AttnArgs a) {
     using C = FwdCfg<D, NW>;
     constexpr int BM = 32 * NW * NQ;
@@ -144,15 +171,35 @@ __global__ __launch_bounds__(64 * NW, OCC) void mfma_fwd(AttnArgs a) {
         koff[i] = static_cast<int>((c / C::NCH) * a.k_st + (c % C::NCH) * 8) * 2;
         voff[i] = static_cast<int>((c / C::NCH) * a.v_st + (c % C::NCH) * 8) * 2;
     }
+    TileCursor kc(a.k, kb, a.k_st, t * BN, a.T, D), vc(a.v, vb, a.v_st, t * BN, a.T, D);
+    auto load_next = [&](int tn) {
+        if (WIN) {
+            load_kv_regs<D, NW>(a, kb, vb, tn * BN, koff, voff, kr, vr);
+        } else {
+            kc.next();
+            vc.next();
+            const __amdgpu_buffer_rsrc_t krs = kc.rsrc(), vrs = vc.rsrc();
+#pragma unroll
+            for (int i = 0; i < C::CPT; ++i) {
+                kr[i] = tile_load16(krs, koff[i]);
+                vr[i] = tile_load16(vrs, voff[i]);
+            }
+        }
+    };
     load_kv_regs<D, NW>(a, kb, vb, t * BN, koff, voff, kr, vr);
     store_kv_lds<D, NW>(Kbuf[0], Vbuf[0], kr, vr);
     __syncthreads();
     int cur = 0;
+    // no band, one 32-query block per wavefront: tiles [0, t_last] are visible to this wavefront's block, tiles
+    // [0, t_full) need no mask (wholly inside the sequence and, when causal, wholly at or before its first query)
+    const int qlo_w = q0 + w * NQ * 32;
+    const int t_last = qlo_w >= a.T ? -1 : (a.causal ? min(hi, (qlo_w + 32 * NQ - 1) / BN) : hi);
+    const int t_full = min(a.T / BN, a.causal ? (qlo_w + 1) / BN : 0x7fffffff);
 
     while (t <= hi) {
         const int n0 = t * BN;
         const int tn = (t + 1 == ns) ? lo : t + 1;
-        if (tn <= hi) load_kv_regs<D, NW>(a, kb, vb, tn * BN, koff, voff, kr, vr);  // in flight during the math
+        if (tn <= hi) load_next(tn);  // in flight during the math
         const uint16_t* Ks = Kbuf[cur];
         const uint16_t* Vs = Vbuf[cur];
 
@@ -160,9 +207,13 @@ __global__ __launch_bounds__(64 * NW, OCC) void mfma_fwd(AttnArgs a) {
         for (int qb = 0; qb < NQ; ++qb) {
             const int qlo = q0 + (w * NQ + qb) * 32, qhi = qlo + 31;
             // wavefront-uniform: nothing of this 32x64 block is visible
-            if (qlo >= a.T) continue;
-            if (a.causal && n0 > qhi) continue;
-            if (a.window > 0 && n0 + BN - 1 + a.window <= qlo && n0 >= a.sinks) continue;
+            if (!WIN && NQ == 1) {
+                if (t > t_last) continue;
+            } else {
+                if (qlo >= a.T) continue;
+                if (a.causal && n0 > qhi) continue;
+                if (a.window > 0 && n0 + BN - 1 + a.window <= qlo && n0 >= a.sinks) continue;
+            }
 
             // Two independent accumulator chains, issued alternately: a dependent
             // v_mfma_32x32x16 pair costs 52 cycles, an independent one 32.
@@ -180,8 +231,9 @@ __global__ __launch_bounds__(64 * NW, OCC) void mfma_fwd(AttnArgs a) {
                 s[1] = mfma32(k1f, qreg[qb][kk], s[1]);
             }
             __builtin_amdgcn_s_setprio(0);
-            const bool full = (n0 + BN - 1 < a.T) && (!a.causal || n0 + BN - 1 <= qlo) &&
-                              (a.window == 0 || n0 + a.window > qhi || n0 + BN - 1 < a.sinks);
+            const bool full = (!WIN && NQ == 1) ? t < t_full
+                                                 : (n0 + BN - 1 < a.T) && (!a.causal || n0 + BN - 1 <= qlo) &&
+                                                       (a.window == 0 || n0 + a.window > qhi || n0 + BN - 1 < a.sinks);
             if (!full) {
                 const QueryVis vis(qlo + c32, a.T, a.causal, a.window, a.sinks);
 #pragma unroll
@@ -209,16 +261,17 @@ __global__ __launch_bounds__(64 * NW, OCC) void mfma_fwd(AttnArgs a) {
                     for (int r = 0; r < 16; ++r) acc_o[qb][db][r] *= alpha;
             }
             const float mc = m[qb] * cexp;
-            float psum = 0.0f;
+            // four independent chains: an addition that waits for the one before it takes half as long again to issue
+            float psum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const float p = __builtin_amdgcn_exp2f(fmaf(s[nb][r], cexp, -mc));
                     s[nb][r] = p;
-                    psum += p;
+                    psum[r & 3] += p;
                 }
-            l[qb] += psum;  // per-lane partial; the two halves meet in the epilogue
+            l[qb] += (psum[0] + psum[1]) + (psum[2] + psum[3]);  // per-lane partial; the two halves meet in the epilogue
 
             __builtin_amdgcn_s_setprio(1);
 #pragma unroll
@@ -259,15 +312,22 @@ __global__ __launch_bounds__(64 * NW, OCC) void mfma_fwd(AttnArgs a) {
   }
 }
 
-template <int D, int NQ, int OCC, int NW>
-int launch(const AttnArgs& a, hipStream_t st) {
+template <int D, int NQ, int OCC, int NW, bool WIN>
+int launch_win(const AttnArgs& a, hipStream_t st) {
     constexpr int BM = 32 * NW * NQ;
     const int nqb = (a.T + BM - 1) / BM;
     const bool paired = pair_causal_blocks(nqb, a.Hq * a.B, a.causal, a.window);
     dim3 grid(xcd_grid(paired ? (nqb + 1) / 2 : nqb, a.Hq / a.Hkv, a.Hkv * a.B));
-    hipLaunchKernelGGL((mfma_fwd<D, NQ, OCC, NW>), grid, dim3(64 * NW), 0, st, a);
+    hipLaunchKernelGGL((mfma_fwd<D, NQ, OCC, NW, WIN>), grid, dim3(64 * NW), 0, st, a);
     PK_HIP(hipGetLastError());
     return PK_OK;
+}
+template <int D, int NQ, int OCC, int NW>
+int launch(const AttnArgs& a, hipStream_t st) {
+    // the cursor form keeps byte counts in 32 bits: K and V of one (batch, head) must span less than 2 GiB
+    const int64_t span = static_cast<int64_t>(a.T) * (a.k_st > a.v_st ? a.k_st : a.v_st) * 2;
+    if (a.window == 0 && span < (int64_t{1} << 31)) return launch_win<D, NQ, OCC, NW, false>(a, st);
+    return launch_win<D, NQ, OCC, NW, true>(a, st);
 }
 
 // 16-byte-aligned rows, and a row stride that keeps a tile's per-thread byte offsets
