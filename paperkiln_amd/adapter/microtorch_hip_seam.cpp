@@ -9,6 +9,7 @@
 #include <cstring>
 #include <stdexcept>
 #include <string>
+#include <unordered_map>
 
 #include "microtorch/device.hpp"
 #include "microtorch/ops.hpp"
@@ -27,8 +28,17 @@ struct DevState {
 namespace {
 
 Device g_where = Device::CPU;
-bool g_ops_on = false, g_step_on = false, g_window_open = false, g_ready = false;
+bool g_ops_on = false, g_step_on = false, g_window_open = false, g_ready = false, g_resident_on = false;
 unsigned long long g_stamp = 0;
+
+// Explicit residency (include/microtorch/device_cache.hpp:19-25; the reference's table is src/cuda_resident.cu:175-207):
+// device copies of host matrices the caller asked to keep, keyed by the host data pointer. Nothing enters it
+// implicitly and nothing detects a stale copy: the caller invalidates or refreshes after mutating host data.
+struct Resident {
+    void* ptr;
+    size_t rows, cols;
+};
+std::unordered_map<const float*, Resident> g_resident;
 
 void must(int rc, const char* what) {
     if (rc != PK_OK) throw std::runtime_error(std::string(what) + ": " + pk_last_error());
@@ -76,6 +86,13 @@ struct Operand {
 void stage(const Matrix& m, DevState** slot, Operand& out) {
     const size_t bytes = m.rows() * m.cols() * sizeof(float);
     const bool cache = slot && g_step_on && g_window_open;
+    if (!cache && g_resident_on) {  // an operand the caller made resident: its device copy as it stands
+        const auto it = g_resident.find(m.get_data());
+        if (it != g_resident.end() && it->second.rows == m.rows() && it->second.cols == m.cols()) {
+            out.ptr = it->second.ptr;
+            return;
+        }
+    }
     if (!cache) {
         must(pk_alloc(bytes, &out.ptr), "pk_alloc");
         out.temp = true;
@@ -181,13 +198,41 @@ Matrix gemm(const Matrix& A, DevState** devA, Trans tA, const Matrix& B, DevStat
 Matrix matmul(const Matrix& a, const Matrix& b) { return gemm(a, nullptr, Trans::N, b, nullptr, Trans::N); }
 
 // ---- include/microtorch/device_cache.hpp: residency -----------------------------------------------------
-// The pointer-keyed table of Phase B1 is not carried over: operands are cached in their Variable's own slot.
-void set_residency(bool) {}
-bool residency_enabled() { return false; }
-void make_resident(const Matrix&) {}
-void invalidate(const Matrix&) {}
-void evict_all() {}
-size_t resident_count() { return 0; }
+void set_residency(bool on) { g_resident_on = on; }
+bool residency_enabled() { return g_resident_on; }
+void make_resident(const Matrix& m) {  // upload now, or refresh in place when the shape still matches
+    bring_up();
+    const float* key = m.get_data();
+    const size_t bytes = m.rows() * m.cols() * sizeof(float);
+    auto it = g_resident.find(key);
+    if (it != g_resident.end() && (it->second.rows != m.rows() || it->second.cols != m.cols())) {
+        pk_free(it->second.ptr);
+        g_resident.erase(it);
+        it = g_resident.end();
+    }
+    if (it == g_resident.end()) {
+        void* d = nullptr;
+        must(pk_alloc(bytes ? bytes : 4, &d), "pk_alloc");
+        it = g_resident.emplace(key, Resident{d, m.rows(), m.cols()}).first;
+    }
+    const int rc = pk_memcpy_h2d(it->second.ptr, key, bytes, nullptr);
+    if (rc != PK_OK) {  // no half-made entry stays behind
+        pk_free(it->second.ptr);
+        g_resident.erase(it);
+        must(rc, "upload");
+    }
+}
+void invalidate(const Matrix& m) {
+    const auto it = g_resident.find(m.get_data());
+    if (it == g_resident.end()) return;
+    pk_free(it->second.ptr);
+    g_resident.erase(it);
+}
+void evict_all() {
+    for (auto& kv : g_resident) pk_free(kv.second.ptr);
+    g_resident.clear();
+}
+size_t resident_count() { return g_resident.size(); }
 
 void set_step_residency(bool on) { g_step_on = on; }
 bool step_residency_enabled() { return g_step_on; }

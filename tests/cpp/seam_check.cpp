@@ -4,7 +4,9 @@
 // device GPU through libpaperkiln_amd.so -- and compares, as tests/test_cuda_ops.cpp:263-300 and
 // tests/test_step_residency.cpp:142-172 of the reference do for its CUDA seam:
 //   1. the op-set entries (add, sub, mul, scale, axpy, fill, rmsnorm, silu) against the host formulas;
-//   2. device::gemm with all four transpose combinations;
+//   2. device::gemm with all four transpose combinations, and the explicit residency table
+//      (make_resident / invalidate / evict_all / resident_count) with the reference's mutate -> invalidate ->
+//      resident-again leg;
 //   3. ops::fused_attention / ops::swa_attention (host loops, [T,T] weights kept) against the O + logsumexp
 //      nodes fused_attention_hip / swa_attention_hip: output and dQ, dK, dV within 1e-5;
 //   4. a whole nn::Llama forward + cross-entropy + backward, plain and with checkpointed blocks, with the
@@ -143,6 +145,52 @@ void leg_gemm() {
     }
 }
 
+// Explicit residency, the legs of tests/test_resident_parity.cpp:65-104 of the reference: both operands resident,
+// one resident and one uploaded per call, and the contract leg -- mutate host data, invalidate, make resident again,
+// and the product must be that of the mutated operand. One leg more than the reference has: a resident copy that
+// was NOT refreshed after a host mutation must still give the OLD product, which shows that the table is really
+// what the product reads (stubs that upload on every call would pass every other leg).
+void leg_residency() {
+    std::printf("-- explicit residency: make_resident / invalidate / evict_all / resident_count --\n");
+    const size_t M = 37, K = 53, N = 41;
+    Matrix A = filled(M, K, 31), B = filled(K, N, 32);
+    const Matrix c_ref = device::matmul(A, B);  // host
+    device::set(device::Device::CUDA);
+    device::set_residency(true);
+    check(device::residency_enabled(), "residency_enabled after set_residency(true)", 0.0);
+    device::make_resident(A);
+    device::make_resident(B);
+    check(device::resident_count() == 2, "resident_count after 2 uploads", static_cast<double>(device::resident_count()));
+    const Matrix c_b1 = device::matmul(A, B);
+    check(max_abs_diff(c_ref, c_b1) <= 1e-4, "both operands resident vs host", max_abs_diff(c_ref, c_b1));
+    device::make_resident(A);  // same pointer, same shape: refreshed in place, no second entry
+    check(device::resident_count() == 2, "make_resident twice keeps one entry", static_cast<double>(device::resident_count()));
+    device::invalidate(B);
+    check(device::resident_count() == 1, "resident_count after invalidate", static_cast<double>(device::resident_count()));
+    const Matrix c_mixed = device::matmul(A, B);
+    check(max_abs_diff(c_ref, c_mixed) <= 1e-4, "A resident, B uploaded per call vs host", max_abs_diff(c_ref, c_mixed));
+    // host mutation without a refresh: the device copy is the old one, by contract
+    A.get_data()[0] += 0.5f;
+    A.get_data()[M * K - 1] -= 0.25f;
+    const Matrix c_stale = device::matmul(A, B);
+    check(max_abs_diff(c_ref, c_stale) <= 1e-4, "stale resident copy gives the old product", max_abs_diff(c_ref, c_stale));
+    // the contract leg
+    device::invalidate(A);
+    device::make_resident(A);
+    device::make_resident(B);
+    device::set(device::Device::CPU);
+    const Matrix c_ref2 = device::matmul(A, B);
+    device::set(device::Device::CUDA);
+    const Matrix c_after = device::matmul(A, B);
+    check(max_abs_diff(c_ref2, c_after) <= 1e-4, "mutate -> invalidate -> resident again matches the new host product",
+          max_abs_diff(c_ref2, c_after));
+    check(max_abs_diff(c_ref, c_ref2) > 1e-2, "(the mutation does change the product)", max_abs_diff(c_ref, c_ref2));
+    device::evict_all();
+    check(device::resident_count() == 0, "evict_all empties the table", static_cast<double>(device::resident_count()));
+    device::set_residency(false);
+    device::set(device::Device::CPU);
+}
+
 struct HeadRun {
     Matrix y, dq, dk, dv;
 };
@@ -248,6 +296,7 @@ int main() {
         device::set(device::Device::CPU);
         leg_op_set();
         leg_gemm();
+        leg_residency();
         leg_attention();
         leg_llama();
     } catch (const std::exception& e) {
