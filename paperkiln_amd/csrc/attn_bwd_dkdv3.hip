@@ -43,6 +43,7 @@
 // what must run between two phases is kept to the eight pack instructions the next phase
 // needs at once. LDS reads, LDS writes and global loads cost their issue slot and no more
 // when the matrix pipe is the bound (one per four matrix instructions measured free).
+#include <cstdlib>
 #include <type_traits>
 
 #include "mfma_common.h"
@@ -629,7 +630,12 @@ bool mfma_dkdv3_takes(const AttnArgs& a) {
     // head_dim 64 (phases of 8 matrix instructions instead of 16) or 128; with a band the 32-key kernel is ahead
     // (0.22 against 0.24 ms at head_dim 128, window 256 + 4 sinks, T 4096): the steps are
     // few, most of them masked, and the workgroup that owns the sink keys alone walks every query tile
-    return (a.dk_dim == 128 || a.dk_dim == 64) && a.window == 0 && reach < (int64_t{1} << 31);
+    // Short sequences (a workgroup meets a handful of query steps) are left to the 32-key kernel, which is ahead
+    // below T = 512 at head_dim 128 and below T = 1024 at head_dim 64 (measured, B x H = 16 .. 256) -- unless query
+    // heads share KV heads: only this kernel deals the heads of a group to several workgroups.
+    const int t_min = a.dk_dim == 128 ? 512 : 1024;
+    return (a.dk_dim == 128 || a.dk_dim == 64) && a.window == 0 && (a.T >= t_min || a.Hq > a.Hkv) &&
+           reach < (int64_t{1} << 31);
 }
 
 int launch_gqa_reduce(const AttnArgs& a, hipStream_t st) {

@@ -30,6 +30,8 @@
 // reads it (tests/test_asm_hazards.py checks both on the compiled assembly).
 #include <type_traits>
 
+#include <cstdlib>
+
 #include "mfma_common.h"
 #include "pk_internal.h"
 
@@ -108,7 +110,10 @@ __global__ __launch_bounds__(256, 1) void mfma_dq3(AttnArgs a) {
     const int nqb = (a.T + BM - 1) / BM, rep = a.Hq / a.Hkv;
     const bool paired = pair_causal_blocks(nqb, a.Hq * a.B, a.causal, a.window);
     int blk, rr, kvu;
-    if (!xcd_map(paired ? (nqb + 1) / 2 : nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
+    // unpaired causal blocks without a band: heaviest blocks of every unit first
+    if (!paired && a.causal && a.window == 0 ? !xcd_map_block_major(nqb, rep, a.Hkv * a.B, blk, rr, kvu)
+                                             : !xcd_map(paired ? (nqb + 1) / 2 : nqb, rep, a.Hkv * a.B, blk, rr, kvu))
+        return;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv, h = hk * rep + rr;
     const int npass = (paired && blk != nqb - 1 - blk) ? 2 : 1;
     const float cexp = a.scale * LOG2E;
@@ -531,7 +536,12 @@ int launch(const AttnArgs& a, bool fuse_delta, hipStream_t st) {
 bool mfma_dq3_takes(const AttnArgs& a) {
     // a lane's byte offset inside a 64-row tile of K / V is kept in 32 bits
     const int64_t reach = 2 * BN * (a.k_st > a.v_st ? a.k_st : a.v_st);
-    return (a.dk_dim == 128 || a.dk_dim == 64) && a.window == 0 && reach < (int64_t{1} << 31);
+    // One workgroup of 256 queries fills a CU, so nothing hides its prologue and epilogue (two memory round trips and a
+    // pipeline fill, the cost of about six key tiles): it is ahead of the 128-query kernel, two workgroups per CU,
+    // only where a workgroup walks many tiles. Measured over B x H = 16 .. 256, full causal: ahead from T = 2048 at
+    // head_dim 128 (4 .. 26 %) and from T = 4096 at head_dim 64 (2 .. 13 %), behind below that (3 .. 35 %).
+    const int t_min = a.dk_dim == 128 ? 2048 : 4096;
+    return (a.dk_dim == 128 || a.dk_dim == 64) && a.window == 0 && a.T >= t_min && reach < (int64_t{1} << 31);
 }
 
 int launch_mfma_dq3(const AttnArgs& a, bool fuse_delta, hipStream_t st) {

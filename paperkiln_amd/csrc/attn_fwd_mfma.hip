@@ -118,7 +118,10 @@ __global__ __launch_bounds__(64 * NW, OCC) void mfma_fwd(AttnArgs a) {
     // does not idle three quarters of the chip.
     const bool paired = pair_causal_blocks(nqb, a.Hq * a.B, a.causal, a.window);
     int blk, rr, kvu;
-    if (!xcd_map(paired ? (nqb + 1) / 2 : nqb, rep, a.Hkv * a.B, blk, rr, kvu)) return;
+    // unpaired causal blocks without a band: heaviest blocks of every unit first
+    if (!paired && a.causal && a.window == 0 ? !xcd_map_block_major(nqb, rep, a.Hkv * a.B, blk, rr, kvu)
+                                             : !xcd_map(paired ? (nqb + 1) / 2 : nqb, rep, a.Hkv * a.B, blk, rr, kvu))
+        return;
     const int hk = kvu % a.Hkv, b = kvu / a.Hkv, h = hk * rep + rr;
     const int npass = (paired && blk != nqb - 1 - blk) ? 2 : 1;
   for (int pass = 0; pass < npass; ++pass) {

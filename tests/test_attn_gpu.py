@@ -204,6 +204,11 @@ D128_CASES = [(B, T, rep, Hkv, causal, (T % 2) == 1, dk)
               for (B, T, rep, Hkv) in [(1, 63, 1, 1), (2, 64, 2, 1), (1, 65, 1, 2), (1, 127, 3, 1), (2, 129, 1, 1), (1, 191, 4, 1),
                                        (1, 257, 2, 2), (1, 449, 1, 1), (1, 700, 3, 1), (1, 1025, 2, 1)]
               for causal in (True, False)]
+# The 64-row kernels take over from the 32-row ones at a sequence length that depends on head_dim (dQ: 2048 at 128,
+# 4096 at 64; dK/dV: 512 / 1024): ragged lengths just past each threshold, so that their edge handling is met on the
+# shapes they really run at.
+D128_CASES += [(1, 2111, 1, 1, True, True, 128), (1, 2048, 2, 1, True, False, 128), (1, 4100, 1, 1, True, True, 64),
+               (1, 1030, 1, 1, False, False, 64), (2, 515, 1, 1, True, True, 128)]
 
 
 @pytest.mark.parametrize("case", D128_CASES, ids=lambda c: f"d{c[6]}_B{c[0]}_T{c[1]}_r{c[2]}_kv{c[3]}_c{int(c[4])}_g32{int(c[5])}")
