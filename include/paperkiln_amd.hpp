@@ -42,11 +42,15 @@ int status_of(const std::exception& e);
 // src/cuda_resident.cu:226-263, src/cuda_ops.cu:63-72) and supplies the memory
 // receipt the reference can only give as a node count (live_variables(),
 // include/microtorch/autograd.hpp:61-64). Blocks are recycled in stream order:
-// a freed block remembers the stream of the thread that freed it (tape_stream())
-// and is handed out again at once, but only to a request made for that same
-// stream, whose later work is ordered after the work that last used the block.
+// a block remembers the stream that used it last (the stream it was allocated
+// for, or the stream of the last C-ABI call that was handed it: dev_touch) and,
+// once freed, is handed out again at once, but only to a request made for that
+// same stream, whose later work is ordered after the work that last used the
+// block; a request for another stream may take it over only when that stream
+// has nothing queued any more.
 void* dev_alloc(size_t bytes);
 bool dev_free(void* p);       // false: not a block this allocator has handed out (nothing is done then)
+void dev_touch(const void* p, void* stream);  // a block of this allocator is about to be used on `stream` (no-op for other pointers)
 bool dev_owns(const void* p);  // a block this allocator handed out and has not been given back
 size_t dev_live_bytes();
 size_t dev_peak_bytes();

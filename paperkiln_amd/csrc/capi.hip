@@ -167,6 +167,8 @@ int pk_attn_fwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k
     AttnArgs a;
     fill_common(a, s, q, k, v, o);
     a.lse = lse;
+    const void* used[] = {q->ptr, k->ptr, v->ptr, o->ptr, lse};
+    for (const void* p : used) dev_touch(p, stream);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (s->dtype == PK_BF16 && mfma_supported(a)) return launch_mfma_fwd(a, st);
     if (s->dtype == PK_F32 && f32_mfma_supported(a)) return launch_f32_mfma_fwd(a, st);
@@ -240,6 +242,8 @@ int bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k,
     a.dq = dq->ptr; a.dq_sb = dq->stride_b; a.dq_st = dq->stride_t; a.dq_sh = dq->stride_h;
     a.dk = dk->ptr; a.dk_sb = dk->stride_b; a.dk_st = dk->stride_t; a.dk_sh = dk->stride_h;
     a.dv = dv->ptr; a.dv_sb = dv->stride_b; a.dv_st = dv->stride_t; a.dv_sh = dv->stride_h;
+    const void* used[] = {q->ptr, k->ptr, v->ptr, o->ptr, lse, d_o->ptr, dq->ptr, dk->ptr, dv->ptr, workspace};
+    for (const void* p : used) dev_touch(p, stream);
     a.delta = static_cast<float*>(workspace);
     if (tail_bytes(s)) {
         const size_t db = delta_bytes(s);

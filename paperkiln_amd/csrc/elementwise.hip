@@ -6,6 +6,7 @@
 #include <hipcub/hipcub.hpp>
 #include <rocblas/rocblas.h>
 
+#include <atomic>
 #include <cstdlib>
 #include <map>
 #include <cmath>
@@ -38,7 +39,7 @@ struct Pool {
     // GPU, which is only safe for work queued behind its last use, i.e. on that same stream
     std::multimap<std::pair<hipStream_t, size_t>, void*> free_blocks;
     std::unordered_map<void*, size_t> sizes;          // every block handed out or cached
-    std::unordered_map<void*, bool> handed_out;       // blocks a caller holds right now
+    std::unordered_map<void*, hipStream_t> handed_out;  // blocks a caller holds right now -> the stream that used them last
     size_t live = 0, peak = 0, reserved = 0;
     void release_cached() {  // give every cached block back to the driver (hipFree waits for the device)
         for (auto& kv : free_blocks) {
@@ -67,7 +68,27 @@ void* dev_alloc(size_t bytes) {
     std::lock_guard<std::mutex> lk(P.mu);
     void* p = nullptr;
     auto it = P.free_blocks.lower_bound({st, n});
-    if (it != P.free_blocks.end() && it->first.first == st && it->first.second <= n + n / 4 + 512) {  // near-fitting only
+    auto fits = [&](decltype(it) i, hipStream_t s) {  // near-fitting only
+        return i != P.free_blocks.end() && i->first.first == s && i->first.second <= n + n / 4 + 512;
+    };
+    if (!fits(it, st)) {
+        // A block cached for ANOTHER stream may be taken over once that stream has nothing queued any more (its
+        // last use of the block has then completed); otherwise blocks of a stream nobody uses again would sit in
+        // the cache until an allocation fails. Streams are visited in key order, one query each.
+        it = P.free_blocks.end();
+        for (auto j = P.free_blocks.begin(); j != P.free_blocks.end(); j = P.free_blocks.upper_bound({j->first.first, SIZE_MAX})) {
+            const hipStream_t other = j->first.first;
+            if (other == st) continue;
+            auto cand = P.free_blocks.lower_bound({other, n});
+            if (!fits(cand, other)) continue;
+            if (hipStreamQuery(other) == hipSuccess) {
+                it = cand;
+                break;
+            }
+            (void)hipGetLastError();  // still busy (or no longer a stream): leave its blocks alone
+        }
+    }
+    if (it != P.free_blocks.end()) {
         p = it->second;
         P.live += it->first.second;
         P.free_blocks.erase(it);
@@ -87,7 +108,7 @@ void* dev_alloc(size_t bytes) {
         P.reserved += n;
         P.live += n;
     }
-    P.handed_out[p] = true;
+    P.handed_out[p] = st;
     if (P.live > P.peak) P.peak = P.live;
     return p;
 }
@@ -98,11 +119,23 @@ bool dev_free(void* p) {
     std::lock_guard<std::mutex> lk(P.mu);
     auto held = P.handed_out.find(p);
     if (held == P.handed_out.end()) return false;
+    // cached for the stream that used the block last (dev_touch), not for whichever context happens to free it: a
+    // block used on stream S and freed outside any scope must not go to the next allocation of the null stream
+    const hipStream_t last = held->second;
     P.handed_out.erase(held);
     const size_t n = P.sizes.at(p);
     P.live -= n;
-    P.free_blocks.emplace(std::make_pair(tape_stream(), n), p);
+    P.free_blocks.emplace(std::make_pair(last, n), p);
     return true;
+}
+
+void dev_touch(const void* p, void* stream) {
+    if (!p) return;
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    Pool& P = pool();
+    std::lock_guard<std::mutex> lk(P.mu);
+    auto held = P.handed_out.find(const_cast<void*>(p));
+    if (held != P.handed_out.end()) held->second = st;
 }
 
 bool dev_owns(const void* p) {
@@ -1031,13 +1064,15 @@ rocblas_handle blas() {
 }  // namespace
 
 namespace {
-int g_gemm_hand_written = [] {
+// Process-wide and read by every model's thread, set by pk_set_gemm_backend from any thread: an atomic, relaxed
+// (a product sees either the old or the new choice, both of which give the same numbers up to rounding order).
+std::atomic<int> g_gemm_hand_written{[] {
     const char* v = std::getenv("PK_GEMM");
     return (v && std::string(v) == "library") ? 0 : 1;
-}();
+}()};
 }
-void set_gemm_backend(int hand_written) { g_gemm_hand_written = hand_written; }
-int gemm_backend() { return g_gemm_hand_written; }
+void set_gemm_backend(int hand_written) { g_gemm_hand_written.store(hand_written, std::memory_order_relaxed); }
+int gemm_backend() { return g_gemm_hand_written.load(std::memory_order_relaxed); }
 
 void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dtype, int64_t M, int64_t N, int64_t ldc,
           float beta, int64_t lda) {
@@ -1055,8 +1090,9 @@ void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dty
     // multiple of 256, because the library's 176 - 256-wide tiles waste more of their last column there than
     // 128 x 128 tiles do: [8192, 512] x [512, 2752] 42.9 against 55.0 us, [8192, 512] x [1376, 512]^T 23.7 against
     // 38.1 us. That class goes to the hand-written kernel, everything else to the library.
-    // g_gemm_hand_written == 2 sends everything the hand-written kernel takes to it.
-    const bool mine = g_gemm_hand_written == 2 || (g_gemm_hand_written == 1 && !tA && Ka <= 1024 && N % 256 != 0 && N >= 1024);
+    // backend 2 sends everything the hand-written kernel takes to it.
+    const int backend = gemm_backend();
+    const bool mine = backend == 2 || (backend == 1 && !tA && Ka <= 1024 && N % 256 != 0 && N >= 1024);
     if (A.dtype == PK_BF16 && mine &&
         gemm_mfma_bf16(A.ptr(), tA, lda, B.ptr(), tB, B.cols, C, c_dtype, M, N, Ka, ldc, beta, tape_stream()))
         return;
@@ -1113,7 +1149,7 @@ void gemm_tn_split(const Tensor& A, const Tensor& B, float* const* dst, int nspl
     if (B.rows != K) throw std::runtime_error("gemm: inner dimensions disagree");
     if (nsplit < 1 || nsplit > 4 || W % nsplit != 0) throw std::runtime_error("gemm_tn_split: bad column split");
     if (A.dtype != B.dtype) throw std::runtime_error("gemm: operand dtypes differ");
-    if (A.dtype == PK_BF16 && g_gemm_hand_written == 2) {  // one product [M, W] in fp32, then the column blocks go to their tensors
+    if (A.dtype == PK_BF16 && gemm_backend() == 2) {  // one product [M, W] in fp32, then the column blocks go to their tensors
         Buffer whole(sizeof(float) * static_cast<size_t>(M) * W);
         if (gemm_mfma_bf16(A.ptr(), true, M, B.ptr(), false, W, whole.p, PK_F32, M, W, K, W, 0.0f, tape_stream())) {
             SplitDst d{};

@@ -35,7 +35,13 @@ int op_guard(void* stream, F&& f) {
     }
 }
 
-Tensor vec(const void* p, int64_t n, int dt) { return Tensor::borrow(p, 1, n, dt); }
+// a caller's matrix as a borrowed tensor; if it is a block of the library's allocator, the allocator learns which
+// stream uses it now
+Tensor mat(const void* p, int64_t r, int64_t c, int dt) {
+    dev_touch(p, tape_stream());
+    return Tensor::borrow(p, r, c, dt);
+}
+Tensor vec(const void* p, int64_t n, int dt) { return mat(p, 1, n, dt); }
 
 }  // namespace
 }  // namespace pk
@@ -95,8 +101,8 @@ int pk_op_rmsnorm_fwd(const void* x, const float* w, float eps, void* y, float* 
                       int dtype, void* stream) {
     return op_guard(stream, [&] {
         if (!rms_inv) throw std::runtime_error("rmsnorm: rms_inv is required");
-        k_rmsnorm_fwd(Tensor::borrow(x, rows, cols, dtype), Tensor::borrow(w, 1, cols, PK_F32), eps,
-                      Tensor::borrow(y, rows, cols, dtype), rms_inv);
+        k_rmsnorm_fwd(mat(x, rows, cols, dtype), mat(w, 1, cols, PK_F32), eps,
+                      mat(y, rows, cols, dtype), rms_inv);
     });
 }
 int pk_op_rmsnorm_bwd(const void* dy, const void* x, const float* rms_inv, const float* w, float* dw, void* dx,
@@ -105,12 +111,12 @@ int pk_op_rmsnorm_bwd(const void* dy, const void* x, const float* rms_inv, const
         if (!rms_inv) throw std::runtime_error("rmsnorm: rms_inv is required");
         Tensor tdw, tdx;
         if (dw) {
-            tdw = Tensor::borrow(dw, 1, cols, PK_F32);
+            tdw = mat(dw, 1, cols, PK_F32);
             k_fill(tdw, 0.0f);  // the launcher accumulates, as the tape's grad does; this entry point overwrites
         }
-        if (dx) tdx = Tensor::borrow(dx, rows, cols, dtype);
-        k_rmsnorm_bwd(Tensor::borrow(dy, rows, cols, dtype), Tensor::borrow(x, rows, cols, dtype), rms_inv,
-                      Tensor::borrow(w, 1, cols, PK_F32), dw ? &tdw : nullptr, dx ? &tdx : nullptr);
+        if (dx) tdx = mat(dx, rows, cols, dtype);
+        k_rmsnorm_bwd(mat(dy, rows, cols, dtype), mat(x, rows, cols, dtype), rms_inv,
+                      mat(w, 1, cols, PK_F32), dw ? &tdw : nullptr, dx ? &tdx : nullptr);
     });
 }
 int pk_op_rope(const void* qkv, const int* pos, float theta, int64_t rows, int64_t d, int head_dim, int all_heads,
@@ -119,29 +125,29 @@ int pk_op_rope(const void* qkv, const int* pos, float theta, int64_t rows, int64
         if (!pos) throw std::runtime_error("apply_rope: positions are required");
         if (d <= 0 || head_dim <= 0) throw std::runtime_error("apply_rope: head_dim must be even and <= d");
         const int rot = all_heads ? static_cast<int>(d / head_dim) : 1;
-        k_rope(Tensor::borrow(qkv, rows, 3 * d, dtype), pos, theta, static_cast<int>(d), head_dim, rot, inverse != 0,
-               Tensor::borrow(y, rows, 3 * d, dtype));
+        k_rope(mat(qkv, rows, 3 * d, dtype), pos, theta, static_cast<int>(d), head_dim, rot, inverse != 0,
+               mat(y, rows, 3 * d, dtype));
     });
 }
 int pk_op_embedding_fwd(const float* table, const int* ids, void* y, int64_t n, int64_t vocab, int64_t d, int dtype,
                         void* stream) {
     return op_guard(stream, [&] {
         if (!ids) throw std::runtime_error("embedding: ids are required");
-        k_embedding_fwd(Tensor::borrow(table, vocab, d, PK_F32), ids, Tensor::borrow(y, n, d, dtype));
+        k_embedding_fwd(mat(table, vocab, d, PK_F32), ids, mat(y, n, d, dtype));
     });
 }
 int pk_op_embedding_bwd(const void* dy, const int* ids, float* dtable, int64_t n, int64_t vocab, int64_t d, int dtype,
                         void* stream) {
     return op_guard(stream, [&] {
         if (!ids) throw std::runtime_error("embedding: ids are required");
-        k_embedding_bwd(Tensor::borrow(dy, n, d, dtype), ids, Tensor::borrow(dtable, vocab, d, PK_F32));
+        k_embedding_bwd(mat(dy, n, d, dtype), ids, mat(dtable, vocab, d, PK_F32));
     });
 }
 int pk_op_cross_entropy(void* logits, const int* targets, int64_t rows, int64_t vocab, float upstream, float* nll_rows,
                         float* loss, int dtype, void* stream) {
     return op_guard(stream, [&] {
         if (!targets || !nll_rows) throw std::runtime_error("cross_entropy: one target per row");
-        k_ce_rows(Tensor::borrow(logits, rows, vocab, dtype), targets, upstream / static_cast<float>(rows), nll_rows);
+        k_ce_rows(mat(logits, rows, vocab, dtype), targets, upstream / static_cast<float>(rows), nll_rows);
         if (loss) *loss = static_cast<float>(k_sum_f32_to_host(nll_rows, rows) / static_cast<double>(rows));
     });
 }
@@ -169,8 +175,8 @@ int pk_op_gemm(const void* a, int trans_a, const void* b, int trans_b, void* c, 
                int dtype, int c_dtype, int accumulate, void* stream) {
     return op_guard(stream, [&] {
         if (!c) throw std::runtime_error("null device pointer");
-        const Tensor A = trans_a ? Tensor::borrow(a, k, m, dtype) : Tensor::borrow(a, m, k, dtype);
-        const Tensor B = trans_b ? Tensor::borrow(b, n, k, dtype) : Tensor::borrow(b, k, n, dtype);
+        const Tensor A = trans_a ? mat(a, k, m, dtype) : mat(a, m, k, dtype);
+        const Tensor B = trans_b ? mat(b, n, k, dtype) : mat(b, k, n, dtype);
         gemm(A, trans_a != 0, B, trans_b != 0, c, c_dtype, m, n, n, accumulate ? 1.0f : 0.0f);
     });
 }

@@ -21,6 +21,10 @@ int hip_fail(hipError_t e, const char* what);
         if (_e != hipSuccess) return ::pk::hip_fail(_e, #expr); \
     } while (0)
 
+// elementwise.hip: tells the caching allocator that one of its blocks is about to be used on `stream`, so that the
+// block, once freed, is only recycled behind that use (no-op for pointers that are not its blocks)
+void dev_touch(const void* p, void* stream);
+
 // Kernel-side view of one attention problem. Strides are in elements.
 struct AttnArgs {
     const void* q;

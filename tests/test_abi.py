@@ -43,7 +43,8 @@ def test_argument_errors_do_not_need_a_gpu():
 
 
 def test_backward_workspace_follows_the_mask():
-    """pk_attn_bwd_workspace_bytes: delta [B, Hq, T] fp32 for every mask; a band mask with 1..32 sink keys on a
+    """pk_attn_bwd_workspace_bytes: delta [B, Hq, T] fp32 for every mask; without a band, query heads that share KV
+    heads on a grid that would leave CUs idle add the per-split partial dK / dV; a band mask with 1..32 sink keys on a
     sequence longer than key block 0's band adds the partial sink rows of a split sink tail
     ((chunks of 512 queries + 1) x {dK, dV} x 32 rows x head_dim fp32 per (batch, KV head), 256-byte aligned)."""
     L = _lib.lib()
@@ -54,7 +55,11 @@ def test_backward_workspace_follows_the_mask():
         sh = _lib.AttnShape(B, t, Hq, Hkv, dk, 1, window, sinks, 0.5, _lib.PK_BF16, _lib.PK_BF16)
         return L.pk_attn_bwd_workspace_bytes(ctypes.byref(sh))
 
-    assert ws(0, 0) == delta
+    # no band, 2 query heads per KV head, 16 paired key blocks x 8 (batch, KV head) units = 128 dK/dV workgroups for
+    # 256 CUs: the heads of a group are dealt to 2 workgroups, whose fp32 partial dK and dV follow delta
+    assert ws(0, 0) == delta + 4 * 2 * (B * Hkv) * 2 * T * dk
+    mha = _lib.AttnShape(B, T, Hq, Hq, dk, 1, 0, 0, 0.5, _lib.PK_BF16, _lib.PK_BF16)
+    assert L.pk_attn_bwd_workspace_bytes(ctypes.byref(mha)) == delta   # one query head per KV head: nothing to deal
     assert ws(256, 0) == delta          # no sink keys: nothing to split
     assert ws(256, 33) == delta         # more sink keys than one wavefront owns: not split
     q0 = ((127 + 256 - 1) // 64 + 1) * 64   # first 64-query tile wholly past key block 0's band
@@ -70,7 +75,7 @@ def test_a_window_that_covers_the_sequence_is_no_band():
     (tests/test_swa.cpp:47-57), so INT32_MAX is a legal "no band": the shape is brought into range on the host,
     before any index arithmetic, and sizes its workspace as the causal mask does."""
     L = _lib.lib()
-    B, T, Hq, Hkv, dk = 2, 4096, 8, 4, 128
+    B, T, Hq, Hkv, dk = 2, 4096, 8, 8, 128
 
     def ws(window, sinks):
         sh = _lib.AttnShape(B, T, Hq, Hkv, dk, 1, window, sinks, 0.5, _lib.PK_BF16, _lib.PK_BF16)

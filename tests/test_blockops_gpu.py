@@ -230,6 +230,42 @@ def test_error_behaviour(bo):
         bo.add(x, dev(synth.randn(433, (4, 9), 1.0)))
 
 
+def test_allocator_recycles_a_block_behind_the_stream_that_used_it_last(bo):
+    """A block from pk_alloc that a C-ABI call used on stream S is cached, once freed, for S and not for the stream of
+    whoever frees it: an allocation for the null stream made while S still has work queued must not get that block
+    back; once S is idle the block may be taken over. (S is kept busy with a long chain of fills on a large
+    buffer; the check is skipped if the stream has drained by the time the allocation is made.)"""
+    import ctypes as C
+    from paperkiln_amd import _lib
+    L = _lib.lib()
+    n = 64 << 20
+    side = torch.cuda.Stream()
+    big = torch.empty(1 << 28, dtype=torch.float32, device="cuda")   # 1 GiB: each fill takes a fraction of a millisecond
+    p = C.c_void_p()
+    _lib.check(L.pk_alloc(n, C.byref(p)))
+    first = p.value
+    torch.cuda.synchronize()
+    S = C.c_void_p(side.cuda_stream)
+    with torch.cuda.stream(side):
+        for _ in range(40):
+            big.fill_(1.0)
+    _lib.check(L.pk_op_fill(p, 2.0, n // 4, _lib.PK_F32, S))       # queued on S behind the fills
+    _lib.check(L.pk_free(p))                                         # freed by a thread whose own stream is the null stream
+    q = C.c_void_p()
+    _lib.check(L.pk_alloc(n, C.byref(q)))                            # for the null stream
+    still_busy = not side.query()
+    if still_busy:
+        assert q.value != first, "a block whose last user is still running was handed to another stream"
+    torch.cuda.synchronize()
+    _lib.check(L.pk_free(q))
+    r = C.c_void_p()
+    _lib.check(L.pk_alloc(n, C.byref(r)))                            # S is idle now: either cached block may come back
+    assert r.value in (first, q.value)
+    _lib.check(L.pk_free(r))
+    if not still_busy:
+        pytest.skip("the side stream drained before the allocation; only the take-over path was exercised")
+
+
 GEMM_SHAPES = [(128, 128, 64), (560, 136, 200), (8, 8, 8), (2056, 520, 1376), (512, 1536, 4096), (264, 40, 8192),
                (1000, 2048, 512), (300, 264, 72)]
 
