@@ -20,6 +20,7 @@
 // Step = 64 queries of one query head. Q / dO tiles sit in a three-deep LDS
 // ring (role 0 reads step s, role 1 step s-1, step s+1 is being stored).
 #include <cstdlib>
+#include <type_traits>
 
 #include "mfma_common.h"
 #include "pk_internal.h"
@@ -115,12 +116,6 @@ __global__ __launch_bounds__(4 * BNK, 2) void mfma_dkdv2(AttnArgs a) {
                 kv[kk] = *reinterpret_cast<const bf16x8*>(&z);
             }
         }
-        f32x16 acc[DB];  // dV^T (role 0) or dK^T (role 1)
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[db][r] = 0.0f;
-
         // Query tiles that can see keys [k0, k0+127] (paperkiln src/ops.cpp:960-965 inverted).
         const int khi = min(k0 + BNK, a.T) - 1;
         int qt_lo = a.causal ? k0 / BMQ : 0;
@@ -137,24 +132,32 @@ __global__ __launch_bounds__(4 * BNK, 2) void mfma_dkdv2(AttnArgs a) {
 
         u32x4 qr[CPT], gr[CPT];
         float lse_r = 0.0f, dl_r = 0.0f;
-        auto fetch = [&](int step) {  // global -> registers, rows past the end clamped
-            const int h = hk * rep + step / nqt, q0 = (qt_lo + step % nqt) * BMQ;
+        // Steps are fetched in order, so the (head, query tile) of the next fetch is counted up, not divided out of
+        // the step number, and a thread's position inside a tile (row tid / NCH + RPI i, chunk tid % NCH) is formed once.
+        // (Tile positions as scalar bases plus per-thread 32-bit offsets, as the 64-key kernel keeps them, take a
+        // third of the vector instructions out of the staging and measured no faster here, slower at head_dim 64.)
+        int f_h = hk * rep, f_qt = 0;
+        const int frow = static_cast<int>(threadIdx.x) / NCH, fch = static_cast<int>(threadIdx.x) % NCH;
+        constexpr int RPI = NTHR / NCH;  // tile rows between a thread's consecutive chunks
+        auto fetch = [&]() {  // global -> registers, rows past the end clamped
+            const int q0 = (qt_lo + f_qt) * BMQ;
+            const uint16_t* qb = static_cast<const uint16_t*>(a.q) + b * a.q_sb + f_h * a.q_sh + fch * 8;
+            const uint16_t* gb = static_cast<const uint16_t*>(a.d_o) + b * a.do_sb + f_h * a.do_sh + fch * 8;
 #pragma unroll
             for (int i = 0; i < CPT; ++i) {
-                const int c = threadIdx.x + NTHR * i;
-                const int row = c / NCH, ch = c % NCH;
-                const int t = min(q0 + row, a.T - 1);
-                qr[i] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.q) + b * a.q_sb + h * a.q_sh +
-                                                        t * a.q_st + ch * 8);
-                gr[i] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(a.d_o) + b * a.do_sb +
-                                                        h * a.do_sh + t * a.do_st + ch * 8);
+                const int t = min(q0 + frow + RPI * i, a.T - 1);
+                qr[i] = *reinterpret_cast<const u32x4*>(qb + t * a.q_st);
+                gr[i] = *reinterpret_cast<const u32x4*>(gb + t * a.do_st);
             }
             if (threadIdx.x < BMQ) {
                 const int t = min(q0 + static_cast<int>(threadIdx.x), a.T - 1);
-                const int64_t lrow = (static_cast<int64_t>(b) * a.Hq + h) * a.T + t;
+                const int64_t lrow = (static_cast<int64_t>(b) * a.Hq + f_h) * a.T + t;
                 lse_r = a.lse[lrow];  // scaled when it is stored: arithmetic on it here would wait for every load just issued
                 dl_r = a.delta[lrow];
             }
+            const bool wrap = f_qt + 1 == nqt;
+            f_qt = wrap ? 0 : f_qt + 1;
+            f_h += wrap;
         };
         auto commit = [&](int slot) {  // registers -> LDS ring slot
             // The store addresses are rebuilt from the thread index at every call (the
@@ -174,9 +177,9 @@ __global__ __launch_bounds__(4 * BNK, 2) void mfma_dkdv2(AttnArgs a) {
                 dl_s[slot][tid] = dl_r;
             }
         };
-        // wavefront-uniform: is anything of (query block qb of step `step`) x (this key block) visible?
-        auto block_live = [&](int step, int qb, int& qlo) {
-            qlo = (qt_lo + step % nqt) * BMQ + qb * 32;
+        // wavefront-uniform: is anything of (query block qb of the step at query tile `qt`) x (this key block) visible?
+        auto block_live = [&](int qt, int qb, int& qlo) {
+            qlo = (qt_lo + qt) * BMQ + qb * 32;
             const int qhi = qlo + 31;
             if (qlo >= a.T || kw0 >= a.T) return false;
             if (a.causal && kw0 > qhi) return false;
@@ -185,9 +188,9 @@ __global__ __launch_bounds__(4 * BNK, 2) void mfma_dkdv2(AttnArgs a) {
         };
 
         if (steps > 0) {
-            fetch(0);
+            fetch();
             commit(0);
-            if (steps > 1) fetch(1);
+            if (steps > 1) fetch();
         }
         // Every load issued so far -- the resident K / V rows above all -- has landed before the step loop is
         // entered. Without this the wait-count bookkeeping carries "kv may still be in flight" around the loop
@@ -205,25 +208,36 @@ __global__ __launch_bounds__(4 * BNK, 2) void mfma_dkdv2(AttnArgs a) {
             const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             return *reinterpret_cast<const bf16x8*>(&v);
         };
-        // iteration s: role 0 works on step s, role 1 on step s-1
+        // The step loop and the stores are instantiated once per role and entered through one branch on the role: with
+        // the role tested inside the loop the two sides of the branch each get their own copy of the accumulators,
+        // which are moved back at the join in every step (64 register moves a step, found in the compiled loop).
+        auto run_role = [&](auto role_tag) {
+        constexpr int rl = decltype(role_tag)::value;
+        f32x16 acc[DB];  // dV^T (role 0) or dK^T (role 1)
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[db][r] = 0.0f;
+        // iteration s: role 0 works on step s, role 1 on step s-1; the query tile of either is counted, not divided out
+        int c_qt = 0, slot = 0;  // query tile and ring slot of the step this role works on
         for (int s = 0; s <= steps; ++s) {
             if (s + 1 < steps) {
                 commit((s + 1) % 3);  // slot last read (by role 1) before the previous barrier
-                if (s + 2 < steps) fetch(s + 2);
+                if (s + 2 < steps) fetch();
             }
-            if (role == 0) {
+            if (rl == 0) {
                 if (s < steps) {
                     // One register each for the row-read and the transposing-read address of
                         // this step; every fragment is then an immediate offset away. Left to
                         // itself the compiler keeps a dozen pre-offset copies and spills.
-                    int xrow = (s % 3) * (BMQ * S) + row_lane;                  // Q rows
-                    int ytr = (3 + s % 3) * (BMQ * S) + tr_lane;                // dO transposed
+                    int xrow = slot * (BMQ * S) + row_lane;                     // Q rows
+                    int ytr = (3 + slot) * (BMQ * S) + tr_lane;                 // dO transposed
                     asm volatile("" : "+v"(xrow), "+v"(ytr));
                     const uint16_t* flat = &tiles[0][0][0];
 #pragma unroll
                     for (int qb = 0; qb < NQB; ++qb) {
                         int qlo;
-                        if (!block_live(s, qb, qlo)) continue;
+                        if (!block_live(c_qt, qb, qlo)) continue;
                         // One accumulator chain: the other role's wavefront on this SIMD issues
                         // into the gaps a dependent MFMA pair leaves, and the registers of a
                         // second chain would push the kernel into scratch.
@@ -239,7 +253,7 @@ __global__ __launch_bounds__(4 * BNK, 2) void mfma_dkdv2(AttnArgs a) {
                         // lane = key kj; element r = query qlo + (r/4)*8 + 4g + r%4
 #pragma unroll
                         for (int qd = 0; qd < 4; ++qd) {
-                            const f32x4 nl = *reinterpret_cast<const f32x4*>(&nlse_s[s % 3][qb * 32 + qd * 8 + g * 4]);
+                            const f32x4 nl = *reinterpret_cast<const f32x4*>(&nlse_s[slot][qb * 32 + qd * 8 + g * 4]);
 #pragma unroll
                             for (int e = 0; e < 4; ++e)
                                 sc[qd * 4 + e] = __builtin_amdgcn_exp2f(fmaf(sc[qd * 4 + e], cexp, nl[e]));
@@ -272,18 +286,20 @@ __global__ __launch_bounds__(4 * BNK, 2) void mfma_dkdv2(AttnArgs a) {
                         for (int db = 0; db < DB; ++db)
                             acc[db] = mfma32(tr_operand(flat + ytr, qb * 32 + 16, db), p1, acc[db]);
                     }
+                    c_qt = c_qt + 1 == nqt ? 0 : c_qt + 1;
+                    slot = slot == 2 ? 0 : slot + 1;
                 }
             } else {
                 if (s >= 1) {
                     const int sp = s - 1;
-                    int xrow = (3 + sp % 3) * (BMQ * S) + row_lane;             // dO rows
-                    int ytr = (sp % 3) * (BMQ * S) + tr_lane;                   // Q transposed
+                    int xrow = (3 + slot) * (BMQ * S) + row_lane;               // dO rows
+                    int ytr = slot * (BMQ * S) + tr_lane;                       // Q transposed
                     asm volatile("" : "+v"(xrow), "+v"(ytr));
                     const uint16_t* flat = &tiles[0][0][0];
 #pragma unroll
                     for (int qb = 0; qb < NQB; ++qb) {
                         int qlo;
-                        if (!block_live(sp, qb, qlo)) continue;
+                        if (!block_live(c_qt, qb, qlo)) continue;
                         f32x16 dp;
 #pragma unroll
                         for (int r = 0; r < 16; ++r) dp[r] = 0.0f;
@@ -298,7 +314,7 @@ __global__ __launch_bounds__(4 * BNK, 2) void mfma_dkdv2(AttnArgs a) {
                         // dS = P .* (dP - delta); P arrives as fp16 pairs of elements (2i, 2i+1)
 #pragma unroll
                         for (int qd = 0; qd < 4; ++qd) {
-                            const f32x4 dl = *reinterpret_cast<const f32x4*>(&dl_s[sp % 3][qb * 32 + qd * 8 + g * 4]);
+                            const f32x4 dl = *reinterpret_cast<const f32x4*>(&dl_s[slot][qb * 32 + qd * 8 + g * 4]);
                             dp[qd * 4 + 0] = static_cast<float>(ph[2 * qd][0]) * (dp[qd * 4 + 0] - dl[0]);
                             dp[qd * 4 + 1] = static_cast<float>(ph[2 * qd][1]) * (dp[qd * 4 + 1] - dl[1]);
                             dp[qd * 4 + 2] = static_cast<float>(ph[2 * qd + 1][0]) * (dp[qd * 4 + 2] - dl[2]);
@@ -313,6 +329,8 @@ __global__ __launch_bounds__(4 * BNK, 2) void mfma_dkdv2(AttnArgs a) {
                         for (int db = 0; db < DB; ++db)
                             acc[db] = mfma32(tr_operand(flat + ytr, qb * 32 + 16, db), d1, acc[db]);
                     }
+                    c_qt = c_qt + 1 == nqt ? 0 : c_qt + 1;
+                    slot = slot == 2 ? 0 : slot + 1;
                 }
             }
             __syncthreads();
@@ -322,8 +340,8 @@ __global__ __launch_bounds__(4 * BNK, 2) void mfma_dkdv2(AttnArgs a) {
         // (a chunk writes nothing else; the band part of block 0 writes its other rows as usual).
         const bool piece = TAIL && kblk == 0;
         if (piece && kbw == 0 && kj < a.sinks) {
-            float* rows = sink_tail_rows(a.tail, kvu, tl.nch, chunk >= 0 ? chunk : tl.nch, role == 0 ? 1 : 0, D) + kj * D;
-            const float sc = role == 0 ? 1.0f : a.scale;
+            float* rows = sink_tail_rows(a.tail, kvu, tl.nch, chunk >= 0 ? chunk : tl.nch, rl == 0 ? 1 : 0, D) + kj * D;
+            const float sc = rl == 0 ? 1.0f : a.scale;
 #pragma unroll
             for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -332,10 +350,10 @@ __global__ __launch_bounds__(4 * BNK, 2) void mfma_dkdv2(AttnArgs a) {
                                   acc[db][qd * 4 + 2] * sc, acc[db][qd * 4 + 3] * sc);
         }
         if (kj < a.T && chunk < 0 && !(piece && kj < a.sinks)) {
-            void* dst = role == 0 ? a.dv : a.dk;
-            const int64_t ob = role == 0 ? b * a.dv_sb + hk * a.dv_sh + kj * a.dv_st
+            void* dst = rl == 0 ? a.dv : a.dk;
+            const int64_t ob = rl == 0 ? b * a.dv_sb + hk * a.dv_sh + kj * a.dv_st
                                          : b * a.dk_sb + hk * a.dk_sh + kj * a.dk_st;
-            const float sc = role == 0 ? 1.0f : a.scale;
+            const float sc = rl == 0 ? 1.0f : a.scale;
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 if (!GF32) {
@@ -348,6 +366,11 @@ __global__ __launch_bounds__(4 * BNK, 2) void mfma_dkdv2(AttnArgs a) {
                                   acc[db][qd * 4 + 2] * sc, acc[db][qd * 4 + 3] * sc);
             }
         }
+        };  // run_role
+        if (role == 0)
+            run_role(std::integral_constant<int, 0>{});
+        else
+            run_role(std::integral_constant<int, 1>{});
         __syncthreads();  // the next pass refills the ring
     }
 }
