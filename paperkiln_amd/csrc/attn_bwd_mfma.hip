@@ -203,10 +203,13 @@ __global__ __launch_bounds__(64 * NW, 2) void mfma_dq(AttnArgs a) {
         const bool skip = qlo >= a.T || (a.causal && n0 > qhi) ||
                           (a.window > 0 && n0 + BN - 1 + a.window <= qlo && n0 >= a.sinks);
         if (!skip) {
-            const bool full = (n0 + BN - 1 < a.T) && (!a.causal || n0 + BN - 1 <= qlo) &&
-                              (a.window == 0 || n0 + a.window > qhi || n0 + BN - 1 < a.sinks);
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) {
+                // a 32-key half no query of this wavefront can see (past the diagonal, or before the band and without
+                // a sink key) costs nothing; which of the mask's tests the half can fail decides its masking loop
+                const int k0 = n0 + nb * 32, k1 = k0 + 31;
+                if ((a.causal && k0 > qhi) || (a.window > 0 && k1 + a.window <= qlo && k0 >= a.sinks)) continue;
+                const MaskKind kind = mask_kind(k0, k1, qlo, qhi, a.T, a.causal, a.window, a.sinks);
                 f32x16 s, dp;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.0f;
@@ -223,11 +226,8 @@ __global__ __launch_bounds__(64 * NW, 2) void mfma_dq(AttnArgs a) {
                 // lane = query qi; element r = key n0 + nb*32 + (r/4)*8 + 4g + r%4
 #pragma unroll
                 for (int r = 0; r < 16; ++r) dp[r] = __builtin_amdgcn_exp2f(fmaf(s[r], cexp, nlse)) * (dp[r] - dl);
-                if (!full) {  // off the common path: interior tiles carry no mask arithmetic at all
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        dp[r] = qvis(n0 + nb * 32 + (r >> 2) * 8 + g * 4 + (r & 3)) ? dp[r] : 0.0f;
-                }
+                // off the common path: interior blocks carry no mask arithmetic at all
+                if (kind != MaskKind::NONE) mask_block(dp, kind, qvis, k0 + g * 4, 0.0f);
                 const bf16x8 d0 = c_to_operand<0>(dp), d1 = c_to_operand<1>(dp);
                 __builtin_amdgcn_s_setprio(1);
                 // dQ^T += K^T dS^T, DB independent chains per k-chunk

@@ -221,31 +221,63 @@ __global__ __launch_bounds__(64 * NW, OCC) void mfma_fwd(AttnArgs a) {
             // Two independent accumulator chains, issued alternately: a dependent
             // v_mfma_32x32x16 pair costs 52 cycles, an independent one 32.
             f32x16 s[2];
+            // With a band, a 32-key half of the tile that no query of this wavefront can see (past the diagonal, or
+            // before the band and without a sink key) is neither multiplied nor exponentiated: at window 256 that is
+            // one half in four (the band's two edges and most of the sink tile).
+            bool half_live[2] = {true, true};
+            if (WIN) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s[0][r] = s[1][r] = 0.0f;
+                for (int nb = 0; nb < 2; ++nb) {
+                    const int k0 = n0 + nb * 32, k1 = k0 + 31;
+                    half_live[nb] = !(a.causal && k0 > qhi) && !(a.window > 0 && k1 + a.window <= qlo && k0 >= a.sinks);
+                }
+            }
             // Waves in a matrix phase issue ahead of co-resident waves in the
             // exponent phase: the matrix pipe is the scarcer resource.
             __builtin_amdgcn_s_setprio(1);
+            if (!WIN || (half_live[0] && half_live[1])) {
 #pragma unroll
-            for (int kk = 0; kk < KK; ++kk) {
-                const bf16x8 k0f = lds_read8(Ks + c32 * C::KS + kk * 16 + g * 8);
-                const bf16x8 k1f = lds_read8(Ks + (32 + c32) * C::KS + kk * 16 + g * 8);
-                s[0] = mfma32(k0f, qreg[qb][kk], s[0]);
-                s[1] = mfma32(k1f, qreg[qb][kk], s[1]);
+                for (int r = 0; r < 16; ++r) s[0][r] = s[1][r] = 0.0f;
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) {
+                    const bf16x8 k0f = lds_read8(Ks + c32 * C::KS + kk * 16 + g * 8);
+                    const bf16x8 k1f = lds_read8(Ks + (32 + c32) * C::KS + kk * 16 + g * 8);
+                    s[0] = mfma32(k0f, qreg[qb][kk], s[0]);
+                    s[1] = mfma32(k1f, qreg[qb][kk], s[1]);
+                }
+            } else {  // one half only (the other reads as -inf: its exponentials are zeros and its PV is skipped)
+                const int nl = half_live[0] ? 0 : 1;
+                f32x16 sl;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sl[r] = 0.0f;
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk)
+                    sl = mfma32(lds_read8(Ks + (nl * 32 + c32) * C::KS + kk * 16 + g * 8), qreg[qb][kk], sl);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    s[0][r] = nl == 0 ? sl[r] : -INFINITY;
+                    s[1][r] = nl == 1 ? sl[r] : -INFINITY;
+                }
             }
             __builtin_amdgcn_s_setprio(0);
-            const bool full = (!WIN && NQ == 1) ? t < t_full
-                                                 : (n0 + BN - 1 < a.T) && (!a.causal || n0 + BN - 1 <= qlo) &&
-                                                       (a.window == 0 || n0 + a.window > qhi || n0 + BN - 1 < a.sinks);
-            if (!full) {
+            // Which of the mask's tests a half can fail is wavefront-uniform: none on interior tiles (no mask
+            // arithmetic at all), one on the diagonal or on the band's far edge (one compare and one select an element)
+            if (!WIN && NQ == 1) {
+                if (!(t < t_full)) {
+                    const QueryVis vis(qlo + c32, a.T, a.causal, a.window, a.sinks);
+#pragma unroll
+                    for (int nb = 0; nb < 2; ++nb) {
+                        const MaskKind kind = mask_kind(n0 + nb * 32, n0 + nb * 32 + 31, qlo, qhi, a.T, a.causal, 0, 0);
+                        if (kind != MaskKind::NONE) mask_block(s[nb], kind, vis, n0 + nb * 32 + g * 4, -INFINITY);
+                    }
+                }
+            } else {
                 const QueryVis vis(qlo + c32, a.T, a.causal, a.window, a.sinks);
 #pragma unroll
-                for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int kj = n0 + nb * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
-                        s[nb][r] = vis(kj) ? s[nb][r] : -INFINITY;
-                    }
+                for (int nb = 0; nb < 2; ++nb) {
+                    const MaskKind kind = mask_kind(n0 + nb * 32, n0 + nb * 32 + 31, qlo, qhi, a.T, a.causal, a.window, a.sinks);
+                    if (half_live[nb] && kind != MaskKind::NONE) mask_block(s[nb], kind, vis, n0 + nb * 32 + g * 4, -INFINITY);
+                }
             }
             float mx = -INFINITY;
 #pragma unroll
@@ -279,6 +311,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void mfma_fwd(AttnArgs a) {
             __builtin_amdgcn_s_setprio(1);
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) {
+                if (WIN && !half_live[nb]) continue;  // P of this half is all zeros
                 const bf16x8 p0 = c_to_operand<0>(s[nb]);
                 const bf16x8 p1 = c_to_operand<1>(s[nb]);
 #pragma unroll

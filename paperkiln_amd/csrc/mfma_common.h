@@ -271,6 +271,46 @@ struct QueryVis {
           sinks(window > 0 ? sinks_ : 0) {}
     __device__ bool operator()(int kj) const { return (kj < hi) & ((kj >= win_lo) | (kj < sinks)); }
 };
+// Which of QueryVis's three tests a block of keys [k0, k1] can fail at all for a wavefront whose queries are
+// [qlo, qhi] -- wavefront-uniform, so the mask of a block becomes one scalar branch to a loop with ONE compare and
+// one select per element instead of three compares, two mask combinations and a select: with a band of a few
+// tiles every other live block of a wavefront lies on one of the band's edges and pays for its mask.
+//   UPPER: only `kj < hi` can fail (the diagonal, or the end of the sequence);
+//   LOWER: only `kj >= win_lo` can fail (the band's far edge; no sink key in the block);
+//   SINKS: nothing of the block is inside any query's band: only `kj < sinks` decides;
+//   ALL:   anything else.
+enum class MaskKind { NONE, UPPER, LOWER, SINKS, ALL };
+__device__ inline MaskKind mask_kind(int k0, int k1, int qlo, int qhi, int T, int causal, int window, int sinks) {
+    const bool upper = k1 >= T || (causal && k1 > qlo);                 // some (query, key) pair fails kj < hi
+    const bool lower = window > 0 && k0 + window <= qhi;                // some pair fails kj >= win_lo
+    const bool has_sink = window > 0 && k0 < sinks;
+    if (!upper && (!lower || (has_sink && k1 < sinks))) return MaskKind::NONE;
+    if (upper && !lower) return MaskKind::UPPER;
+    if (!upper && lower && !has_sink) return MaskKind::LOWER;
+    if (!upper && lower && k1 + window <= qlo) return MaskKind::SINKS;  // wholly outside every band: sink keys only
+    return MaskKind::ALL;
+}
+// x[r] of a C tile (lane = query, element r = key kbase + (r/4)*8 + r%4, kbase already carrying the lane's 4g) kept
+// where the key is visible, else `fill`
+__device__ inline void mask_block(f32x16& x, MaskKind kind, const QueryVis& vis, int kbase, float fill) {
+    if (kind == MaskKind::UPPER) {
+        const int lim = vis.hi - kbase;  // visible: offset < lim
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x[r] = ((r >> 2) * 8 + (r & 3) < lim) ? x[r] : fill;
+    } else if (kind == MaskKind::LOWER) {
+        const int lim = vis.win_lo - kbase;  // visible: offset >= lim
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x[r] = ((r >> 2) * 8 + (r & 3) >= lim) ? x[r] : fill;
+    } else if (kind == MaskKind::SINKS) {
+        const int lim = vis.sinks - kbase;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x[r] = ((r >> 2) * 8 + (r & 3) < lim) ? x[r] : fill;
+    } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x[r] = vis(kbase + (r >> 2) * 8 + (r & 3)) ? x[r] : fill;
+    }
+}
+
 // KeyVis: fixed key, varying query (lane = key kernels).
 struct KeyVis {
     int q_lo;    // queries >= q_lo pass the causal test
