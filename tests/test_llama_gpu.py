@@ -102,6 +102,33 @@ def test_bf16_checkpointing_keeps_the_loss(name):
     m.close()
 
 
+def test_config5_loss_at_full_size_against_the_reference():
+    """BASELINE config 5 at its full size (6 layers, d 512, 8 heads, d_ff 1376, vocab 32000 tied, B=8 x T=1024): the
+    loss the compiled reference computes on one CPU core in 19 minutes (tests/golden/llama_cfg5_loss.json, written by
+    tests/golden/make_llama_cfg5_loss.py with parameters and token ids from this repository's portable generator)
+    against the HIP path: fp32 compute within 1e-4 (the bar BASELINE sets between two runs of the same step),
+    bf16 compute within 2e-2, checkpointed == plain in both."""
+    import json
+    ref = json.load(open(os.path.join(GOLDEN, "llama_cfg5_loss.json")))
+    cfg, B, T = ref["cfg"], ref["B"], ref["T"]
+    params = {}
+    for i, (n, shp) in enumerate(zip(ref["names"], ref["shapes"])):
+        is_norm = n.endswith("norm.weight") or n.endswith("layernorm.weight")
+        params[n] = np.ones(shp, np.float32) if is_norm else synth.randn(1000 + i, tuple(shp), 0.02)
+    toks = synth.randint(9, B * T + 1, cfg["vocab"])
+    x, y = toks[:-1], toks[1:]
+    for dtype, bar in (("fp32", 1e-4), ("bf16", 2e-2)):
+        m = Llama(compute_dtype=dtype, **cfg)
+        assert set(m.names) == set(params)
+        m.set_params(params)
+        loss_c, _ = m.loss_backward(x, y, T, checkpoint=True)
+        loss_p, _ = m.loss_backward(x, y, T, checkpoint=False)
+        print(f"\n  config 5 {dtype}: loss {loss_c:.7f} (checkpointed) {loss_p:.7f} (plain) vs reference {ref['loss']:.7f}")
+        assert abs(loss_c - loss_p) <= 1e-4
+        assert abs(loss_c - ref["loss"]) <= bar
+        m.close()
+
+
 def test_larger_model_checkpoint_receipt():
     """A model big enough for the byte receipt to mean something: 4 layers, d=256, 1024 tokens, bf16."""
     cfg = dict(vocab=2048, d=256, n_layers=4, n_heads=4, d_ff=688)
