@@ -29,16 +29,19 @@ PEAK_HBM_GBS = 8000.0      # MI355X HBM3E, published
 PEAK_FP32_TFLOPS = 157.3   # MI355X dense fp32 MFMA, published
 
 PMC_SUMMARY = os.path.join(ROOT, "profiles", "attn_fwd_bwd_causal_B4_H16_T4096_d128_pmc.txt")
+PMC_SUMMARY_WINDOW = os.path.join(ROOT, "profiles", "attn_fwd_bwd_window256_sinks4_B4_H16_T4096_d128_pmc.txt")
+TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel as committed under profiles/ (a constant read "
+                  "from that summary, not a measurement of this run)")
 
 
-def measured_traffic_bytes():
-    """HBM bytes per launch of each headline kernel, read from the committed summary of the two `rocprofv3 --pmc`
+def measured_traffic_bytes(path=PMC_SUMMARY):
+    """HBM bytes per launch of each kernel of a workload, read from the committed summary of the two `rocprofv3 --pmc`
     runs (FETCH_SIZE, WRITE_SIZE, each scaled by what the same counter reads for a copy kernel of known size; the
     factors are stated in that file). Returns {} when the summary is missing: traffic is then reported as null."""
     import re
     out, kernel = {}, None
     try:
-        for line in open(PMC_SUMMARY):
+        for line in open(path):
             m = re.match(r"(mfma_\w+)<", line)
             if m:
                 kernel = {"mfma_fwd": "fwd", "mfma_dq": "dq", "mfma_dq3": "dq", "mfma_dkdv2": "dkdv",
@@ -129,10 +132,14 @@ def window_variant(ops, q, k, v, d_o, out, scale, B, H, T, dk, warmup, steps):
     ms = (time.perf_counter() - t0) / steps * 1e3
     pairs = synth.visible_pairs(T, True, W, S)
     nbytes = 12.0 * B * T * H * dk * 2 + 2.0 * B * H * T * 4
+    traffic = measured_traffic_bytes(PMC_SUMMARY_WINDOW)  # the three kernels of one step together
     return {"workload": "same shape, window=256, sinks=4", "ms_per_step": round(ms, 4),
             "tflops": round(14.0 * dk * pairs * B * H / (ms * 1e-3) / 1e12, 2),
             "roofline": {"bound": "hbm", "achieved": round(nbytes / (ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
-                         "unit": "GB/s", "frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}}
+                         "unit": "GB/s", "frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                         "algorithmic_bytes": nbytes,
+                         "traffic": sum(traffic.values()) if len(traffic) == 3 else None,
+                         "traffic_source": TRAFFIC_SOURCE}}
 
 
 def other_config(ops, name, B, Hq, Hkv, T, dk, theta, bound, steps=400, warmup=50):
@@ -376,8 +383,7 @@ def main():
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                      "traffic": measured_traffic_bytes().get(dominant),
-                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel as committed under "
-                                       "profiles/ (a constant read from that summary, not a measurement of this run)"},
+                     "traffic_source": TRAFFIC_SOURCE},
     }
     extras = [x for x in args.sections.split(",") if x]
     if "window" in extras:
