@@ -73,10 +73,14 @@ int pk_attn_fwd(const pk_attn_shape* s, const pk_tensor4* q, const pk_tensor4* k
                 const pk_tensor4* v, const pk_tensor4* o, float* lse, void* stream);
 
 /* Bytes of scratch pk_attn_bwd needs for this shape AND mask: the row sums
- * D_i [B,Hq,T] fp32 and, for a band mask with 1..32 sink keys, room for the
+ * D_i [B,Hq,T] fp32; for a band mask with 1..32 sink keys, room for the
  * partial dK/dV rows of the sink keys (the queries past the band of the first
  * key block may be handed to extra workgroups whose partial sums are added in
- * a fixed order). Ask with the window and sinks the backward will run with. */
+ * a fixed order); and, without a band, where query heads share KV heads
+ * (Hq > Hkv) on a shape too small to fill the GPU, room for the fp32 partial
+ * dK/dV of the workgroups that the heads of a group are dealt to (added in a
+ * fixed order as well). Ask with the window and sinks the backward will run
+ * with. */
 size_t pk_attn_bwd_workspace_bytes(const pk_attn_shape* s);
 
 /* Backward closure of the same node (src/ops.cpp:902-933, 997-1026),
@@ -107,8 +111,11 @@ int pk_attn_bwd_stages(const pk_attn_shape* s, const pk_tensor4* q, const pk_ten
 /* pk_attn_bwd without a workspace argument and without any allocation: the scratch is a device array inside
  * the library (PK_ATTN_BWD_STATIC_MAX_WORKSPACE bytes on every GPU the library runs on, held until the process
  * ends). It has no counterpart in the reference; it is for callers that cannot allocate: code under HIP graph
- * capture, tight serving loops, harnesses that forbid hipMalloc. Same kernels and same results as pk_attn_bwd.
- * A shape whose pk_attn_bwd_workspace_bytes() exceeds the array is refused with PK_ERR_WORKSPACE. All calls on
+ * capture, tight serving loops, harnesses that forbid hipMalloc. Same kernels as pk_attn_bwd, and the same
+ * results bit for bit wherever the array also holds the partial sums of a GQA head split (see
+ * pk_attn_bwd_workspace_bytes); where only those do not fit, the heads of a group are walked by one workgroup,
+ * which changes the order of summation of dK/dV and nothing else. A shape whose row sums and sink rows alone
+ * exceed the array is refused with PK_ERR_WORKSPACE. All calls on
  * one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race; calls
  * on one stream are ordered and safe. pk_init looks the array up for its device; otherwise the first call does. */
 #define PK_ATTN_BWD_STATIC_MAX_WORKSPACE ((size_t)32 << 20)
@@ -122,10 +129,13 @@ int pk_attn_bwd_static(const pk_attn_shape* s, const pk_tensor4* q, const pk_ten
  * the per-call cudaMalloc/cudaFree in src/cuda_resident.cu:226-263 and
  * src/cuda_ops.cu:63-72, and the byte receipt that the reference's
  * live_variables() (include/microtorch/autograd.hpp:61-64) cannot give.
- * A freed block is handed out again at once, without waiting for the GPU: that
- * is safe for work queued on ONE stream (later work on that stream runs after
- * the earlier work that used the block), which is how one model's tape runs.
- * Memory that several streams touch must come from elsewhere. */
+ * A freed block is handed out again at once, without waiting for the GPU, to
+ * a request made for the stream that used the block last (the stream it was
+ * allocated for, or the `stream` argument of the last pk_* call it was passed
+ * to): later work on that stream runs after the earlier work that used the
+ * block. A request for another stream takes the block over only once that
+ * stream has nothing queued any more. A block that several streams use at the
+ * same time is the caller's to keep alive until all of them are done. */
 int pk_alloc(size_t bytes, void** out);
 int pk_free(void* p);   /* PK_ERR_ARGUMENT for a pointer pk_alloc did not return or that was freed before */
 /* Host <-> device copies on `stream`; both return after the copy has completed. They stand where the
