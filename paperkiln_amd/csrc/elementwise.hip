@@ -588,19 +588,30 @@ __global__ void iota_i32(int* x, int n) {
     const int i = blockIdx.x * NT + threadIdx.x;
     if (i < n) x[i] = i;
 }
+// A run may be the whole input (every row the same id), so its columns are dealt to grid.y workgroups of one
+// wavefront each and the rows are fetched EMB_ROWS at a time (independent loads in flight) and then added one by one.
+constexpr int EMB_NT = 64, EMB_ROWS = 8;
 template <typename T>
-__global__ void emb_bwd_runs(const T* dy, const int* sorted_id, const int* row_of, float* dtable, int n, int d) {
+__global__ void __launch_bounds__(EMB_NT) emb_bwd_runs(const T* dy, const int* sorted_id, const int* row_of, float* dtable, int n, int d) {
     const int p = blockIdx.x;
     const int id = sorted_id[p];
     if (p > 0 && sorted_id[p - 1] == id) return;
     int end = p + 1;
     while (end < n && sorted_id[end] == id) ++end;
-    for (int c = threadIdx.x; c < d; c += NT) {
-        float* dst = dtable + static_cast<int64_t>(id) * d + c;
-        float acc = *dst;
-        for (int r = p; r < end; ++r) acc += ldf(dy, static_cast<int64_t>(row_of[r]) * d + c);
-        *dst = acc;
+    const int c = blockIdx.y * EMB_NT + threadIdx.x;
+    if (c >= d) return;
+    float* dst = dtable + static_cast<int64_t>(id) * d + c;
+    float acc = *dst;
+    int r = p;
+    for (; r + EMB_ROWS <= end; r += EMB_ROWS) {
+        float v[EMB_ROWS];
+#pragma unroll
+        for (int u = 0; u < EMB_ROWS; ++u) v[u] = ldf(dy, static_cast<int64_t>(row_of[r + u]) * d + c);
+#pragma unroll
+        for (int u = 0; u < EMB_ROWS; ++u) acc += v[u];
     }
+    for (; r < end; ++r) acc += ldf(dy, static_cast<int64_t>(row_of[r]) * d + c);
+    *dst = acc;
 }
 
 __device__ inline float block_reduce(float x, bool is_max, float* sh) {
@@ -982,7 +993,7 @@ void k_embedding_bwd(const Tensor& dy, const int* ids, const Tensor& dtable) {
     HIPCHK(hipcub::DeviceRadixSort::SortPairs(nullptr, tmp_bytes, ids, i_out, r_in, r_out, n, 0, 32, st));
     Buffer tmp(tmp_bytes ? tmp_bytes : 16);
     HIPCHK(hipcub::DeviceRadixSort::SortPairs(tmp.p, tmp_bytes, ids, i_out, r_in, r_out, n, 0, 32, st));
-    PK_DISPATCH1(T, dy.dtype, hipLaunchKernelGGL((emb_bwd_runs<T>), dim3(n), dim3(NT), 0, st,
+    PK_DISPATCH1(T, dy.dtype, hipLaunchKernelGGL((emb_bwd_runs<T>), dim3(n, (d + EMB_NT - 1) / EMB_NT), dim3(EMB_NT), 0, st,
                                                  static_cast<const T*>(dy.ptr()), i_out, r_out,
                                                  static_cast<float*>(dtable.ptr()), n, d));
     post();

@@ -100,13 +100,14 @@ def test_embedding_vs_reference_vectors(bo, vec):
 
 
 def test_embedding_gradient_is_summed_in_row_order(bo, oracle):
-    """Heavily repeated ids (3000 rows over 7 table rows, plus a table far larger than the row count): the
-    scatter-add forms each table row's sum in ascending row order, as the reference's loop does
-    (src/ops.cpp:338-347), so it equals the CPU restatement bit for bit and is the same on every run."""
-    for vocab, n, seed in ((7, 3000, 51), (40_000, 257, 52)):
-        table = synth.randn(seed, (vocab, 48), 0.5)
+    """Heavily repeated ids (3000 rows over 7 table rows, a table far larger than the row count, and 8192 rows
+    that all name one id, the longest run there can be): the scatter-add forms each table row's sum in ascending
+    row order, as the reference's loop does (src/ops.cpp:338-347), so it equals the CPU restatement bit for bit
+    and is the same on every run."""
+    for vocab, n, d, seed in ((7, 3000, 48, 51), (40_000, 257, 48, 52), (1, 8192, 512, 53), (3, 1001, 130, 54)):
+        table = synth.randn(seed, (vocab, d), 0.5)
         ids = synth.randint(seed + 100, n, vocab).astype(np.int32)
-        g = synth.randn(seed + 200, (n, 48), 1.0)
+        g = synth.randn(seed + 200, (n, d), 1.0)
         _, want = oracle.embedding(table, ids, g)
         runs = [host(bo.embedding(dev(table), dev(ids), dev(g))[1]) for _ in range(3)]
         assert np.array_equal(runs[0], want)
