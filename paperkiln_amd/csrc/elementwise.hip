@@ -1095,15 +1095,13 @@ void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dty
     if (A.dtype != B.dtype) throw std::runtime_error("gemm: operand dtypes differ");
     // Which kernel: measured per shape on the MI355X as GPU time from a kernel trace (timing launches from the host
     // measures the library's longer host path instead), on the Linear shapes of a d = 512 block and of the tied
-    // head. The two are within 15 % of each other on short contractions; the library's kernels are clearly
-    // ahead on long ones (K >= 1376: 695 - 870 TFLOP/s against 490 - 650) and on the split weight-gradient
-    // products. The hand-written kernel is ahead where a short contraction meets an output width that is not a
-    // multiple of 256, because the library's 176 - 256-wide tiles waste more of their last column there than
-    // 128 x 128 tiles do: [8192, 512] x [512, 2752] 42.9 against 55.0 us, [8192, 512] x [1376, 512]^T 23.7 against
-    // 38.1 us. That class goes to the hand-written kernel, everything else to the library.
-    // backend 2 sends everything the hand-written kernel takes to it.
+    // head. The hand-written kernel is ahead of or level with the library on the products whose A is not
+    // transposed (activations times weights, gradients times weights: 8 of 10 shapes, the other two within 11 %)
+    // and on a transposed-A product with an output large enough for 256 x 256 tiles without splitting the
+    // contraction (the tied head's dE); the library keeps the small-output weight-gradient products.
+    // backend 2 sends everything the hand-written kernel takes to it, backend 0 nothing.
     const int backend = gemm_backend();
-    const bool mine = backend == 2 || (backend == 1 && !tA && Ka <= 1024 && N % 256 != 0 && N >= 1024);
+    const bool mine = backend == 2 || (backend == 1 && (!tA || ((M + 255) / 256) * ((N + 255) / 256) >= 240));
     if (A.dtype == PK_BF16 && mine &&
         gemm_mfma_bf16(A.ptr(), tA, lda, B.ptr(), tB, B.cols, C, c_dtype, M, N, Ka, ldc, beta, tape_stream()))
         return;

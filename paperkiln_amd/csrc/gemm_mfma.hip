@@ -35,10 +35,13 @@ constexpr int PITCH_ROW = BK + 8;  // [rows][64 k]: 16-byte row reads conflict-f
 //          hundred tiles, where more and smaller workgroups fill the chip better.
 //   Large: 2 x 4 wavefronts of 4 x 2 -> 256 x 256, 512 threads, one workgroup per CU: half the operand bytes per
 //          MFMA, which is what the vector memory path (64 bytes per clock and CU) asks for on long runs.
-template <int WGM_, int WGN_, int FM_, int FN_>
+//   KS > 1 (ring kernel only): KS sets of WGM x WGN wavefronts share the tile, set q multiplying the q-th part of every
+//          64-deep slice; their accumulators are added through LDS at the end. Two wavefronts per SIMD from one
+//          workgroup, for outputs of so few tiles that a CU gets no second workgroup.
+template <int WGM_, int WGN_, int FM_, int FN_, int KS_ = 1>
 struct Geo {
-    static constexpr int WGM = WGM_, WGN = WGN_, FM = FM_, FN = FN_;
-    static constexpr int BM = WGM * FM * 32, BN = WGN * FN * 32, NTHR = WGM * WGN * 64;
+    static constexpr int WGM = WGM_, WGN = WGN_, FM = FM_, FN = FN_, KS = KS_;
+    static constexpr int BM = WGM * FM * 32, BN = WGN * FN * 32, NTHR = WGM * WGN * KS * 64;
     // [64 k][columns] tiles: a pitch of 32 past a multiple of 128 keeps the transposing reads conflict-free
     static constexpr int PITCH_TR_A = BM + 32, PITCH_TR_B = BN + 32;
     static constexpr int A_EL = BM * PITCH_ROW > BK * PITCH_TR_A ? BM * PITCH_ROW : BK * PITCH_TR_A;
@@ -47,6 +50,7 @@ struct Geo {
 };
 using GeoSmall = Geo<2, 2, 2, 2>;
 using GeoLarge = Geo<2, 4, 4, 2>;
+using GeoSmallK2 = Geo<2, 2, 2, 2, 2>;
 
 struct GemmArgs {
     const uint16_t* a;
@@ -106,10 +110,69 @@ __device__ inline void commit_tile(uint16_t* tile, const u32x4 (&r)[NCH]) {
     }
 }
 
+// Epilogue through LDS, one strip of 32 rows per wavefront row at a time: the strip as [WGM * 32][BN + pad]
+// in the output's element type, then 16-byte chunks of consecutive columns to global memory (read-add-write
+// when accumulating). `lds` is the kernel's whole LDS allocation, free to overwrite when this is called.
+template <typename G, bool CF32>
+__device__ inline void store_tile(const f32x16 (&acc)[G::FM][G::FN], void* lds, const GemmArgs& g, int m0, int n0, int wm, int wn,
+                                  int c32, int gh, bool writer = true) {
+    constexpr int BN = G::BN, NTHR = G::NTHR, FM = G::FM, FN = G::FN;
+    typedef typename std::conditional<CF32, float, uint16_t>::type CT;
+    constexpr int CP = BN + (CF32 ? 4 : 8);  // pitch in elements: rows stay 16-byte aligned
+    constexpr int EPC = CF32 ? 4 : 8;        // elements per 16-byte chunk
+    constexpr int CPR = BN / EPC;            // chunks per strip row
+    CT* cs = reinterpret_cast<CT*>(lds);
+    CT* cout = static_cast<CT*>(g.c) + (g.part_stride ? static_cast<int64_t>(blockIdx.z) * g.part_stride : 0);
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                if (!writer) continue;  // wavefront-uniform: the wavefronts that hold the tile's sums
+                const int row = wm * 32 + c32, col = (wn * FN + j) * 32 + qd * 8 + gh * 4;
+                if (CF32) {
+                    const f32x4 v = {acc[i][j][qd * 4], acc[i][j][qd * 4 + 1], acc[i][j][qd * 4 + 2], acc[i][j][qd * 4 + 3]};
+                    *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(cs) + row * CP + col) = v;
+                } else {
+                    const u32x2 v = {pack_bf16(acc[i][j][qd * 4], acc[i][j][qd * 4 + 1]),
+                                     pack_bf16(acc[i][j][qd * 4 + 2], acc[i][j][qd * 4 + 3])};
+                    *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(cs) + row * CP + col) = v;
+                }
+            }
+        __syncthreads();
+        for (int c = threadIdx.x; c < G::WGM * 32 * CPR; c += NTHR) {
+            const int srow = c / CPR, ch = c % CPR;
+            // strip row srow belongs to wavefront row srow / 32, whose i-th block of 32 rows this is
+            const int m = m0 + ((srow >> 5) * FM + i) * 32 + (srow & 31), n = n0 + ch * EPC;
+            if (m >= g.M || n >= g.N) continue;
+            u32x4 v = *reinterpret_cast<const u32x4*>(cs + srow * CP + ch * EPC);
+            CT* dst = cout + static_cast<int64_t>(m) * g.ldc + n;
+            if (g.beta) {
+                const u32x4 old = *reinterpret_cast<const u32x4*>(dst);
+                if (CF32) {
+                    f32x4 s = *reinterpret_cast<const f32x4*>(&old) + *reinterpret_cast<const f32x4*>(&v);
+                    v = *reinterpret_cast<const u32x4*>(&s);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float lo = __uint_as_float(old[e] << 16) + __uint_as_float(v[e] << 16);
+                        const float hi = __uint_as_float(old[e] & 0xffff0000u) + __uint_as_float(v[e] & 0xffff0000u);
+                        v[e] = pack_bf16(lo, hi);
+                    }
+                }
+            }
+            *reinterpret_cast<u32x4*>(dst) = v;
+        }
+        __syncthreads();
+    }
+}
+
 template <typename G, bool TA, bool TB, bool CF32>
 __global__ __launch_bounds__(G::NTHR, 2) void gemm_bf16(GemmArgs g) {
     constexpr int BM = G::BM, BN = G::BN, NTHR = G::NTHR, FM = G::FM, FN = G::FN;
     __shared__ __attribute__((aligned(16))) uint16_t lds[2 * (G::A_EL + G::B_EL)];  // [buffer][A | B]
+    static_assert(G::WGM * 32 * (G::BN + 8) * (CF32 ? 4 : 2) <= sizeof(lds), "epilogue strip must fit the tile buffers");
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c32 = lane & 31, gh = lane >> 5, wm = w / G::WGN, wn = w % G::WGN;
 
@@ -173,58 +236,220 @@ __global__ __launch_bounds__(G::NTHR, 2) void gemm_bf16(GemmArgs g) {
         buf ^= 1;
     }
 
-    // Epilogue through LDS, one strip of 32 rows per wavefront row at a time: the strip as [WGM * 32][BN + pad]
-    // in the output's element type, then 16-byte chunks of consecutive columns to global memory (read-add-write
-    // when accumulating).
-    typedef typename std::conditional<CF32, float, uint16_t>::type CT;
-    constexpr int CP = BN + (CF32 ? 4 : 8);  // pitch in elements: rows stay 16-byte aligned
-    constexpr int EPC = CF32 ? 4 : 8;        // elements per 16-byte chunk
-    constexpr int CPR = BN / EPC;            // chunks per strip row
-    static_assert(G::WGM * 32 * CP * sizeof(CT) <= sizeof(lds), "epilogue strip must fit the tile buffers");
-    CT* cs = reinterpret_cast<CT*>(lds);
-    CT* cout = static_cast<CT*>(g.c) + (g.part_stride ? static_cast<int64_t>(blockIdx.z) * g.part_stride : 0);
+    store_tile<G, CF32>(acc, lds, g, m0, n0, wm, wn, c32, gh);
+}
+
+// ---- the same tiles fed through a ring of LDS slots ---------------------------------------------------------------
+// With one workgroup per CU (an output of 256 tiles or fewer, or tiles whose buffers fill the LDS) a slice's global
+// loads have one slice of matrix work to hide behind, 512 clocks against a round trip of 1,500 - 2,000: the loop
+// runs at the memory latency. Here the operand slices go from memory straight into LDS (buffer_load_dwordx4 ... lds:
+// no staging registers, no LDS stores, and a lane outside the matrix writes zeros), into a ring of NS slots, and
+// the loads of slice s + NS - 1 are issued before slice s is multiplied: NS - 1 slices of work per round trip. The
+// LDS layouts and the fragment reads are those of gemm_bf16.
+//
+// One instruction fills 1 KB of LDS lane after lane, so a lane's place in LDS is fixed and what varies is which 16
+// bytes of memory it fetches: unit u = 64 * instruction + lane of an operand's slice lies at LDS byte 16 u, i.e.
+// row u / UPR, chunk u % UPR of the padded tile; the padding units ask for an address outside the buffer.
+template <bool TR, int SPAN, int NW>
+struct RingOp {
+    static constexpr int UPR = TR ? (SPAN + 32) / 8 : PITCH_ROW / 8;  // 16-byte units per LDS row
+    static constexpr int DATA = TR ? SPAN / 8 : BK / 8;               // of which hold data
+    static constexpr int ROWS = TR ? BK : SPAN;
+    static_assert(ROWS * UPR % 64 == 0, "a slice is a whole number of wavefront loads");
+    static constexpr int NI = ROWS * UPR / 64;       // wavefront loads per slice
+    static constexpr int PER = (NI + NW - 1) / NW;   // at most this many per wavefront
+    static constexpr int BYTES = NI * 1024;
+    // loads wavefront w issues per slice: instructions w, w + NW, ...
+    __device__ static int count(int w) { return (NI - w + NW - 1) / NW; }
+};
+constexpr uint32_t OUTSIDE = 0x80000000u;  // a byte offset no buffer of less than 2 GiB contains
+
+// An operand's slice cursor: pointer to the tile's first element of the slice in hand, bytes from there to the end of
+// the operand (the buffer's extent, so rows past the matrix -- and, where the contraction index is the row, rows past
+// the contraction's end -- read as zeros), bytes per slice.
+struct SliceCursor {
+    const char* p;
+    int left, step;
+    __device__ u32x4 rsrc() const {
+        const uint64_t a = reinterpret_cast<uint64_t>(p);
+        const u32x4 r = {static_cast<uint32_t>(a), static_cast<uint32_t>(a >> 32) & 0xffffu, static_cast<uint32_t>(left),
+                         0x00020000u};
+        return r;
+    }
+    __device__ void next() {
+        p += step;
+        left = max(left - step, 0);
+    }
+};
+template <bool TR>
+__device__ inline SliceCursor slice_cursor(const uint16_t* base, int64_t ld, int rc0, int rc_count, int k_begin, int k_end) {
+    SliceCursor c;
+    const int64_t kspan = k_end - k_begin, rcs = rc_count - rc0;
+    if (!TR) {  // [row][k]
+        c.p = reinterpret_cast<const char*>(base + static_cast<int64_t>(rc0) * ld + k_begin);
+        c.left = static_cast<int>(((rcs - 1) * ld + kspan) * 2);
+        c.step = BK * 2;
+    } else {  // [k][column]
+        c.p = reinterpret_cast<const char*>(base + static_cast<int64_t>(k_begin) * ld + rc0);
+        c.left = static_cast<int>(((kspan - 1) * ld + rcs) * 2);
+        c.step = static_cast<int>(BK * ld * 2);
+    }
+    return c;
+}
+// m0 is set and used inside the one statement; the compiler never keeps a value of its own in m0 across other code.
+__device__ inline void dma16(uint32_t lds_byte, uint32_t voff, u32x4 rsrc) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_byte), "v"(voff), "s"(rsrc)
+                 : "memory");
+}
+template <int N>
+__device__ inline void wait_loads_then_barrier() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+template <typename G, bool TA, bool TB, bool CF32, int NS>
+__global__ __launch_bounds__(G::NTHR, NS <= 2 ? 2 : 1) void gemm_ring(GemmArgs g) {
+    constexpr int BM = G::BM, BN = G::BN, NTHR = G::NTHR, FM = G::FM, FN = G::FN, NW = NTHR / 64;
+    using OA = RingOp<TA, BM, NW>;
+    using OB = RingOp<!TB, BN, NW>;
+    constexpr int SLOT = OA::BYTES + OB::BYTES;
+    static_assert(NS * SLOT <= 160 * 1024, "the ring must fit the LDS");
+    static_assert(G::WGM * 32 * (G::BN + 8) * (CF32 ? 4 : 2) <= NS * SLOT, "epilogue strip must fit the ring");
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[NS * SLOT];
+    const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    constexpr int KS = G::KS, NWQ = G::WGM * G::WGN, KPW = BK / 16 / KS;  // k-chunks of a slice per wavefront
+    static_assert(KS == 1 || KS == 2, "one or two wavefront sets");
+    static_assert(KS == 1 || NWQ * 64 * FM * FN * 64 <= NS * SLOT, "the second set's accumulators pass through the ring");
+    const int ks = w / NWQ, wq = w - ks * NWQ;
+    const int c32 = lane & 31, gh = lane >> 5, wm = wq / G::WGN, wn = wq % G::WGN;
+
+    const int ntiles = g.tiles_m * g.tiles_n;
+    const int per_xcd = (ntiles + 7) / 8;
+    const int t = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (t >= ntiles) return;
+    const int m0 = (t / g.tiles_n) * BM, n0 = (t % g.tiles_n) * BN;
+    const int k_begin = blockIdx.z * g.k_per_split, k_end = min(g.K, k_begin + g.k_per_split);
+    const int nslices = (k_end - k_begin + BK - 1) / BK, ktail = (k_end - k_begin) % BK;
+
+    // what this lane fetches with its j-th load of a slice; in the contraction's last, partial slice of a [row][k]
+    // operand the chunks past the end must not be read (they are the next row's, or another split's)
+    uint32_t offa[OA::PER], offb[OB::PER], offa_t[OA::PER], offb_t[OB::PER];
 #pragma unroll
-    for (int i = 0; i < FM; ++i) {
+    for (int j = 0; j < OA::PER; ++j) {
+        const int u = (j * NW + w) * 64 + lane, row = u / OA::UPR, ch = u % OA::UPR;
+        const bool ok = ch < OA::DATA && (!TA || m0 + ch * 8 < g.M);
+        offa[j] = ok ? static_cast<uint32_t>(row) * static_cast<uint32_t>(g.lda) * 2u + ch * 16u : OUTSIDE;
+        offa_t[j] = (TA || ch * 8 < ktail) ? offa[j] : OUTSIDE;
+    }
+#pragma unroll
+    for (int j = 0; j < OB::PER; ++j) {
+        const int u = (j * NW + w) * 64 + lane, row = u / OB::UPR, ch = u % OB::UPR;
+        const bool ok = ch < OB::DATA && (TB || n0 + ch * 8 < g.N);
+        offb[j] = ok ? static_cast<uint32_t>(row) * static_cast<uint32_t>(g.ldb) * 2u + ch * 16u : OUTSIDE;
+        offb_t[j] = (!TB || ch * 8 < ktail) ? offb[j] : OUTSIDE;
+    }
+    SliceCursor ca = slice_cursor<TA>(g.a, g.lda, m0, g.M, k_begin, k_end);
+    SliceCursor cb = slice_cursor<!TB>(g.b, g.ldb, n0, g.N, k_begin, k_end);
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+    const int na = OA::count(w), nb = OB::count(w);
+
+    // slices are asked for in order, one call per slice, also past the last one (nothing is fetched then, the
+    // lanes write zeros into a slot nobody reads: every wavefront's count of loads in flight stays the same)
+    int f_slice = 0;
+    auto fetch = [&](int slot) {
+        const bool none = f_slice >= nslices, tail = ktail != 0 && f_slice == nslices - 1;
+        SliceCursor xa = ca, xb = cb;
+        if (none) xa.left = xb.left = 0;
+        const u32x4 ra = xa.rsrc(), rb = xb.rsrc();
+        const uint32_t base = lds0 + static_cast<uint32_t>(slot) * SLOT;
+#pragma unroll
+        for (int j = 0; j < OA::PER; ++j)
+            if (j < na) dma16(base + (j * NW + w) * 1024u, tail ? offa_t[j] : offa[j], ra);
+#pragma unroll
+        for (int j = 0; j < OB::PER; ++j)
+            if (j < nb) dma16(base + OA::BYTES + (j * NW + w) * 1024u, tail ? offb_t[j] : offb[j], rb);
+        ca.next();
+        cb.next();
+        ++f_slice;
+    };
+    // waits until this wavefront's loads of the oldest slice in flight have landed, then for everybody's
+    constexpr int CMAX = OA::PER + OB::PER;
+    const int cnt = na + nb;
+    auto landed = [&]() {
+        if (cnt == CMAX)
+            wait_loads_then_barrier<(NS - 2) * CMAX>();
+        else if (cnt == CMAX - 1)
+            wait_loads_then_barrier<(NS - 2) * (CMAX - 1)>();
+        else
+            wait_loads_then_barrier<(NS - 2) * (CMAX - 2)>();
+    };
+
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j)
 #pragma unroll
-            for (int qd = 0; qd < 4; ++qd) {
-                const int row = wm * 32 + c32, col = (wn * FN + j) * 32 + qd * 8 + gh * 4;
-                if (CF32) {
-                    const f32x4 v = {acc[i][j][qd * 4], acc[i][j][qd * 4 + 1], acc[i][j][qd * 4 + 2], acc[i][j][qd * 4 + 3]};
-                    *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(cs) + row * CP + col) = v;
-                } else {
-                    const u32x2 v = {pack_bf16(acc[i][j][qd * 4], acc[i][j][qd * 4 + 1]),
-                                     pack_bf16(acc[i][j][qd * 4 + 2], acc[i][j][qd * 4 + 3])};
-                    *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(cs) + row * CP + col) = v;
-                }
-            }
-        __syncthreads();
-        for (int c = threadIdx.x; c < G::WGM * 32 * CPR; c += NTHR) {
-            const int srow = c / CPR, ch = c % CPR;
-            // strip row srow belongs to wavefront row srow / 32, whose i-th block of 32 rows this is
-            const int m = m0 + ((srow >> 5) * FM + i) * 32 + (srow & 31), n = n0 + ch * EPC;
-            if (m >= g.M || n >= g.N) continue;
-            u32x4 v = *reinterpret_cast<const u32x4*>(cs + srow * CP + ch * EPC);
-            CT* dst = cout + static_cast<int64_t>(m) * g.ldc + n;
-            if (g.beta) {
-                const u32x4 old = *reinterpret_cast<const u32x4*>(dst);
-                if (CF32) {
-                    f32x4 s = *reinterpret_cast<const f32x4*>(&old) + *reinterpret_cast<const f32x4*>(&v);
-                    v = *reinterpret_cast<const u32x4*>(&s);
-                } else {
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float lo = __uint_as_float(old[e] << 16) + __uint_as_float(v[e] << 16);
-                        const float hi = __uint_as_float(old[e] & 0xffff0000u) + __uint_as_float(v[e] & 0xffff0000u);
-                        v[e] = pack_bf16(lo, hi);
+    for (int s = 0; s < NS - 1; ++s) fetch(s);
+    int slot = 0, fslot = NS - 1;
+    for (int s = 0; s < nslices; ++s) {
+        landed();      // slice s is in its slot, and slice s - 1 has been read by every wavefront
+        fetch(fslot);  // slice s + NS - 1 into the slot slice s - 1 leaves
+        const uint16_t* As = reinterpret_cast<const uint16_t*>(lds + slot * SLOT);
+        const uint16_t* Bs = reinterpret_cast<const uint16_t*>(lds + slot * SLOT + OA::BYTES);
+#pragma unroll
+        for (int kq = 0; kq < KPW; ++kq) {
+            const int kk = ks * KPW + kq;
+            bf16x8 fa[FM], fb[FN];
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+                fa[i] = TA ? read_tr_nat(As, G::PITCH_TR_A, kk * 16, (wm * FM + i) * 32, lane)
+                           : lds_read8(As + ((wm * FM + i) * 32 + c32) * PITCH_ROW + kk * 16 + gh * 8);
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+                fb[j] = !TB ? read_tr_nat(Bs, G::PITCH_TR_B, kk * 16, (wn * FN + j) * 32, lane)
+                            : lds_read8(Bs + ((wn * FN + j) * 32 + c32) * PITCH_ROW + kk * 16 + gh * 8);
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j) acc[i][j] = mfma32(fb[j], fa[i], acc[i][j]);
+        }
+        slot = slot + 1 == NS ? 0 : slot + 1;
+        fslot = fslot + 1 == NS ? 0 : fslot + 1;
+    }
+    wait_loads_then_barrier<0>();  // the zero-filling loads past the end have landed too: the ring is free
+    if (KS == 2) {  // set 1 hands its sums to set 0: [wavefront][16-byte group of the 64 registers][lane]
+        f32x4* red = reinterpret_cast<f32x4*>(lds) + wq * (FM * FN * 4) * 64 + lane;
+        if (ks == 1) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int qd = 0; qd < 4; ++qd) {
+                        const f32x4 v = {acc[i][j][qd * 4], acc[i][j][qd * 4 + 1], acc[i][j][qd * 4 + 2], acc[i][j][qd * 4 + 3]};
+                        red[((i * FN + j) * 4 + qd) * 64] = v;
                     }
-                }
-            }
-            *reinterpret_cast<u32x4*>(dst) = v;
+        }
+        __syncthreads();
+        if (ks == 0) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int qd = 0; qd < 4; ++qd) {
+                        const f32x4 v = red[((i * FN + j) * 4 + qd) * 64];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[i][j][qd * 4 + e] += v[e];
+                    }
         }
         __syncthreads();
     }
+    store_tile<G, CF32>(acc, lds, g, m0, n0, wm, wn, c32, gh, ks == 0);
 }
 
 __global__ void sum_slices(const float* part, void* dst, int nparts, int64_t part_stride, int M, int N, int64_t ldc, int beta,
@@ -258,6 +483,24 @@ void launch_form(bool tA, bool tB, const GemmArgs& g, dim3 grid, hipStream_t st)
     if (!tA && tB) hipLaunchKernelGGL((gemm_bf16<G, false, true, CF32>), grid, dim3(G::NTHR), 0, st, g);
     if (tA && !tB) hipLaunchKernelGGL((gemm_bf16<G, true, false, CF32>), grid, dim3(G::NTHR), 0, st, g);
     if (tA && tB) hipLaunchKernelGGL((gemm_bf16<G, true, true, CF32>), grid, dim3(G::NTHR), 0, st, g);
+}
+template <typename G, bool CF32, int NS>
+void launch_ring_form(bool tA, bool tB, const GemmArgs& g, dim3 grid, hipStream_t st) {
+    if (!tA && !tB) hipLaunchKernelGGL((gemm_ring<G, false, false, CF32, NS>), grid, dim3(G::NTHR), 0, st, g);
+    if (!tA && tB) hipLaunchKernelGGL((gemm_ring<G, false, true, CF32, NS>), grid, dim3(G::NTHR), 0, st, g);
+    if (tA && !tB) hipLaunchKernelGGL((gemm_ring<G, true, false, CF32, NS>), grid, dim3(G::NTHR), 0, st, g);
+    if (tA && tB) hipLaunchKernelGGL((gemm_ring<G, true, true, CF32, NS>), grid, dim3(G::NTHR), 0, st, g);
+}
+template <typename G, int NS>
+void launch_ring(bool tA, bool tB, GemmArgs g, int S, bool c_f32, hipStream_t st) {
+    g.tiles_m = (g.M + G::BM - 1) / G::BM;
+    g.tiles_n = (g.N + G::BN - 1) / G::BN;
+    const unsigned gx = static_cast<unsigned>((g.tiles_m * g.tiles_n + 7) / 8 * 8);
+    if (c_f32)
+        launch_ring_form<G, true, NS>(tA, tB, g, dim3(gx, 1, static_cast<unsigned>(S)), st);
+    else
+        launch_ring_form<G, false, NS>(tA, tB, g, dim3(gx, 1, static_cast<unsigned>(S)), st);
+    hip_check(hipGetLastError(), "gemm_ring launch");
 }
 template <typename G>
 void launch_geo(bool tA, bool tB, GemmArgs g, int S, bool c_f32, hipStream_t st) {
@@ -296,9 +539,14 @@ bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB,
     g.lda = lda, g.ldb = ldb, g.ldc = ldc;
     g.beta = beta != 0.0f;
     g.tiles_m = g.tiles_n = 0;
-    // Large tiles where the output alone gives every CU a 256 x 256 tile (and then some); small tiles otherwise.
+    // Which tiles (measured on the Linear shapes of a d = 512 block and of a 32000-word tied head). 256 x 256 where
+    // the output gives nearly every CU a tile of its own and the contraction is long enough to pay for the larger
+    // prologue, or where there are tiles for two rounds; 128 x 128 otherwise, two workgroups per CU -- except that an
+    // output of at most one such tile per CU with a long contraction takes the two-set form with a deep ring, since
+    // no second workgroup would come to share the CU.
     const int64_t tiles_large = ((M + 255) / 256) * ((N + 255) / 256);
-    const bool large = g_force_geo >= 0 ? g_force_geo == 1 : tiles_large >= 240;
+    const bool large = g_force_geo >= 0 ? (g_force_geo == 1 || g_force_geo == 8)
+                                        : tiles_large >= 240 && (K >= 1024 || tiles_large >= 512);
     const int64_t ntiles = large ? tiles_large : ((M + 127) / 128) * ((N + 127) / 128);
     // Split the contraction when the tiles alone would leave most of the chip idle and the contraction is long.
     int S = 1;
@@ -306,13 +554,32 @@ bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB,
         S = static_cast<int>(std::min<int64_t>({(512 + ntiles - 1) / ntiles, K / 256, 32}));
         if (S < 1) S = 1;
     }
+    // the ring kernels keep offsets and extents in 32 bits
+    const int64_t ext_a = (tA ? K : M) * lda * 2, ext_b = (tB ? N : K) * ldb * 2;
+    const bool ring_ok = ext_a < (int64_t{1} << 31) && ext_b < (int64_t{1} << 31) && lda < (1 << 21) && ldb < (1 << 21);
+    int ring = 0;  // 0: gemm_bf16 (register-staged tiles); otherwise a gemm_ring form
+    if (ring_ok && g_force_geo >= 5) ring = g_force_geo;
+    if (ring_ok && g_force_geo < 0) ring = large ? 8 : (S == 1 && ntiles <= 256 && K >= 1024) ? 11 : 6;
+    auto run = [&](const GemmArgs& ga, int splits, bool f32) {
+        switch (ring) {
+            case 5: launch_ring<GeoSmall, 4>(tA, tB, ga, splits, f32, st); break;
+            case 6: launch_ring<GeoSmall, 2>(tA, tB, ga, splits, f32, st); break;
+            case 7: launch_ring<GeoSmall, 3>(tA, tB, ga, splits, f32, st); break;
+            case 8: launch_ring<GeoLarge, 2>(tA, tB, ga, splits, f32, st); break;
+            case 9: launch_ring<GeoSmallK2, 2>(tA, tB, ga, splits, f32, st); break;
+            case 10: launch_ring<GeoSmallK2, 3>(tA, tB, ga, splits, f32, st); break;
+            case 11: launch_ring<GeoSmallK2, 4>(tA, tB, ga, splits, f32, st); break;
+            default:
+                if (large)
+                    launch_geo<GeoLarge>(tA, tB, ga, splits, f32, st);
+                else
+                    launch_geo<GeoSmall>(tA, tB, ga, splits, f32, st);
+        }
+    };
     if (S == 1) {
         g.k_per_split = g.K;
         g.part_stride = 0;
-        if (large)
-            launch_geo<GeoLarge>(tA, tB, g, 1, c_dtype == PK_F32, st);
-        else
-            launch_geo<GeoSmall>(tA, tB, g, 1, c_dtype == PK_F32, st);
+        run(g, 1, c_dtype == PK_F32);
         return true;
     }
     const int kps = static_cast<int>(((K + S - 1) / S + BK - 1) / BK * BK);
@@ -324,10 +591,7 @@ bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB,
     gp.beta = 0;
     gp.k_per_split = kps;
     gp.part_stride = M * N;
-    if (large)
-        launch_geo<GeoLarge>(tA, tB, gp, S, true, st);
-    else
-        launch_geo<GeoSmall>(tA, tB, gp, S, true, st);
+    run(gp, S, true);
     const int64_t n4 = M * N / 4;
     hipLaunchKernelGGL(sum_slices, dim3(static_cast<unsigned>(std::min<int64_t>((n4 + 255) / 256, 4096))), dim3(256), 0, st,
                        static_cast<const float*>(part.p), c, S, M * N, static_cast<int>(M), static_cast<int>(N), ldc,

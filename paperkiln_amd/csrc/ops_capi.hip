@@ -168,7 +168,7 @@ int pk_op_sumsq(const float* g, int64_t n, double* host_out, void* stream) {
 int pk_set_gemm_backend(int hand_written) {
     const int before = gemm_backend();
     set_gemm_backend(hand_written <= 0 ? 0 : hand_written == 1 ? 1 : 2);
-    gemm_mfma_force_tiles(hand_written == 3 ? 0 : hand_written == 4 ? 1 : -1);
+    gemm_mfma_force_tiles(hand_written == 3 ? 0 : hand_written == 4 ? 1 : hand_written >= 5 ? hand_written : -1);
     return before;
 }
 int pk_op_gemm(const void* a, int trans_a, const void* b, int trans_b, void* c, int64_t m, int64_t n, int64_t k,
