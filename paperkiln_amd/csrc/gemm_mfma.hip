@@ -241,70 +241,106 @@ __global__ __launch_bounds__(G::NTHR, 2) void gemm_bf16(GemmArgs g) {
 
 // ---- the same tiles fed through a ring of LDS slots ---------------------------------------------------------------
 // With one workgroup per CU (an output of 256 tiles or fewer, or tiles whose buffers fill the LDS) a slice's global
-// loads have one slice of matrix work to hide behind, 512 clocks against a round trip of 1,500 - 2,000: the loop
-// runs at the memory latency. Here the operand slices go from memory straight into LDS (buffer_load_dwordx4 ... lds:
-// no staging registers, no LDS stores, and a lane outside the matrix writes zeros), into a ring of NS slots, and
-// the loads of slice s + NS - 1 are issued before slice s is multiplied: NS - 1 slices of work per round trip. The
-// LDS layouts and the fragment reads are those of gemm_bf16.
+// loads have one slice of matrix work to hide behind, 512 clocks against a round trip of 1,500 - 2,000, and a loop
+// that spends four scalar instructions per matrix instruction on addresses and branches is bound by instruction
+// issue. Here the operand slices go from memory straight into LDS (buffer_load_dwordx4 ... lds: no staging
+// registers, no LDS stores, a lane outside the buffer writes zeros), into a ring of NS slots; the loads of slice
+// s + NS - 1 are issued before slice s is multiplied; a tile's buffer descriptors are formed once and the position
+// in the contraction is the instruction's scalar offset (which the hardware counts in its range check); the slice
+// loop is unrolled over the ring, so every LDS address is a register formed once plus an immediate.
 //
-// One instruction fills 1 KB of LDS lane after lane, so a lane's place in LDS is fixed and what varies is which 16
-// bytes of memory it fetches: unit u = 64 * instruction + lane of an operand's slice lies at LDS byte 16 u, i.e.
-// row u / UPR, chunk u % UPR of the padded tile; the padding units ask for an address outside the buffer.
+// One load instruction fills 1 KB of LDS lane after lane, so a lane's place in LDS is fixed and what varies is which
+// 16 bytes of memory it fetches. The tiles are therefore not padded but swizzled:
+//   [row][64 k] operand (A of "N", B of "T"), rows of 128 bytes = 8 chunks: chunk c of row r lies at chunk
+//     c ^ ((r & 7) ^ ((r >> 3) & 3)) of its row. The 16 rows a quarter-wavefront reads with one 16-byte row read
+//     then cover all 64 banks once (and any 8 consecutive rows 32 banks once).
+//   [64 k][columns] operand (A of "T", B of "N"), rows of 2 * SPAN bytes: the 64-byte segment s of row r lies at
+//     segment s ^ (r & 3) within its group of four. The 4 rows x 64 bytes a half-wavefront reads with one
+//     transposing read then cover all 64 banks once.
 template <bool TR, int SPAN, int NW>
 struct RingOp {
-    static constexpr int UPR = TR ? (SPAN + 32) / 8 : PITCH_ROW / 8;  // 16-byte units per LDS row
-    static constexpr int DATA = TR ? SPAN / 8 : BK / 8;               // of which hold data
+    static constexpr int CPR = TR ? SPAN / 8 : BK / 8;    // 16-byte chunks per LDS row
     static constexpr int ROWS = TR ? BK : SPAN;
-    static_assert(ROWS * UPR % 64 == 0, "a slice is a whole number of wavefront loads");
-    static constexpr int NI = ROWS * UPR / 64;       // wavefront loads per slice
-    static constexpr int PER = (NI + NW - 1) / NW;   // at most this many per wavefront
+    static constexpr int ROWB = CPR * 16;                 // bytes per LDS row
+    static constexpr int NI = ROWS * CPR / 64;            // wavefront loads per slice
+    static_assert(NI % NW == 0, "every wavefront issues the same number of loads");
+    static constexpr int PER = NI / NW;                   // consecutive 1 KB pieces per wavefront
+    static_assert(PER == 2 || PER == 4, "one m0 value and immediate offsets below 4096 per group");
     static constexpr int BYTES = NI * 1024;
-    // loads wavefront w issues per slice: instructions w, w + NW, ...
-    __device__ static int count(int w) { return (NI - w + NW - 1) / NW; }
+    // the chunk of its LDS row that holds memory chunk c (and vice versa: the map is an involution)
+    __device__ static int swz(int r, int c) { return TR ? c ^ ((r & 3) << 2) : c ^ ((r & 7) ^ ((r >> 3) & 3)); }
 };
-constexpr uint32_t OUTSIDE = 0x80000000u;  // a byte offset no buffer of less than 2 GiB contains
+// Offsets that are outside every buffer these kernels take (operands of less than 1 GiB): a lane offset, and a scalar
+// offset whose sum with any lane offset and immediate still fits 32 bits.
+constexpr uint32_t OUTSIDE = 0x80000000u, PAST_END = 0x40000000u;
+constexpr int BIAS = 4096;                 // descriptors start this far before the tile, so that an offset minus the
+                                           // instruction's immediate (below 4096) never goes negative
 
-// An operand's slice cursor: pointer to the tile's first element of the slice in hand, bytes from there to the end of
-// the operand (the buffer's extent, so rows past the matrix -- and, where the contraction index is the row, rows past
-// the contraction's end -- read as zeros), bytes per slice.
-struct SliceCursor {
-    const char* p;
-    int left, step;
-    __device__ u32x4 rsrc() const {
-        const uint64_t a = reinterpret_cast<uint64_t>(p);
-        const u32x4 r = {static_cast<uint32_t>(a), static_cast<uint32_t>(a >> 32) & 0xffffu, static_cast<uint32_t>(left),
-                         0x00020000u};
-        return r;
-    }
-    __device__ void next() {
-        p += step;
-        left = max(left - step, 0);
-    }
+// Descriptor of an operand's tile: from BIAS bytes before the tile's first element of the contraction range to the
+// operand's end (rows past the matrix, and rows past the contraction's end where the contraction index is the row,
+// read as zeros); `step` bytes per slice.
+struct TileDesc {
+    u32x4 rsrc;
+    int step;
 };
 template <bool TR>
-__device__ inline SliceCursor slice_cursor(const uint16_t* base, int64_t ld, int rc0, int rc_count, int k_begin, int k_end) {
-    SliceCursor c;
+__device__ inline TileDesc tile_desc(const uint16_t* base, int64_t ld, int rc0, int rc_count, int k_begin, int k_end) {
     const int64_t kspan = k_end - k_begin, rcs = rc_count - rc0;
+    const char* p;
+    int64_t left;
+    TileDesc d;
     if (!TR) {  // [row][k]
-        c.p = reinterpret_cast<const char*>(base + static_cast<int64_t>(rc0) * ld + k_begin);
-        c.left = static_cast<int>(((rcs - 1) * ld + kspan) * 2);
-        c.step = BK * 2;
+        p = reinterpret_cast<const char*>(base + static_cast<int64_t>(rc0) * ld + k_begin);
+        left = ((rcs - 1) * ld + kspan) * 2;
+        d.step = BK * 2;
     } else {  // [k][column]
-        c.p = reinterpret_cast<const char*>(base + static_cast<int64_t>(k_begin) * ld + rc0);
-        c.left = static_cast<int>(((kspan - 1) * ld + rcs) * 2);
-        c.step = static_cast<int>(BK * ld * 2);
+        p = reinterpret_cast<const char*>(base + static_cast<int64_t>(k_begin) * ld + rc0);
+        left = ((kspan - 1) * ld + rcs) * 2;
+        d.step = static_cast<int>(BK * ld * 2);
     }
-    return c;
+    const uint64_t a = reinterpret_cast<uint64_t>(p) - BIAS;
+    d.rsrc[0] = static_cast<uint32_t>(a);
+    d.rsrc[1] = static_cast<uint32_t>(a >> 32) & 0xffffu;
+    d.rsrc[2] = static_cast<uint32_t>(left + BIAS);
+    d.rsrc[3] = 0x00020000u;
+    return d;
 }
+// PER consecutive 1 KB pieces of LDS from `lds_byte` on, lane offsets off[j] (already less j KB), scalar offset soff.
 // m0 is set and used inside the one statement; the compiler never keeps a value of its own in m0 across other code.
-__device__ inline void dma16(uint32_t lds_byte, uint32_t voff, u32x4 rsrc) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_byte), "v"(voff), "s"(rsrc)
-                 : "memory");
+template <int PER>
+__device__ inline void dma_group(uint32_t lds_byte, const uint32_t (&off)[PER], u32x4 rsrc, uint32_t soff) {
+    if constexpr (PER == 2)
+        asm volatile(
+            "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+            "buffer_load_dwordx4 %1, %3, %4 offen lds\n\t"
+            "buffer_load_dwordx4 %2, %3, %4 offen offset:1024 lds" ::"s"(lds_byte),
+            "v"(off[0]), "v"(off[1]), "s"(rsrc), "s"(soff)
+            : "memory");
+    else
+        asm volatile(
+            "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+            "buffer_load_dwordx4 %1, %5, %6 offen lds\n\t"
+            "buffer_load_dwordx4 %2, %5, %6 offen offset:1024 lds\n\t"
+            "buffer_load_dwordx4 %3, %5, %6 offen offset:2048 lds\n\t"
+            "buffer_load_dwordx4 %4, %5, %6 offen offset:3072 lds" ::"s"(lds_byte),
+            "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "s"(rsrc), "s"(soff)
+            : "memory");
 }
 template <int N>
 __device__ inline void wait_loads_then_barrier() {
     static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+// lane offsets of a wavefront's loads of one operand's slice; `ktail` > 0 (and a [row][k] operand): the form for the
+// contraction's last, partial slice, whose chunks past the end must not be read (they are the next row's)
+template <typename O, bool TR>
+__device__ inline void lane_offsets(uint32_t (&off)[O::PER], int w, int lane, int64_t ld, int rc0, int rc_count, int ktail) {
+#pragma unroll
+    for (int j = 0; j < O::PER; ++j) {
+        const int u = (w * O::PER + j) * 64 + lane, r = u / O::CPR, c = O::swz(r, u % O::CPR);
+        const bool ok = TR ? rc0 + c * 8 < rc_count : (ktail == 0 || c * 8 < ktail);
+        off[j] = ok ? static_cast<uint32_t>(r) * static_cast<uint32_t>(ld) * 2u + c * 16u + BIAS - j * 1024u : OUTSIDE;
+    }
 }
 
 template <typename G, bool TA, bool TB, bool CF32, int NS>
@@ -312,9 +348,10 @@ __global__ __launch_bounds__(G::NTHR, NS <= 2 ? 2 : 1) void gemm_ring(GemmArgs g
     constexpr int BM = G::BM, BN = G::BN, NTHR = G::NTHR, FM = G::FM, FN = G::FN, NW = NTHR / 64;
     using OA = RingOp<TA, BM, NW>;
     using OB = RingOp<!TB, BN, NW>;
-    constexpr int SLOT = OA::BYTES + OB::BYTES;
+    constexpr int SLOT = OA::BYTES + OB::BYTES, PERTOT = OA::PER + OB::PER;
     static_assert(NS * SLOT <= 160 * 1024, "the ring must fit the LDS");
     static_assert(G::WGM * 32 * (G::BN + 8) * (CF32 ? 4 : 2) <= NS * SLOT, "epilogue strip must fit the ring");
+    static_assert((NS - 2) * PERTOT < 64, "loads in flight must fit the counter");
     __shared__ __attribute__((aligned(1024))) uint8_t lds[NS * SLOT];
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     constexpr int KS = G::KS, NWQ = G::WGM * G::WGN, KPW = BK / 16 / KS;  // k-chunks of a slice per wavefront
@@ -331,57 +368,74 @@ __global__ __launch_bounds__(G::NTHR, NS <= 2 ? 2 : 1) void gemm_ring(GemmArgs g
     const int k_begin = blockIdx.z * g.k_per_split, k_end = min(g.K, k_begin + g.k_per_split);
     const int nslices = (k_end - k_begin + BK - 1) / BK, ktail = (k_end - k_begin) % BK;
 
-    // what this lane fetches with its j-th load of a slice; in the contraction's last, partial slice of a [row][k]
-    // operand the chunks past the end must not be read (they are the next row's, or another split's)
     uint32_t offa[OA::PER], offb[OB::PER], offa_t[OA::PER], offb_t[OB::PER];
-#pragma unroll
-    for (int j = 0; j < OA::PER; ++j) {
-        const int u = (j * NW + w) * 64 + lane, row = u / OA::UPR, ch = u % OA::UPR;
-        const bool ok = ch < OA::DATA && (!TA || m0 + ch * 8 < g.M);
-        offa[j] = ok ? static_cast<uint32_t>(row) * static_cast<uint32_t>(g.lda) * 2u + ch * 16u : OUTSIDE;
-        offa_t[j] = (TA || ch * 8 < ktail) ? offa[j] : OUTSIDE;
-    }
-#pragma unroll
-    for (int j = 0; j < OB::PER; ++j) {
-        const int u = (j * NW + w) * 64 + lane, row = u / OB::UPR, ch = u % OB::UPR;
-        const bool ok = ch < OB::DATA && (TB || n0 + ch * 8 < g.N);
-        offb[j] = ok ? static_cast<uint32_t>(row) * static_cast<uint32_t>(g.ldb) * 2u + ch * 16u : OUTSIDE;
-        offb_t[j] = (!TB || ch * 8 < ktail) ? offb[j] : OUTSIDE;
-    }
-    SliceCursor ca = slice_cursor<TA>(g.a, g.lda, m0, g.M, k_begin, k_end);
-    SliceCursor cb = slice_cursor<!TB>(g.b, g.ldb, n0, g.N, k_begin, k_end);
+    lane_offsets<OA, TA>(offa, w, lane, g.lda, m0, g.M, 0);
+    lane_offsets<OB, !TB>(offb, w, lane, g.ldb, n0, g.N, 0);
+    lane_offsets<OA, TA>(offa_t, w, lane, g.lda, m0, g.M, ktail);
+    lane_offsets<OB, !TB>(offb_t, w, lane, g.ldb, n0, g.N, ktail);
+    const TileDesc da = tile_desc<TA>(g.a, g.lda, m0, g.M, k_begin, k_end);
+    const TileDesc db = tile_desc<!TB>(g.b, g.ldb, n0, g.N, k_begin, k_end);
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
-    const int na = OA::count(w), nb = OB::count(w);
+    const uint32_t dst_a = lds0 + w * OA::PER * 1024u, dst_b = lds0 + OA::BYTES + w * OB::PER * 1024u;
 
-    // slices are asked for in order, one call per slice, also past the last one (nothing is fetched then, the
-    // lanes write zeros into a slot nobody reads: every wavefront's count of loads in flight stays the same)
+    // Slices are asked for in order, one call per slice, also past the last one: a wavefront's count of loads in
+    // flight stays the same, and past the end the scalar offset is outside every buffer, so nothing is fetched (the
+    // lanes write zeros into a slot nobody reads).
     int f_slice = 0;
+    uint32_t soff_a = 0, soff_b = 0;
     auto fetch = [&](int slot) {
-        const bool none = f_slice >= nslices, tail = ktail != 0 && f_slice == nslices - 1;
-        SliceCursor xa = ca, xb = cb;
-        if (none) xa.left = xb.left = 0;
-        const u32x4 ra = xa.rsrc(), rb = xb.rsrc();
-        const uint32_t base = lds0 + static_cast<uint32_t>(slot) * SLOT;
-#pragma unroll
-        for (int j = 0; j < OA::PER; ++j)
-            if (j < na) dma16(base + (j * NW + w) * 1024u, tail ? offa_t[j] : offa[j], ra);
-#pragma unroll
-        for (int j = 0; j < OB::PER; ++j)
-            if (j < nb) dma16(base + OA::BYTES + (j * NW + w) * 1024u, tail ? offb_t[j] : offb[j], rb);
-        ca.next();
-        cb.next();
+        const bool none = f_slice >= nslices;
+        const uint32_t sa = none ? PAST_END : soff_a, sb = none ? PAST_END : soff_b;
+        const uint32_t la = dst_a + static_cast<uint32_t>(slot) * SLOT, lb = dst_b + static_cast<uint32_t>(slot) * SLOT;
+        if (ktail != 0 && f_slice == nslices - 1) {
+            dma_group<OA::PER>(la, offa_t, da.rsrc, sa);
+            dma_group<OB::PER>(lb, offb_t, db.rsrc, sb);
+        } else {
+            dma_group<OA::PER>(la, offa, da.rsrc, sa);
+            dma_group<OB::PER>(lb, offb, db.rsrc, sb);
+        }
+        soff_a += da.step;
+        soff_b += db.step;
         ++f_slice;
     };
-    // waits until this wavefront's loads of the oldest slice in flight have landed, then for everybody's
-    constexpr int CMAX = OA::PER + OB::PER;
-    const int cnt = na + nb;
-    auto landed = [&]() {
-        if (cnt == CMAX)
-            wait_loads_then_barrier<(NS - 2) * CMAX>();
-        else if (cnt == CMAX - 1)
-            wait_loads_then_barrier<(NS - 2) * (CMAX - 1)>();
-        else
-            wait_loads_then_barrier<(NS - 2) * (CMAX - 2)>();
+
+    // Lane parts of the fragment reads. [row][k]: row c32 of a 32-row block, chunk 2 kk + gh, one address per kk
+    // (the swizzle is an exclusive-or with a lane value, so kk cannot be an immediate); [k][column]: rows
+    // 8 gh + j / 4 (+ 4), columns 16 u + 4 (j % 4) of 32-column block b, one address per block the wavefront reads.
+    const int tj = lane & 15, tu = (lane >> 4) & 1;
+    uint32_t ra_row[BK / 16], rb_row[BK / 16], ra_tr[FM], rb_tr[FN];
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+        const uint32_t v = static_cast<uint32_t>(c32 * 128 + (RingOp<false, 128, 4>::swz(c32, 2 * kk + gh)) * 16);
+        ra_row[kk] = v;
+        rb_row[kk] = v;
+    }
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        const int blk = wm * FM + i, r = 8 * gh + (tj >> 2);
+        ra_tr[i] = static_cast<uint32_t>(r * OA::ROWB + (((blk & ~3) | ((blk & 3) ^ (r & 3))) * 32 + 16 * tu + 4 * (tj & 3)) * 2);
+    }
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+        const int blk = wn * FN + j, r = 8 * gh + (tj >> 2);
+        rb_tr[j] = static_cast<uint32_t>(r * OB::ROWB + (((blk & ~3) | ((blk & 3) ^ (r & 3))) * 32 + 16 * tu + 4 * (tj & 3)) * 2);
+    }
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    auto read_a = [&](const uint8_t* As, int i, int kk) -> bf16x8 {
+        if (!TA) return lds_read8(reinterpret_cast<const uint16_t*>(As + ra_row[kk] + (wm * FM + i) * 32 * 128));
+        const uint8_t* p = As + ra_tr[i] + kk * 16 * OA::ROWB;
+        const s16x4 lo = lds_read_tr4(reinterpret_cast<const uint16_t*>(p));
+        const s16x4 hi = lds_read_tr4(reinterpret_cast<const uint16_t*>(p + 4 * OA::ROWB));
+        const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        return *reinterpret_cast<const bf16x8*>(&v);
+    };
+    auto read_b = [&](const uint8_t* Bs, int j, int kk) -> bf16x8 {
+        if (TB) return lds_read8(reinterpret_cast<const uint16_t*>(Bs + rb_row[kk] + (wn * FN + j) * 32 * 128));
+        const uint8_t* p = Bs + rb_tr[j] + kk * 16 * OB::ROWB;
+        const s16x4 lo = lds_read_tr4(reinterpret_cast<const uint16_t*>(p));
+        const s16x4 hi = lds_read_tr4(reinterpret_cast<const uint16_t*>(p + 4 * OB::ROWB));
+        const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        return *reinterpret_cast<const bf16x8*>(&v);
     };
 
     f32x16 acc[FM][FN];
@@ -394,31 +448,30 @@ __global__ __launch_bounds__(G::NTHR, NS <= 2 ? 2 : 1) void gemm_ring(GemmArgs g
 
 #pragma unroll
     for (int s = 0; s < NS - 1; ++s) fetch(s);
-    int slot = 0, fslot = NS - 1;
-    for (int s = 0; s < nslices; ++s) {
-        landed();      // slice s is in its slot, and slice s - 1 has been read by every wavefront
-        fetch(fslot);  // slice s + NS - 1 into the slot slice s - 1 leaves
-        const uint16_t* As = reinterpret_cast<const uint16_t*>(lds + slot * SLOT);
-        const uint16_t* Bs = reinterpret_cast<const uint16_t*>(lds + slot * SLOT + OA::BYTES);
+    // slice s lives in slot s % NS: the loop is unrolled over the ring so that slots are constants
+    for (int s0 = 0; s0 < nslices; s0 += NS) {
 #pragma unroll
-        for (int kq = 0; kq < KPW; ++kq) {
-            const int kk = ks * KPW + kq;
-            bf16x8 fa[FM], fb[FN];
+        for (int u = 0; u < NS; ++u) {
+            if (s0 + u < nslices) {  // wavefront-uniform
+                wait_loads_then_barrier<(NS - 2) * PERTOT>();  // slice s is in its slot, slice s - 1 has been read by all
+                fetch((u + NS - 1) % NS);                      // slice s + NS - 1 into the slot slice s - 1 leaves
+                const uint8_t* As = lds + u * SLOT;
+                const uint8_t* Bs = As + OA::BYTES;
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
-                fa[i] = TA ? read_tr_nat(As, G::PITCH_TR_A, kk * 16, (wm * FM + i) * 32, lane)
-                           : lds_read8(As + ((wm * FM + i) * 32 + c32) * PITCH_ROW + kk * 16 + gh * 8);
+                for (int kq = 0; kq < KPW; ++kq) {
+                    const int kk = ks * KPW + kq;
+                    bf16x8 fa[FM], fb[FN];
 #pragma unroll
-            for (int j = 0; j < FN; ++j)
-                fb[j] = !TB ? read_tr_nat(Bs, G::PITCH_TR_B, kk * 16, (wn * FN + j) * 32, lane)
-                            : lds_read8(Bs + ((wn * FN + j) * 32 + c32) * PITCH_ROW + kk * 16 + gh * 8);
+                    for (int i = 0; i < FM; ++i) fa[i] = read_a(As, i, kk);
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
+                    for (int j = 0; j < FN; ++j) fb[j] = read_b(Bs, j, kk);
 #pragma unroll
-                for (int j = 0; j < FN; ++j) acc[i][j] = mfma32(fb[j], fa[i], acc[i][j]);
+                    for (int i = 0; i < FM; ++i)
+#pragma unroll
+                        for (int j = 0; j < FN; ++j) acc[i][j] = mfma32(fb[j], fa[i], acc[i][j]);
+                }
+            }
         }
-        slot = slot + 1 == NS ? 0 : slot + 1;
-        fslot = fslot + 1 == NS ? 0 : fslot + 1;
     }
     wait_loads_then_barrier<0>();  // the zero-filling loads past the end have landed too: the ring is free
     if (KS == 2) {  // set 1 hands its sums to set 0: [wavefront][16-byte group of the 64 registers][lane]
@@ -556,10 +609,11 @@ bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB,
     }
     // the ring kernels keep offsets and extents in 32 bits
     const int64_t ext_a = (tA ? K : M) * lda * 2, ext_b = (tB ? N : K) * ldb * 2;
-    const bool ring_ok = ext_a < (int64_t{1} << 31) && ext_b < (int64_t{1} << 31) && lda < (1 << 21) && ldb < (1 << 21);
+    const int64_t ext_max = (int64_t{1} << 30) - 8192;
+    const bool ring_ok = ext_a < ext_max && ext_b < ext_max && lda < (1 << 21) && ldb < (1 << 21);
     int ring = 0;  // 0: gemm_bf16 (register-staged tiles); otherwise a gemm_ring form
     if (ring_ok && g_force_geo >= 5) ring = g_force_geo;
-    if (ring_ok && g_force_geo < 0) ring = large ? 8 : (S == 1 && ntiles <= 256 && K >= 1024) ? 11 : 6;
+    if (ring_ok && g_force_geo < 0) ring = large ? 8 : S > 1 ? 9 : (ntiles <= 256 && K >= 1024) ? 11 : 6;
     auto run = [&](const GemmArgs& ga, int splits, bool f32) {
         switch (ring) {
             case 5: launch_ring<GeoSmall, 4>(tA, tB, ga, splits, f32, st); break;
