@@ -253,10 +253,13 @@ int pk_op_gemm(const void* a, int trans_a, const void* b, int trans_b, void* c, 
                int dtype, int c_dtype, int accumulate, void* stream);
 /* Which kernel multiplies bf16 operands. 1 (default): every shape class goes to whichever measured faster for it
  * on the MI355X -- this library's own matrix-core GEMM (the counterpart of the reference's tiled kernel,
- * src/cuda_resident.cu:141-171) for short contractions, rocBLAS for long ones and for split weight gradients.
- * 0: rocBLAS for everything, as for fp32 operands. 2: the library's own kernel for everything it takes
- * (16-byte aligned rows, sizes that are multiples of 8); 3 / 4: the same with its 128 x 128 / 256 x 256 tile
- * geometry forced (measurements). Process-wide; returns the previous setting. The environment variable
+ * src/cuda_resident.cu:141-171) for products whose A is not transposed and for transposed-A products with a large
+ * output, rocBLAS for the small-output weight-gradient products. 0: rocBLAS for everything, as for fp32 operands.
+ * 2: the library's own kernel for everything it takes (16-byte aligned rows, sizes that are multiples of 8), in
+ * the form it picks per shape. Measurement settings, all like 2 but with one form forced: 3 / 4 the register-staged
+ * kernel with 128 x 128 / 256 x 256 tiles; 5, 6, 7 the LDS-ring kernel with 128 x 128 tiles and 4, 2, 3 ring slots;
+ * 8 the ring kernel with 256 x 256 tiles; 9, 10, 11 the ring kernel with 128 x 128 tiles shared by two wavefront sets
+ * and 2, 3, 4 slots. Process-wide; returns the previous setting (0, 1 or 2). The environment variable
  * PK_GEMM=library selects 0 at load time. */
 int pk_set_gemm_backend(int mode);
 

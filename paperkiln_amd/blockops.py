@@ -190,8 +190,8 @@ def clip_grad_norm_(grads, max_norm):
 
 def set_gemm_backend(mode: int) -> int:
     """Choose the kernel for bf16 GEMMs (pk_set_gemm_backend): 1 = per shape class whichever measured faster
-    (default), 0 = rocBLAS only, 2 = the library's own matrix-core kernel wherever it applies, 3 / 4 = the same
-    with small / large tiles forced. Returns the previous setting."""
+    (default), 0 = rocBLAS only, 2 = the library's own matrix-core kernel wherever it applies, 3 .. 11 = the same
+    with one kernel form forced (measurements; see include/paperkiln_amd.h). Returns the previous setting (0, 1, 2)."""
     return int(_lib.lib().pk_set_gemm_backend(int(mode)))
 
 

@@ -62,6 +62,7 @@ struct GemmArgs {
     int k_per_split;  // contraction elements per blockIdx.z (a multiple of BK); K when not split
     int64_t part_stride;  // elements between the fp32 partial results of two slices (split only)
     int tiles_m, tiles_n;
+    int splits;  // slices of the contraction (gemm_ring walks them itself; gemm_bf16 takes them from blockIdx.z)
 };
 
 // Transposing operand read in natural k order: lane (c32, g) receives rows row0 + 8g .. 8g + 7 of column
@@ -331,85 +332,175 @@ __device__ inline void wait_loads_then_barrier() {
     static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
 }
-// lane offsets of a wavefront's loads of one operand's slice; `ktail` > 0 (and a [row][k] operand): the form for the
-// contraction's last, partial slice, whose chunks past the end must not be read (they are the next row's)
+// lane offsets of a wavefront's loads of one operand's slice, for a tile in the matrix's interior (every column there,
+// every slice whole)
+template <typename O>
+__device__ inline void lane_offsets(uint32_t (&off)[O::PER], int w, int lane, int64_t ld) {
+#pragma unroll
+    for (int j = 0; j < O::PER; ++j) {
+        const int u = (w * O::PER + j) * 64 + lane, r = u / O::CPR, c = O::swz(r, u % O::CPR);
+        off[j] = static_cast<uint32_t>(r) * static_cast<uint32_t>(ld) * 2u + c * 16u + BIAS - j * 1024u;
+    }
+}
+// ... and with the chunks that must not be read sent outside the buffer: columns past the matrix's edge of a
+// [k][column] operand (every slice of an edge tile), chunks past the contraction's end in the last, partial slice of
+// a [row][k] operand (they are the next row's)
 template <typename O, bool TR>
-__device__ inline void lane_offsets(uint32_t (&off)[O::PER], int w, int lane, int64_t ld, int rc0, int rc_count, int ktail) {
+__device__ inline void lane_offsets_masked(uint32_t (&off)[O::PER], const uint32_t (&whole)[O::PER], int w, int lane, int rc0,
+                                           int rc_count, int ktail) {
 #pragma unroll
     for (int j = 0; j < O::PER; ++j) {
         const int u = (w * O::PER + j) * 64 + lane, r = u / O::CPR, c = O::swz(r, u % O::CPR);
         const bool ok = TR ? rc0 + c * 8 < rc_count : (ktail == 0 || c * 8 < ktail);
-        off[j] = ok ? static_cast<uint32_t>(r) * static_cast<uint32_t>(ld) * 2u + c * 16u + BIAS - j * 1024u : OUTSIDE;
+        off[j] = ok ? whole[j] : OUTSIDE;
     }
 }
+__device__ inline void store16(u32x4 v, uint32_t off, u32x4 rsrc, uint32_t soff) {
+    // invisible to the compiler's count of memory operations in flight, like the loads above; the data registers
+    // may be overwritten by the very next instruction, which a 16-byte store does not allow: one idle state
+    asm volatile("buffer_store_dwordx4 %0, %1, %2, %3 offen\n\ts_nop 0" ::"v"(v), "v"(off), "s"(rsrc), "s"(soff) : "memory");
+}
+template <int N>
+__device__ inline void wait_loads() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ inline void barrier() { asm volatile("s_barrier" ::: "memory"); }
 
+// What a workgroup stores per tile, for the count of memory operations in flight: FM strips of all WGM * 32 rows
+// (bf16) or FM * WGM strips of 32 rows (fp32, whose wider rows would not fit a ring slot otherwise), each
+// rows * chunks-per-row / threads stores per thread.
+template <typename G, bool CF32>
+struct TileStore {
+    static constexpr int EPC = CF32 ? 4 : 8;  // elements per 16-byte chunk
+    static constexpr int CPR = G::BN / EPC;   // chunks per strip row
+    static constexpr int SR = CF32 ? 32 : G::WGM * 32;
+    static constexpr int PHASES = CF32 ? G::FM * G::WGM : G::FM;
+    static_assert(SR * CPR % G::NTHR == 0 && G::NTHR % CPR == 0, "whole stores per thread, one chunk column per thread");
+    static constexpr int PER_PHASE = SR * CPR / G::NTHR;
+    static constexpr int NST = PHASES * PER_PHASE;
+    static constexpr int CP = G::BN + EPC;  // strip pitch in elements: rows stay 16-byte aligned, writes conflict-free
+    static constexpr int BYTES = SR * CP * (CF32 ? 4 : 2);
+};
+
+// C = op(A) op(B), persistent: gridDim.x workgroups walk the virtual blocks v = blockIdx.x, + gridDim.x, ...
+// (virtual block -> (contraction slice, tile) as gemm_bf16 maps (blockIdx.z, blockIdx.x), XCD by XCD), and the ring
+// runs on across tile boundaries: the first slices of the next tile are on their way while the last ones of this tile
+// are multiplied and its result is stored, so a tile's first round trip to memory is paid once per workgroup.
 template <typename G, bool TA, bool TB, bool CF32, int NS>
-__global__ __launch_bounds__(G::NTHR, NS <= 2 ? 2 : 1) void gemm_ring(GemmArgs g) {
+__global__ __launch_bounds__(G::NTHR, NS * (RingOp<TA, G::BM, G::NTHR / 64>::BYTES + RingOp<!TB, G::BN, G::NTHR / 64>::BYTES) <= 80 * 1024 ? 2 : 1)
+void gemm_ring(GemmArgs g) {
     constexpr int BM = G::BM, BN = G::BN, NTHR = G::NTHR, FM = G::FM, FN = G::FN, NW = NTHR / 64;
     using OA = RingOp<TA, BM, NW>;
     using OB = RingOp<!TB, BN, NW>;
+    using ST = TileStore<G, CF32>;
     constexpr int SLOT = OA::BYTES + OB::BYTES, PERTOT = OA::PER + OB::PER;
-    static_assert(NS * SLOT <= 160 * 1024, "the ring must fit the LDS");
-    static_assert(G::WGM * 32 * (G::BN + 8) * (CF32 ? 4 : 2) <= NS * SLOT, "epilogue strip must fit the ring");
-    static_assert((NS - 2) * PERTOT < 64, "loads in flight must fit the counter");
+    static_assert(NS >= 2 && NS * SLOT <= 160 * 1024, "the ring must fit the LDS");
+    static_assert(ST::BYTES <= SLOT, "an epilogue strip must fit one ring slot");
+    static_assert((NS - 2) * PERTOT + ST::NST < 64, "memory operations in flight must fit the counter");
     __shared__ __attribute__((aligned(1024))) uint8_t lds[NS * SLOT];
     const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     constexpr int KS = G::KS, NWQ = G::WGM * G::WGN, KPW = BK / 16 / KS;  // k-chunks of a slice per wavefront
     static_assert(KS == 1 || KS == 2, "one or two wavefront sets");
-    static_assert(KS == 1 || NWQ * 64 * FM * FN * 64 <= NS * SLOT, "the second set's accumulators pass through the ring");
+    static_assert(KS == 1 || (FM % 2 == 0 && NWQ * 64 * (FM / 2) * FN * 64 <= SLOT), "half of the second set's sums per slot");
     const int ks = w / NWQ, wq = w - ks * NWQ;
     const int c32 = lane & 31, gh = lane >> 5, wm = wq / G::WGN, wn = wq % G::WGN;
 
-    const int ntiles = g.tiles_m * g.tiles_n;
-    const int per_xcd = (ntiles + 7) / 8;
-    const int t = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (t >= ntiles) return;
-    const int m0 = (t / g.tiles_n) * BM, n0 = (t % g.tiles_n) * BN;
-    const int k_begin = blockIdx.z * g.k_per_split, k_end = min(g.K, k_begin + g.k_per_split);
-    const int nslices = (k_end - k_begin + BK - 1) / BK, ktail = (k_end - k_begin) % BK;
+    // virtual blocks
+    const int ntiles = g.tiles_m * g.tiles_n, per_xcd = (ntiles + 7) / 8, xpad = per_xcd * 8, V = xpad * g.splits;
+    const int stride = static_cast<int>(gridDim.x);
+    struct Block {
+        int m0, n0, k_begin, k_end, z;
+    };
+    auto next_block = [&](int v, Block& bl) {  // first virtual block at or after v (in steps of the grid) that is a tile
+        for (; v < V; v += stride) {
+            const int z = v / xpad, x = v - z * xpad, t = (x & 7) * per_xcd + (x >> 3);
+            if (t >= ntiles) continue;
+            bl.m0 = (t / g.tiles_n) * BM;
+            bl.n0 = (t % g.tiles_n) * BN;
+            bl.z = z;
+            bl.k_begin = z * g.k_per_split;
+            bl.k_end = min(g.K, bl.k_begin + g.k_per_split);
+            return v;
+        }
+        return V;
+    };
 
-    uint32_t offa[OA::PER], offb[OB::PER], offa_t[OA::PER], offb_t[OB::PER];
-    lane_offsets<OA, TA>(offa, w, lane, g.lda, m0, g.M, 0);
-    lane_offsets<OB, !TB>(offb, w, lane, g.ldb, n0, g.N, 0);
-    lane_offsets<OA, TA>(offa_t, w, lane, g.lda, m0, g.M, ktail);
-    lane_offsets<OB, !TB>(offb_t, w, lane, g.ldb, n0, g.N, ktail);
-    const TileDesc da = tile_desc<TA>(g.a, g.lda, m0, g.M, k_begin, k_end);
-    const TileDesc db = tile_desc<!TB>(g.b, g.ldb, n0, g.N, k_begin, k_end);
+    // ---- fetch side: a stream of slices, tile after tile ----
+    uint32_t offa[OA::PER], offb[OB::PER], offa_c[OA::PER], offb_c[OB::PER];
+    lane_offsets<OA>(offa, w, lane, g.lda);
+    lane_offsets<OB>(offb, w, lane, g.ldb);
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
     const uint32_t dst_a = lds0 + w * OA::PER * 1024u, dst_b = lds0 + OA::BYTES + w * OB::PER * 1024u;
-
-    // Slices are asked for in order, one call per slice, also past the last one: a wavefront's count of loads in
-    // flight stays the same, and past the end the scalar offset is outside every buffer, so nothing is fetched (the
-    // lanes write zeros into a slot nobody reads).
-    int f_slice = 0;
+    Block fb;
+    int fv = next_block(static_cast<int>(blockIdx.x), fb);
+    if (fv >= V) return;  // nothing for this workgroup (before any barrier)
+    TileDesc da, db;
+    int f_slice = 0, f_nslices = 0, f_ktail = 0;
     uint32_t soff_a = 0, soff_b = 0;
+    auto open = [&]() {  // the fetch stream enters virtual block fv
+        f_slice = 0;
+        soff_a = soff_b = 0;
+        if (fv >= V) {  // past the last block: descriptors stay, every offset goes outside
+            f_nslices = 0;
+            return;
+        }
+        f_nslices = (fb.k_end - fb.k_begin + BK - 1) / BK;
+        f_ktail = (fb.k_end - fb.k_begin) % BK;
+        da = tile_desc<TA>(g.a, g.lda, fb.m0, g.M, fb.k_begin, fb.k_end);
+        db = tile_desc<!TB>(g.b, g.ldb, fb.n0, g.N, fb.k_begin, fb.k_end);
+        // the masked lane offsets: used by every slice of a [k][column] operand, by the last slice of a [row][k] one
+        if (TA ? fb.m0 + BM > g.M : f_ktail != 0)
+            lane_offsets_masked<OA, TA>(offa_c, offa, w, lane, fb.m0, g.M, f_ktail);
+        else {
+#pragma unroll
+            for (int j = 0; j < OA::PER; ++j) offa_c[j] = offa[j];
+        }
+        if (!TB ? fb.n0 + BN > g.N : f_ktail != 0)
+            lane_offsets_masked<OB, !TB>(offb_c, offb, w, lane, fb.n0, g.N, f_ktail);
+        else {
+#pragma unroll
+            for (int j = 0; j < OB::PER; ++j) offb_c[j] = offb[j];
+        }
+    };
+    // One call per slice of the stream, in order, also past the stream's end: a wavefront's count of loads in flight
+    // stays the same, and the scalar offset is then outside every buffer, so nothing is fetched (the lanes write zeros
+    // into a slot nobody reads).
     auto fetch = [&](int slot) {
-        const bool none = f_slice >= nslices;
+        const bool none = f_nslices == 0;
         const uint32_t sa = none ? PAST_END : soff_a, sb = none ? PAST_END : soff_b;
         const uint32_t la = dst_a + static_cast<uint32_t>(slot) * SLOT, lb = dst_b + static_cast<uint32_t>(slot) * SLOT;
-        if (ktail != 0 && f_slice == nslices - 1) {
-            dma_group<OA::PER>(la, offa_t, da.rsrc, sa);
-            dma_group<OB::PER>(lb, offb_t, db.rsrc, sb);
+        const bool last = f_slice == f_nslices - 1;
+        if ((TA || last) && (!TB || last)) {  // wavefront-uniform
+            dma_group<OA::PER>(la, offa_c, da.rsrc, sa);
+            dma_group<OB::PER>(lb, offb_c, db.rsrc, sb);
+        } else if (TA || last) {
+            dma_group<OA::PER>(la, offa_c, da.rsrc, sa);
+            dma_group<OB::PER>(lb, offb, db.rsrc, sb);
+        } else if (!TB || last) {
+            dma_group<OA::PER>(la, offa, da.rsrc, sa);
+            dma_group<OB::PER>(lb, offb_c, db.rsrc, sb);
         } else {
             dma_group<OA::PER>(la, offa, da.rsrc, sa);
             dma_group<OB::PER>(lb, offb, db.rsrc, sb);
         }
         soff_a += da.step;
         soff_b += db.step;
-        ++f_slice;
+        if (!none && ++f_slice == f_nslices) {
+            fv = next_block(fv + stride, fb);
+            open();
+        }
     };
 
-    // Lane parts of the fragment reads. [row][k]: row c32 of a 32-row block, chunk 2 kk + gh, one address per kk
-    // (the swizzle is an exclusive-or with a lane value, so kk cannot be an immediate); [k][column]: rows
-    // 8 gh + j / 4 (+ 4), columns 16 u + 4 (j % 4) of 32-column block b, one address per block the wavefront reads.
+    // ---- lane parts of the fragment reads ----
+    // [row][k]: row c32 of a 32-row block, chunk 2 kk + gh, one address per kk (the swizzle is an exclusive-or with a
+    // lane value, so kk cannot be an immediate); [k][column]: rows 8 gh + j / 4 (+ 4), columns 16 u + 4 (j % 4) of
+    // 32-column block b, one address per block the wavefront reads.
     const int tj = lane & 15, tu = (lane >> 4) & 1;
-    uint32_t ra_row[BK / 16], rb_row[BK / 16], ra_tr[FM], rb_tr[FN];
+    uint32_t r_row[BK / 16], ra_tr[FM], rb_tr[FN];
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-        const uint32_t v = static_cast<uint32_t>(c32 * 128 + (RingOp<false, 128, 4>::swz(c32, 2 * kk + gh)) * 16);
-        ra_row[kk] = v;
-        rb_row[kk] = v;
-    }
+    for (int kk = 0; kk < BK / 16; ++kk)
+        r_row[kk] = static_cast<uint32_t>(c32 * 128 + (RingOp<false, 128, 4>::swz(c32, 2 * kk + gh)) * 16);
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
         const int blk = wm * FM + i, r = 8 * gh + (tj >> 2);
@@ -421,88 +512,192 @@ __global__ __launch_bounds__(G::NTHR, NS <= 2 ? 2 : 1) void gemm_ring(GemmArgs g
         rb_tr[j] = static_cast<uint32_t>(r * OB::ROWB + (((blk & ~3) | ((blk & 3) ^ (r & 3))) * 32 + 16 * tu + 4 * (tj & 3)) * 2);
     }
     typedef short s16x8 __attribute__((ext_vector_type(8)));
-    auto read_a = [&](const uint8_t* As, int i, int kk) -> bf16x8 {
-        if (!TA) return lds_read8(reinterpret_cast<const uint16_t*>(As + ra_row[kk] + (wm * FM + i) * 32 * 128));
-        const uint8_t* p = As + ra_tr[i] + kk * 16 * OA::ROWB;
+    auto read_tr = [](const uint8_t* p, int rowb) -> bf16x8 {
         const s16x4 lo = lds_read_tr4(reinterpret_cast<const uint16_t*>(p));
-        const s16x4 hi = lds_read_tr4(reinterpret_cast<const uint16_t*>(p + 4 * OA::ROWB));
+        const s16x4 hi = lds_read_tr4(reinterpret_cast<const uint16_t*>(p + 4 * rowb));
         const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         return *reinterpret_cast<const bf16x8*>(&v);
+    };
+    auto read_a = [&](const uint8_t* As, int i, int kk) -> bf16x8 {
+        if (!TA) return lds_read8(reinterpret_cast<const uint16_t*>(As + r_row[kk] + (wm * FM + i) * 32 * 128));
+        return read_tr(As + ra_tr[i] + kk * 16 * OA::ROWB, OA::ROWB);
     };
     auto read_b = [&](const uint8_t* Bs, int j, int kk) -> bf16x8 {
-        if (TB) return lds_read8(reinterpret_cast<const uint16_t*>(Bs + rb_row[kk] + (wn * FN + j) * 32 * 128));
-        const uint8_t* p = Bs + rb_tr[j] + kk * 16 * OB::ROWB;
-        const s16x4 lo = lds_read_tr4(reinterpret_cast<const uint16_t*>(p));
-        const s16x4 hi = lds_read_tr4(reinterpret_cast<const uint16_t*>(p + 4 * OB::ROWB));
-        const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        return *reinterpret_cast<const bf16x8*>(&v);
+        if (TB) return lds_read8(reinterpret_cast<const uint16_t*>(Bs + r_row[kk] + (wn * FN + j) * 32 * 128));
+        return read_tr(Bs + rb_tr[j] + kk * 16 * OB::ROWB, OB::ROWB);
     };
 
-    f32x16 acc[FM][FN];
+    // ---- epilogue: lane parts of the stores (tile-relative), formed once ----
+    typedef typename std::conditional<CF32, float, uint16_t>::type CT;
+    constexpr int ES = CF32 ? 4 : 2;
+    const int st_ch = static_cast<int>(threadIdx.x) % ST::CPR;  // the chunk column this thread stores in every strip
+    uint32_t coff[ST::PER_PHASE];
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    for (int k = 0; k < ST::PER_PHASE; ++k) {
+        const int srow = (static_cast<int>(threadIdx.x) + k * NTHR) / ST::CPR;
+        // bf16 strips hold the i-th 32-row block of every wavefront row: strip row -> tile row (srow / 32) FM 32 + srow % 32
+        const int trow = CF32 ? srow : (srow >> 5) * FM * 32 + (srow & 31);
+        coff[k] = (static_cast<uint32_t>(trow) * static_cast<uint32_t>(g.ldc) + st_ch * ST::EPC) * ES;
+    }
 
+    f32x16 acc[FM][FN];
+    auto zero_acc = [&]() {
 #pragma unroll
-    for (int s = 0; s < NS - 1; ++s) fetch(s);
-    // slice s lives in slot s % NS: the loop is unrolled over the ring so that slots are constants
-    for (int s0 = 0; s0 < nslices; s0 += NS) {
+        for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int u = 0; u < NS; ++u) {
-            if (s0 + u < nslices) {  // wavefront-uniform
-                wait_loads_then_barrier<(NS - 2) * PERTOT>();  // slice s is in its slot, slice s - 1 has been read by all
-                fetch((u + NS - 1) % NS);                      // slice s + NS - 1 into the slot slice s - 1 leaves
-                const uint8_t* As = lds + u * SLOT;
-                const uint8_t* Bs = As + OA::BYTES;
+            for (int j = 0; j < FN; ++j)
 #pragma unroll
-                for (int kq = 0; kq < KPW; ++kq) {
-                    const int kk = ks * KPW + kq;
-                    bf16x8 fa[FM], fb[FN];
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    };
+    // the tile's result, through the ring slot `strip` (which every wavefront has finished reading)
+    auto store_result = [&](uint8_t* strip, const Block& bl) {
+        if (KS == 2) {  // set 1 hands its sums to set 0, half of them at a time: [wavefront][16-byte group][lane]
+            f32x4* red = reinterpret_cast<f32x4*>(strip) + wq * ((FM / 2) * FN * 4) * 64 + lane;
 #pragma unroll
-                    for (int i = 0; i < FM; ++i) fa[i] = read_a(As, i, kk);
+            for (int half = 0; half < 2; ++half) {
+                if (ks == 1) {
 #pragma unroll
-                    for (int j = 0; j < FN; ++j) fb[j] = read_b(Bs, j, kk);
+                    for (int i = 0; i < FM / 2; ++i)
 #pragma unroll
-                    for (int i = 0; i < FM; ++i)
+                        for (int j = 0; j < FN; ++j)
 #pragma unroll
-                        for (int j = 0; j < FN; ++j) acc[i][j] = mfma32(fb[j], fa[i], acc[i][j]);
+                            for (int qd = 0; qd < 4; ++qd) {
+                                const f32x16& a = acc[half * (FM / 2) + i][j];
+                                const f32x4 v = {a[qd * 4], a[qd * 4 + 1], a[qd * 4 + 2], a[qd * 4 + 3]};
+                                red[((i * FN + j) * 4 + qd) * 64] = v;
+                            }
                 }
+                __syncthreads();
+                if (ks == 0) {
+#pragma unroll
+                    for (int i = 0; i < FM / 2; ++i)
+#pragma unroll
+                        for (int j = 0; j < FN; ++j)
+#pragma unroll
+                            for (int qd = 0; qd < 4; ++qd) {
+                                const f32x4 v = red[((i * FN + j) * 4 + qd) * 64];
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) acc[half * (FM / 2) + i][j][qd * 4 + e] += v[e];
+                            }
+                }
+                __syncthreads();
             }
         }
-    }
-    wait_loads_then_barrier<0>();  // the zero-filling loads past the end have landed too: the ring is free
-    if (KS == 2) {  // set 1 hands its sums to set 0: [wavefront][16-byte group of the 64 registers][lane]
-        f32x4* red = reinterpret_cast<f32x4*>(lds) + wq * (FM * FN * 4) * 64 + lane;
-        if (ks == 1) {
+        // descriptor of C from the tile's first element on (rows past the matrix are dropped by the range check,
+        // columns past it by the lane's offset)
+        CT* ctile = static_cast<CT*>(g.c) + (g.part_stride ? static_cast<int64_t>(bl.z) * g.part_stride : 0) +
+                    static_cast<int64_t>(bl.m0) * g.ldc + bl.n0;
+        const int64_t cleft = (static_cast<int64_t>(g.M - bl.m0 - 1) * g.ldc + (g.N - bl.n0)) * ES;
+        const uint32_t crec = cleft > 0x7ffffff0 ? 0x7ffffff0u : static_cast<uint32_t>(cleft);
+        const uint64_t ca = reinterpret_cast<uint64_t>(ctile);
+        const u32x4 crs = {static_cast<uint32_t>(ca), static_cast<uint32_t>(ca >> 32) & 0xffffu, crec, 0x00020000u};
+        const __amdgpu_buffer_rsrc_t crs_b = __builtin_amdgcn_make_buffer_rsrc(ctile, 0, static_cast<int>(crec), 0x00020000);
+        const uint32_t cmask = bl.n0 + st_ch * ST::EPC < g.N ? 0u : OUTSIDE;
+        CT* cs = reinterpret_cast<CT*>(strip);
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
-#pragma unroll
-                for (int j = 0; j < FN; ++j)
-#pragma unroll
-                    for (int qd = 0; qd < 4; ++qd) {
-                        const f32x4 v = {acc[i][j][qd * 4], acc[i][j][qd * 4 + 1], acc[i][j][qd * 4 + 2], acc[i][j][qd * 4 + 3]};
-                        red[((i * FN + j) * 4 + qd) * 64] = v;
-                    }
-        }
-        __syncthreads();
-        if (ks == 0) {
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
+        for (int ph = 0; ph < ST::PHASES; ++ph) {
+            const int i = CF32 ? ph / G::WGM : ph, ws = CF32 ? ph % G::WGM : 0;
+            if (ks == 0 && (!CF32 || wm == ws)) {  // wavefront-uniform: the wavefronts that hold this strip's sums
 #pragma unroll
                 for (int j = 0; j < FN; ++j)
 #pragma unroll
                     for (int qd = 0; qd < 4; ++qd) {
-                        const f32x4 v = red[((i * FN + j) * 4 + qd) * 64];
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) acc[i][j][qd * 4 + e] += v[e];
+                        const int row = (CF32 ? 0 : wm * 32) + c32, col = (wn * FN + j) * 32 + qd * 8 + gh * 4;
+                        if (CF32) {
+                            const f32x4 v = {acc[i][j][qd * 4], acc[i][j][qd * 4 + 1], acc[i][j][qd * 4 + 2], acc[i][j][qd * 4 + 3]};
+                            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(cs) + row * ST::CP + col) = v;
+                        } else {
+                            const u32x2 v = {pack_bf16(acc[i][j][qd * 4], acc[i][j][qd * 4 + 1]),
+                                             pack_bf16(acc[i][j][qd * 4 + 2], acc[i][j][qd * 4 + 3])};
+                            *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(cs) + row * ST::CP + col) = v;
+                        }
                     }
+            }
+            __syncthreads();
+            // rows of C this strip holds start at tile row (ws FM + i) 32 (fp32) or i 32 (bf16, plus the lane's part)
+            const uint32_t soff = static_cast<uint32_t>((CF32 ? ws * FM + i : i) * 32) * static_cast<uint32_t>(g.ldc) * ES;
+#pragma unroll
+            for (int k = 0; k < ST::PER_PHASE; ++k) {
+                const int srow = (static_cast<int>(threadIdx.x) + k * NTHR) / ST::CPR;
+                u32x4 v = *reinterpret_cast<const u32x4*>(cs + srow * ST::CP + st_ch * ST::EPC);
+                const uint32_t off = coff[k] | cmask;
+                if (g.beta) {
+                    const u32x4 old = __builtin_amdgcn_raw_buffer_load_b128(crs_b, static_cast<int>(off), static_cast<int>(soff), 0);
+                    if (CF32) {
+                        f32x4 s = *reinterpret_cast<const f32x4*>(&old) + *reinterpret_cast<const f32x4*>(&v);
+                        v = *reinterpret_cast<const u32x4*>(&s);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float lo = __uint_as_float(old[e] << 16) + __uint_as_float(v[e] << 16);
+                            const float hi = __uint_as_float(old[e] & 0xffff0000u) + __uint_as_float(v[e] & 0xffff0000u);
+                            v[e] = pack_bf16(lo, hi);
+                        }
+                    }
+                }
+                store16(v, off, crs, soff);
+            }
+            __syncthreads();
         }
-        __syncthreads();
+    };
+
+    // ---- the stream ----
+    open();
+    {
+        int slot = 0;
+        for (int s = 0; s < NS - 1; ++s) fetch(slot++);
     }
-    store_tile<G, CF32>(acc, lds, g, m0, n0, wm, wn, c32, gh, ks == 0);
+    Block cb;  // compute side: the block in hand
+    int cv = next_block(static_cast<int>(blockIdx.x), cb);
+    int c_slice = 0, c_nslices = (cb.k_end - cb.k_begin + BK - 1) / BK;
+    int since_store = NS;  // waits since the last tile's stores were issued; below NS - 1 they are still counted
+    zero_acc();
+    for (;;) {
+        bool done = false;
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+            // Slice in hand landed: everything this wavefront issued after that slice's loads may still be in flight
+            // -- the loads of NS - 2 later slices and, for the NS - 1 slices asked for before the last tile's
+            // stores, those stores (memory operations complete in order).
+            if (since_store < NS - 1)
+                wait_loads<(NS - 2) * PERTOT + ST::NST>();
+            else
+                wait_loads<(NS - 2) * PERTOT>();
+            since_store = min(since_store + 1, NS);
+            barrier();                 // ... for every wavefront, and all have read the slice before
+            fetch((u + NS - 1) % NS);  // slice + NS - 1 of the stream into the slot the slice before leaves
+            const uint8_t* As = lds + u * SLOT;
+            const uint8_t* Bs = As + OA::BYTES;
+#pragma unroll
+            for (int kq = 0; kq < KPW; ++kq) {
+                const int kk = ks * KPW + kq;
+                bf16x8 fa[FM], fbb[FN];
+#pragma unroll
+                for (int i = 0; i < FM; ++i) fa[i] = read_a(As, i, kk);
+#pragma unroll
+                for (int j = 0; j < FN; ++j) fbb[j] = read_b(Bs, j, kk);
+#pragma unroll
+                for (int i = 0; i < FM; ++i)
+#pragma unroll
+                    for (int j = 0; j < FN; ++j) acc[i][j] = mfma32(fbb[j], fa[i], acc[i][j]);
+            }
+            if (++c_slice == c_nslices) {  // wavefront-uniform
+                barrier();  // every wavefront has read slot u: it takes the result on its way out
+                store_result(lds + u * SLOT, cb);
+                since_store = 0;
+                cv = next_block(cv + stride, cb);
+                if (cv >= V) {
+                    done = true;
+                    break;
+                }
+                c_slice = 0;
+                c_nslices = (cb.k_end - cb.k_begin + BK - 1) / BK;
+                zero_acc();
+            }
+        }
+        if (done) break;
+    }
+    wait_loads<0>();  // the zero-filling loads past the end write LDS: they must have landed before the workgroup ends
 }
 
 __global__ void sum_slices(const float* part, void* dst, int nparts, int64_t part_stride, int M, int N, int64_t ldc, int beta,
@@ -544,15 +739,31 @@ void launch_ring_form(bool tA, bool tB, const GemmArgs& g, dim3 grid, hipStream_
     if (tA && !tB) hipLaunchKernelGGL((gemm_ring<G, true, false, CF32, NS>), grid, dim3(G::NTHR), 0, st, g);
     if (tA && tB) hipLaunchKernelGGL((gemm_ring<G, true, true, CF32, NS>), grid, dim3(G::NTHR), 0, st, g);
 }
+int cu_count() {
+    static const int n = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            cus <= 0)
+            return 256;
+        return cus;
+    }();
+    return n;
+}
 template <typename G, int NS>
 void launch_ring(bool tA, bool tB, GemmArgs g, int S, bool c_f32, hipStream_t st) {
     g.tiles_m = (g.M + G::BM - 1) / G::BM;
     g.tiles_n = (g.N + G::BN - 1) / G::BN;
-    const unsigned gx = static_cast<unsigned>((g.tiles_m * g.tiles_n + 7) / 8 * 8);
+    g.splits = S;
+    // persistent: as many workgroups as the chip holds at once (a multiple of 8, one XCD's share each), or fewer
+    constexpr int NW = G::NTHR / 64;
+    constexpr int RING = NS * (RingOp<false, G::BM, NW>::BYTES + RingOp<false, G::BN, NW>::BYTES);  // same for every form
+    const int64_t vblocks = static_cast<int64_t>((g.tiles_m * g.tiles_n + 7) / 8 * 8) * S;
+    const int64_t slots = static_cast<int64_t>(cu_count()) / 8 * 8 * (RING <= 80 * 1024 ? 2 : 1);
+    const unsigned gx = static_cast<unsigned>(std::min(vblocks, slots));
     if (c_f32)
-        launch_ring_form<G, true, NS>(tA, tB, g, dim3(gx, 1, static_cast<unsigned>(S)), st);
+        launch_ring_form<G, true, NS>(tA, tB, g, dim3(gx), st);
     else
-        launch_ring_form<G, false, NS>(tA, tB, g, dim3(gx, 1, static_cast<unsigned>(S)), st);
+        launch_ring_form<G, false, NS>(tA, tB, g, dim3(gx), st);
     hip_check(hipGetLastError(), "gemm_ring launch");
 }
 template <typename G>
@@ -592,6 +803,7 @@ bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB,
     g.lda = lda, g.ldb = ldb, g.ldc = ldc;
     g.beta = beta != 0.0f;
     g.tiles_m = g.tiles_n = 0;
+    g.splits = 1;
     // Which tiles (measured on the Linear shapes of a d = 512 block and of a 32000-word tied head). 256 x 256 where
     // the output gives nearly every CU a tile of its own and the contraction is long enough to pay for the larger
     // prologue, or where there are tiles for two rounds; 128 x 128 otherwise, two workgroups per CU -- except that an
@@ -610,7 +822,7 @@ bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB,
     // the ring kernels keep offsets and extents in 32 bits
     const int64_t ext_a = (tA ? K : M) * lda * 2, ext_b = (tB ? N : K) * ldb * 2;
     const int64_t ext_max = (int64_t{1} << 30) - 8192;
-    const bool ring_ok = ext_a < ext_max && ext_b < ext_max && lda < (1 << 21) && ldb < (1 << 21);
+    const bool ring_ok = ext_a < ext_max && ext_b < ext_max && lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 20);
     int ring = 0;  // 0: gemm_bf16 (register-staged tiles); otherwise a gemm_ring form
     if (ring_ok && g_force_geo >= 5) ring = g_force_geo;
     if (ring_ok && g_force_geo < 0) ring = large ? 8 : S > 1 ? 9 : (ntiles <= 256 && K >= 1024) ? 11 : 6;

@@ -268,16 +268,21 @@ def test_allocator_recycles_a_block_behind_the_stream_that_used_it_last(bo):
 
 
 GEMM_SHAPES = [(128, 128, 64), (560, 136, 200), (8, 8, 8), (2056, 520, 1376), (512, 1536, 4096), (264, 40, 8192),
-               (1000, 2048, 512), (300, 264, 72)]
+               (1000, 2048, 512), (300, 264, 72), (8192, 2752, 72), (4096, 4096, 136)]
 
 
-@pytest.mark.parametrize("mode", [3, 4], ids=["tiles128", "tiles256"])
+@pytest.mark.parametrize("mode", [3, 4, 5, 6, 8, 9, 11, 2],
+                         ids=["tiles128", "tiles256", "ring128x4", "ring128x2", "ring256", "ring128_two_sets",
+                              "ring128_two_sets_x4", "by_shape"])
 @pytest.mark.parametrize("shape", GEMM_SHAPES, ids=lambda s: f"M{s[0]}_N{s[1]}_K{s[2]}")
 def test_matrix_core_gemm_against_float64(bo, mode, shape):
     """The library's own bf16 GEMM (the counterpart of the reference's tiled kernel with transpose flags,
-    src/cuda_resident.cu:141-171) in both tile geometries, all four transpose combinations, bf16 and fp32 results,
-    overwrite and accumulate, ragged edges, contractions that are not a multiple of the slice and long ones that are
-    split across workgroups -- against a float64 product of the same bf16 operands. The bar: the fp32 accumulation
+    src/cuda_resident.cu:141-171) in every form it has -- register-staged tiles and the persistent LDS-ring kernel,
+    both tile geometries, ring depths 2 and 4, one and two wavefront sets per tile, and the form the library picks by
+    shape -- all four transpose combinations, bf16 and fp32 results, overwrite and accumulate, ragged edges,
+    contractions that are not a multiple of the slice, long ones that are split across workgroups, and outputs of more
+    tiles than the chip holds workgroups (so that a workgroup walks several tiles with its loads running ahead across
+    the tile boundary) -- against a float64 product of the same bf16 operands. The bar: the fp32 accumulation
     error of a K-term sum (a few 1e-6 relative to the largest |C|, the library kernel's own distance is printed beside
     it), plus one bf16 rounding where the result is stored in bf16. Two runs give the same bits."""
     M, N, K = shape
