@@ -1095,13 +1095,13 @@ void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dty
     if (A.dtype != B.dtype) throw std::runtime_error("gemm: operand dtypes differ");
     // Which kernel: measured per shape on the MI355X as GPU time from a kernel trace (timing launches from the host
     // measures the library's longer host path instead), on the Linear shapes of a d = 512 block and of the tied
-    // head. The hand-written kernel is ahead of or level with the library on the products whose A is not
-    // transposed (activations times weights, gradients times weights: 8 of 10 shapes, the other two within 11 %)
-    // and on a transposed-A product with an output large enough for 256 x 256 tiles without splitting the
-    // contraction (the tied head's dE); the library keeps the small-output weight-gradient products.
+    // head. The hand-written kernel is ahead of the library on 12 of the 15 products and level on one; the
+    // library keeps the class it is ahead in by 5 - 15 %: A and B both with the contraction index contiguous
+    // (gradient times weight), an output of at most one 128 x 128 tile per CU and a contraction of 1024 or more.
     // backend 2 sends everything the hand-written kernel takes to it, backend 0 nothing.
     const int backend = gemm_backend();
-    const bool mine = backend == 2 || (backend == 1 && (!tA || ((M + 255) / 256) * ((N + 255) / 256) >= 240));
+    const bool theirs = !tA && tB && ((M + 127) / 128) * ((N + 127) / 128) <= 256 && Ka >= 1024;
+    const bool mine = backend == 2 || (backend == 1 && !theirs);
     if (A.dtype == PK_BF16 && mine &&
         gemm_mfma_bf16(A.ptr(), tA, lda, B.ptr(), tB, B.cols, C, c_dtype, M, N, Ka, ldc, beta, tape_stream()))
         return;
@@ -1158,19 +1158,23 @@ void gemm_tn_split(const Tensor& A, const Tensor& B, float* const* dst, int nspl
     if (B.rows != K) throw std::runtime_error("gemm: inner dimensions disagree");
     if (nsplit < 1 || nsplit > 4 || W % nsplit != 0) throw std::runtime_error("gemm_tn_split: bad column split");
     if (A.dtype != B.dtype) throw std::runtime_error("gemm: operand dtypes differ");
-    if (A.dtype == PK_BF16 && gemm_backend() == 2) {  // one product [M, W] in fp32, then the column blocks go to their tensors
-        Buffer whole(sizeof(float) * static_cast<size_t>(M) * W);
-        if (gemm_mfma_bf16(A.ptr(), true, M, B.ptr(), false, W, whole.p, PK_F32, M, W, K, W, 0.0f, tape_stream())) {
+    if (A.dtype == PK_BF16 && gemm_backend() != 0) {
+        // the product [M, W] as fp32 partial products over slices of the tokens; the kernel that adds them deals the
+        // column blocks to their tensors (measured ahead of the library's batched form on all four weight-gradient
+        // shapes of a d = 512 block once the slices are one per resident workgroup)
+        std::unique_ptr<Buffer> part;
+        int nparts = 0;
+        if (gemm_mfma_bf16_parts(A.ptr(), true, M, B.ptr(), false, W, M, W, K, tape_stream(), part, nparts)) {
             SplitDst d{};
             for (int k = 0; k < nsplit; ++k) d.p[k] = dst[k];
             bool vec = (W / nsplit) % 4 == 0;
             for (int k = 0; k < nsplit; ++k) vec = vec && aligned16p(dst[k]);
             if (vec)
                 hipLaunchKernelGGL(add_parts_split4, ew_grid(M * W / 4), dim3(NT), 0, tape_stream(),
-                                   static_cast<const float*>(whole.p), d, 1, M, W / nsplit, nsplit, beta);
+                                   static_cast<const float*>(part->p), d, nparts, M, W / nsplit, nsplit, beta);
             else
                 hipLaunchKernelGGL(add_parts_split, ew_grid(M * W), dim3(NT), 0, tape_stream(),
-                                   static_cast<const float*>(whole.p), d, 1, M, W / nsplit, nsplit, beta);
+                                   static_cast<const float*>(part->p), d, nparts, M, W / nsplit, nsplit, beta);
             post();
             return;
         }

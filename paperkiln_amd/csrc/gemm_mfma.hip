@@ -19,6 +19,7 @@
 // into slices that separate workgroups multiply into fp32 partial tiles; the partial tiles are added in slice
 // order by a second kernel -- no atomics, the same bits on every run.
 #include <algorithm>
+#include <memory>
 #include <type_traits>
 
 #include "mfma_common.h"
@@ -786,83 +787,130 @@ int g_force_geo = -1;  // -1: choose by shape; 0 / 1: small / large tiles always
 
 void gemm_mfma_force_tiles(int which) { g_force_geo = which; }
 
-// Returns false, having done nothing, for what the kernel does not take (fp32 operands, unaligned rows, sizes
-// that are not multiples of 8): the caller then uses the library GEMM.
-bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB, int64_t ldb, void* c, int c_dtype,
-                    int64_t M, int64_t N, int64_t K, int64_t ldc, float beta, hipStream_t st) {
-    if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return false;
-    if (beta != 0.0f && beta != 1.0f) return false;
-    if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return false;
-    if (lda % 8 || ldb % 8 || K % 8 || N % 8 || ldc % 8) return false;
-    if (tA && M % 8) return false;  // A^T is read in 16-byte chunks along M
-    GemmArgs g;
-    g.a = static_cast<const uint16_t*>(a);
-    g.b = static_cast<const uint16_t*>(b);
-    g.c = c;
-    g.M = static_cast<int>(M), g.N = static_cast<int>(N), g.K = static_cast<int>(K);
-    g.lda = lda, g.ldb = ldb, g.ldc = ldc;
-    g.beta = beta != 0.0f;
-    g.tiles_m = g.tiles_n = 0;
-    g.splits = 1;
+namespace {
+// How a product is run: tile geometry and kernel form, and into how many slices the contraction is cut.
+struct Plan {
+    bool large;  // 256 x 256 tiles
+    int ring;    // 0: gemm_bf16 (register-staged tiles); otherwise a gemm_ring form (the numbers of pk_set_gemm_backend)
+    int S;       // slices of the contraction, each multiplied into an fp32 partial product of its own
+    int kps;     // contraction elements per slice (a multiple of BK)
+};
+Plan make_plan(bool tA, bool tB, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc) {
+    Plan p;
     // Which tiles (measured on the Linear shapes of a d = 512 block and of a 32000-word tied head). 256 x 256 where
     // the output gives nearly every CU a tile of its own and the contraction is long enough to pay for the larger
     // prologue, or where there are tiles for two rounds; 128 x 128 otherwise, two workgroups per CU -- except that an
     // output of at most one such tile per CU with a long contraction takes the two-set form with a deep ring, since
     // no second workgroup would come to share the CU.
     const int64_t tiles_large = ((M + 255) / 256) * ((N + 255) / 256);
-    const bool large = g_force_geo >= 0 ? (g_force_geo == 1 || g_force_geo == 8)
-                                        : tiles_large >= 240 && (K >= 1024 || tiles_large >= 512);
-    const int64_t ntiles = large ? tiles_large : ((M + 127) / 128) * ((N + 127) / 128);
-    // Split the contraction when the tiles alone would leave most of the chip idle and the contraction is long.
-    int S = 1;
-    if (ntiles < 192 && K >= 1024) {
-        S = static_cast<int>(std::min<int64_t>({(512 + ntiles - 1) / ntiles, K / 256, 32}));
-        if (S < 1) S = 1;
-    }
+    p.large = g_force_geo >= 0 ? (g_force_geo == 1 || g_force_geo == 8) : tiles_large >= 240 && (K >= 1024 || tiles_large >= 512);
+    const int64_t ntiles = p.large ? tiles_large : ((M + 127) / 128) * ((N + 127) / 128);
     // the ring kernels keep offsets and extents in 32 bits
     const int64_t ext_a = (tA ? K : M) * lda * 2, ext_b = (tB ? N : K) * ldb * 2;
     const int64_t ext_max = (int64_t{1} << 30) - 8192;
     const bool ring_ok = ext_a < ext_max && ext_b < ext_max && lda < (1 << 21) && ldb < (1 << 21) && ldc < (1 << 20);
-    int ring = 0;  // 0: gemm_bf16 (register-staged tiles); otherwise a gemm_ring form
-    if (ring_ok && g_force_geo >= 5) ring = g_force_geo;
-    if (ring_ok && g_force_geo < 0) ring = large ? 8 : S > 1 ? 9 : (ntiles <= 256 && K >= 1024) ? 11 : 6;
-    auto run = [&](const GemmArgs& ga, int splits, bool f32) {
-        switch (ring) {
-            case 5: launch_ring<GeoSmall, 4>(tA, tB, ga, splits, f32, st); break;
-            case 6: launch_ring<GeoSmall, 2>(tA, tB, ga, splits, f32, st); break;
-            case 7: launch_ring<GeoSmall, 3>(tA, tB, ga, splits, f32, st); break;
-            case 8: launch_ring<GeoLarge, 2>(tA, tB, ga, splits, f32, st); break;
-            case 9: launch_ring<GeoSmallK2, 2>(tA, tB, ga, splits, f32, st); break;
-            case 10: launch_ring<GeoSmallK2, 3>(tA, tB, ga, splits, f32, st); break;
-            case 11: launch_ring<GeoSmallK2, 4>(tA, tB, ga, splits, f32, st); break;
-            default:
-                if (large)
-                    launch_geo<GeoLarge>(tA, tB, ga, splits, f32, st);
-                else
-                    launch_geo<GeoSmall>(tA, tB, ga, splits, f32, st);
-        }
-    };
-    if (S == 1) {
-        g.k_per_split = g.K;
-        g.part_stride = 0;
-        run(g, 1, c_dtype == PK_F32);
+    p.ring = 0;
+    if (ring_ok && g_force_geo >= 5) p.ring = g_force_geo;
+    if (ring_ok && g_force_geo < 0) p.ring = p.large ? 8 : (ntiles <= 256 && K >= 1024) ? 11 : 6;
+    // Split the contraction when the tiles alone would leave most of the chip idle and the contraction is long: as
+    // many slices as give every workgroup the chip holds at once one (tile, slice) -- a second round costs more than
+    // longer slices -- but none shorter than 1024, since every slice is another partial product to write and add
+    // (measured on [512, 1536], [512, 512], [512, 2752] and [1376, 512] outputs over 8192 tokens and on
+    // [2048, 512] over 32000). Split products take the 128 x 128 form with two workgroups per CU.
+    p.S = 1;
+    if (ntiles < 192 && K >= 2048) {
+        if (ring_ok && g_force_geo < 0) p.ring = 6;
+        const bool one_per_cu = p.ring == 5 || p.ring == 7 || p.ring == 8 || p.ring == 10 || p.ring == 11;
+        const int64_t s = std::min<int64_t>({(one_per_cu ? cu_count() : 2 * cu_count()) / ntiles, K / 1024, 16});
+        p.S = static_cast<int>(std::max<int64_t>(s, 1));
+    }
+    p.kps = static_cast<int>(((K + p.S - 1) / p.S + BK - 1) / BK * BK);
+    p.S = static_cast<int>((K + p.kps - 1) / p.kps);
+    return p;
+}
+void run_plan(const Plan& p, bool tA, bool tB, const GemmArgs& ga, int splits, bool f32, hipStream_t st) {
+    switch (p.ring) {
+        case 5: launch_ring<GeoSmall, 4>(tA, tB, ga, splits, f32, st); break;
+        case 6: launch_ring<GeoSmall, 2>(tA, tB, ga, splits, f32, st); break;
+        case 7: launch_ring<GeoSmall, 3>(tA, tB, ga, splits, f32, st); break;
+        case 8: launch_ring<GeoLarge, 2>(tA, tB, ga, splits, f32, st); break;
+        case 9: launch_ring<GeoSmallK2, 2>(tA, tB, ga, splits, f32, st); break;
+        case 10: launch_ring<GeoSmallK2, 3>(tA, tB, ga, splits, f32, st); break;
+        case 11: launch_ring<GeoSmallK2, 4>(tA, tB, ga, splits, f32, st); break;
+        default:
+            if (p.large)
+                launch_geo<GeoLarge>(tA, tB, ga, splits, f32, st);
+            else
+                launch_geo<GeoSmall>(tA, tB, ga, splits, f32, st);
+    }
+}
+bool takes(const void* a, bool tA, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return false;
+    if (!aligned16(a) || !aligned16(b)) return false;
+    if (lda % 8 || ldb % 8 || K % 8 || N % 8) return false;
+    if (tA && M % 8) return false;  // A^T is read in 16-byte chunks along M
+    return true;
+}
+GemmArgs gemm_args(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K) {
+    GemmArgs g;
+    g.a = static_cast<const uint16_t*>(a);
+    g.b = static_cast<const uint16_t*>(b);
+    g.c = nullptr;
+    g.M = static_cast<int>(M), g.N = static_cast<int>(N), g.K = static_cast<int>(K);
+    g.lda = lda, g.ldb = ldb, g.ldc = N;
+    g.beta = 0;
+    g.k_per_split = g.K;
+    g.part_stride = 0;
+    g.tiles_m = g.tiles_n = 0;
+    g.splits = 1;
+    return g;
+}
+}  // namespace
+
+// Returns false, having done nothing, for what the kernel does not take (fp32 operands, unaligned rows, sizes
+// that are not multiples of 8): the caller then uses the library GEMM.
+bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB, int64_t ldb, void* c, int c_dtype,
+                    int64_t M, int64_t N, int64_t K, int64_t ldc, float beta, hipStream_t st) {
+    if (!takes(a, tA, lda, b, ldb, M, N, K) || !aligned16(c) || ldc % 8) return false;
+    if (beta != 0.0f && beta != 1.0f) return false;
+    GemmArgs g = gemm_args(a, lda, b, ldb, M, N, K);
+    g.c = c;
+    g.ldc = ldc;
+    g.beta = beta != 0.0f;
+    const Plan p = make_plan(tA, tB, M, N, K, lda, ldb, ldc);
+    if (p.S == 1) {
+        run_plan(p, tA, tB, g, 1, c_dtype == PK_F32, st);
         return true;
     }
-    const int kps = static_cast<int>(((K + S - 1) / S + BK - 1) / BK * BK);
-    S = static_cast<int>((K + kps - 1) / kps);
-    Buffer part(sizeof(float) * static_cast<size_t>(S) * M * N);
+    Buffer part(sizeof(float) * static_cast<size_t>(p.S) * M * N);
     GemmArgs gp = g;
     gp.c = part.p;
     gp.ldc = N;
     gp.beta = 0;
-    gp.k_per_split = kps;
+    gp.k_per_split = p.kps;
     gp.part_stride = M * N;
-    run(gp, S, true);
+    run_plan(p, tA, tB, gp, p.S, true, st);
     const int64_t n4 = M * N / 4;
     hipLaunchKernelGGL(sum_slices, dim3(static_cast<unsigned>(std::min<int64_t>((n4 + 255) / 256, 4096))), dim3(256), 0, st,
-                       static_cast<const float*>(part.p), c, S, M * N, static_cast<int>(M), static_cast<int>(N), ldc,
+                       static_cast<const float*>(part.p), c, p.S, M * N, static_cast<int>(M), static_cast<int>(N), ldc,
                        g.beta, c_dtype == PK_F32 ? 1 : 0);
     hip_check(hipGetLastError(), "sum_slices launch");
+    return true;
+}
+
+// The same product left as its fp32 partial products part[s][M][N], s < nparts (one where the contraction is not
+// cut), for a caller that adds them itself on the way to where the result goes.
+bool gemm_mfma_bf16_parts(const void* a, bool tA, int64_t lda, const void* b, bool tB, int64_t ldb, int64_t M, int64_t N,
+                          int64_t K, hipStream_t st, std::unique_ptr<Buffer>& part, int& nparts) {
+    if (!takes(a, tA, lda, b, ldb, M, N, K)) return false;
+    const Plan p = make_plan(tA, tB, M, N, K, lda, ldb, N);
+    part.reset(new Buffer(sizeof(float) * static_cast<size_t>(p.S) * M * N));
+    GemmArgs g = gemm_args(a, lda, b, ldb, M, N, K);
+    g.c = part->p;
+    g.k_per_split = p.kps;
+    g.part_stride = p.S > 1 ? M * N : 0;
+    run_plan(p, tA, tB, g, p.S, true, st);
+    nparts = p.S;
     return true;
 }
 

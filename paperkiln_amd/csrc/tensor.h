@@ -2,6 +2,7 @@
 // host-side tape. The types themselves (Tensor, Buffer, the allocator, the
 // tape context) are public and live in include/paperkiln_amd.hpp.
 #pragma once
+#include <memory>
 #include <hip/hip_runtime.h>
 
 #include "paperkiln_amd.hpp"
@@ -62,11 +63,15 @@ void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dty
 // gemm_mfma.hip: the hand-written bf16 matrix-core GEMM. Returns false (nothing done) for operands it does not take.
 bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB, int64_t ldb, void* c, int c_dtype,
                     int64_t M, int64_t N, int64_t K, int64_t ldc, float beta, hipStream_t st);
+// The same product left as fp32 partial products part[s][M][N], s < nparts (the contraction cut into slices where the
+// output alone would leave the chip idle), for a caller that adds them on the way to where the result goes.
+bool gemm_mfma_bf16_parts(const void* a, bool tA, int64_t lda, const void* b, bool tB, int64_t ldb, int64_t M, int64_t N,
+                          int64_t K, hipStream_t st, std::unique_ptr<Buffer>& part, int& nparts);
 // Which GEMM serves bf16 operands: 1 (default) = each shape class goes to the kernel that measured faster for it,
 // 0 = the library only, 2 = the hand-written kernel for everything it takes. Set from the environment
 // (PK_GEMM=library) or by a caller that wants to compare them.
 void set_gemm_backend(int hand_written);
-void gemm_mfma_force_tiles(int which);  // -1: by shape (default), 0: 128 x 128 tiles, 1: 256 x 256 tiles (measurement)
+void gemm_mfma_force_tiles(int which);  // -1: by shape (default); 0, 1, 5 .. 11: one kernel form always (measurement)
 int gemm_backend();
 // dst[k] ([A.cols, B.cols/nsplit] fp32, contiguous) = beta * dst[k] + A^T B[:, k-th column block], k < nsplit <= 4
 void gemm_tn_split(const Tensor& A, const Tensor& B, float* const* dst, int nsplit, float beta);
