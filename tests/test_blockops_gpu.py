@@ -313,6 +313,46 @@ def test_matrix_core_gemm_against_float64(bo, mode, shape):
         bo.set_gemm_backend(prev)
 
 
+def test_matrix_core_gemm_under_graph_capture(bo):
+    """The persistent GEMM allocates nothing, clears nothing and keeps no state between launches, so a caller can record
+    it into a HIP graph: a product of several tiles per workgroup, one of a single tile per workgroup with the two-set
+    form, and an accumulating one, replayed three times with fresh operands copied into the captured tensors and eager
+    products in between; every replay equals the eager product of the same operands bit for bit."""
+    gen = torch.Generator(device="cuda").manual_seed(17)
+    cases = [(8192, 2752, 512, False, False, torch.bfloat16), (2048, 512, 1536, False, True, torch.bfloat16),
+             (1024, 768, 264, True, False, torch.float32)]
+    prev = bo.set_gemm_backend(2)
+    try:
+        for M, N, K, ta, tb, od in cases:
+            a = torch.randn((K, M) if ta else (M, K), generator=gen, device="cuda").bfloat16()
+            b = torch.randn((N, K) if tb else (K, N), generator=gen, device="cuda").bfloat16()
+            acc = torch.zeros((M, N), dtype=od, device="cuda")
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):  # warm-up outside the capture, as torch asks
+                bo.matmul(a, b, ta, tb, out_dtype=od)
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                c = bo.matmul(a, b, ta, tb, out_dtype=od)
+                bo.matmul(a, b, ta, tb, out=acc)
+            acc.zero_()
+            total = torch.zeros_like(acc)
+            for rep in range(3):
+                fa, fb = torch.randn_like(a.float()).bfloat16(), torch.randn_like(b.float()).bfloat16()
+                a.copy_(fa)
+                b.copy_(fb)
+                graph.replay()
+                torch.cuda.synchronize()
+                want = bo.matmul(fa, fb, ta, tb, out_dtype=od)  # eager work between replays
+                bo.matmul(fa, fb, ta, tb, out=total)
+                torch.cuda.synchronize()
+                assert torch.equal(c, want), (M, N, K, "replay", rep)
+                assert torch.equal(acc, total), (M, N, K, "accumulating replay", rep)
+    finally:
+        bo.set_gemm_backend(prev)
+
+
 def test_gemm_dispatch_modes_agree(bo):
     """Default dispatch (per shape class), library only, and the hand-written kernel everywhere give the same
     product to fp32 accumulation accuracy on a Linear-shaped problem; operands the hand-written kernel does not take
