@@ -272,12 +272,6 @@ struct RingOp {
     // the chunk of its LDS row that holds memory chunk c (and vice versa: the map is an involution)
     __device__ static int swz(int r, int c) { return TR ? c ^ ((r & 3) << 2) : c ^ ((r & 7) ^ ((r >> 3) & 3)); }
 };
-// Offsets that are outside every buffer these kernels take (operands of less than 1 GiB): a lane offset, and a scalar
-// offset whose sum with any lane offset and immediate still fits 32 bits.
-constexpr uint32_t OUTSIDE = 0x80000000u, PAST_END = 0x40000000u;
-constexpr int BIAS = 4096;                 // descriptors start this far before the tile, so that an offset minus the
-                                           // instruction's immediate (below 4096) never goes negative
-
 // Descriptor of an operand's tile: from BIAS bytes before the tile's first element of the contraction range to the
 // operand's end (rows past the matrix, and rows past the contraction's end where the contraction index is the row,
 // read as zeros); `step` bytes per slice.
@@ -306,27 +300,6 @@ __device__ inline TileDesc tile_desc(const uint16_t* base, int64_t ld, int rc0, 
     d.rsrc[2] = static_cast<uint32_t>(left + BIAS);
     d.rsrc[3] = 0x00020000u;
     return d;
-}
-// PER consecutive 1 KB pieces of LDS from `lds_byte` on, lane offsets off[j] (already less j KB), scalar offset soff.
-// m0 is set and used inside the one statement; the compiler never keeps a value of its own in m0 across other code.
-template <int PER>
-__device__ inline void dma_group(uint32_t lds_byte, const uint32_t (&off)[PER], u32x4 rsrc, uint32_t soff) {
-    if constexpr (PER == 2)
-        asm volatile(
-            "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
-            "buffer_load_dwordx4 %1, %3, %4 offen lds\n\t"
-            "buffer_load_dwordx4 %2, %3, %4 offen offset:1024 lds" ::"s"(lds_byte),
-            "v"(off[0]), "v"(off[1]), "s"(rsrc), "s"(soff)
-            : "memory");
-    else
-        asm volatile(
-            "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
-            "buffer_load_dwordx4 %1, %5, %6 offen lds\n\t"
-            "buffer_load_dwordx4 %2, %5, %6 offen offset:1024 lds\n\t"
-            "buffer_load_dwordx4 %3, %5, %6 offen offset:2048 lds\n\t"
-            "buffer_load_dwordx4 %4, %5, %6 offen offset:3072 lds" ::"s"(lds_byte),
-            "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "s"(rsrc), "s"(soff)
-            : "memory");
 }
 template <int N>
 __device__ inline void wait_loads_then_barrier() {
@@ -361,13 +334,6 @@ __device__ inline void store16(u32x4 v, uint32_t off, u32x4 rsrc, uint32_t soff)
     // may be overwritten by the very next instruction, which a 16-byte store does not allow: one idle state
     asm volatile("buffer_store_dwordx4 %0, %1, %2, %3 offen\n\ts_nop 0" ::"v"(v), "v"(off), "s"(rsrc), "s"(soff) : "memory");
 }
-template <int N>
-__device__ inline void wait_loads() {
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-__device__ inline void barrier() { asm volatile("s_barrier" ::: "memory"); }
-
 // What a workgroup stores per tile, for the count of memory operations in flight: FM strips of all WGM * 32 rows
 // (bf16) or FM * WGM strips of 32 rows (fp32, whose wider rows would not fit a ring slot otherwise), each
 // rows * chunks-per-row / threads stores per thread.

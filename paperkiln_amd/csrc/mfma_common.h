@@ -196,6 +196,56 @@ __device__ inline u32x4 tile_load16(__amdgpu_buffer_rsrc_t rsrc, int byte_off) {
     return __builtin_amdgcn_raw_buffer_load_b128(rsrc, byte_off, 0, 0);
 }
 
+// ---- tiles straight from memory into LDS (buffer_load_dwordx4 ... offen lds) ----
+// One such instruction fills 1 KB of LDS lane after lane from M0 + immediate on; each lane names the 16 bytes of memory it
+// fetches (lane offset + scalar offset + immediate, all counted by the range check of the descriptor; a lane outside
+// the buffer writes zeros). The instructions are invisible to the compiler's count of memory operations in flight:
+// the kernels that use them wait with wait_loads<N> on counts of their own.
+// Offsets that are outside every buffer these kernels take (operands of less than 1 GiB): a lane offset, and a scalar
+// offset whose sum with any lane offset and immediate still fits 32 bits.
+constexpr uint32_t OUTSIDE = 0x80000000u, PAST_END = 0x40000000u;
+// Descriptors start this far before the tile, so that a lane offset minus the instruction's immediate (below 4096)
+// never goes negative.
+constexpr int BIAS = 4096;
+// PER consecutive 1 KB pieces of LDS from `lds_byte` on, lane offsets off[j] (already less j KB), scalar offset soff.
+// m0 is set and used inside the one statement; the compiler never keeps a value of its own in m0 across other code.
+template <int PER>
+__device__ inline void dma_group(uint32_t lds_byte, const uint32_t (&off)[PER], u32x4 rsrc, uint32_t soff) {
+    static_assert(PER == 1 || PER == 2 || PER == 4, "groups of one, two or four pieces");
+    if constexpr (PER == 1)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(lds_byte), "v"(off[0]),
+                     "s"(rsrc), "s"(soff)
+                     : "memory");
+    else if constexpr (PER == 2)
+        asm volatile(
+            "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+            "buffer_load_dwordx4 %1, %3, %4 offen lds\n\t"
+            "buffer_load_dwordx4 %2, %3, %4 offen offset:1024 lds" ::"s"(lds_byte),
+            "v"(off[0]), "v"(off[1]), "s"(rsrc), "s"(soff)
+            : "memory");
+    else
+        asm volatile(
+            "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+            "buffer_load_dwordx4 %1, %5, %6 offen lds\n\t"
+            "buffer_load_dwordx4 %2, %5, %6 offen offset:1024 lds\n\t"
+            "buffer_load_dwordx4 %3, %5, %6 offen offset:2048 lds\n\t"
+            "buffer_load_dwordx4 %4, %5, %6 offen offset:3072 lds" ::"s"(lds_byte),
+            "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "s"(rsrc), "s"(soff)
+            : "memory");
+}
+template <int N>
+__device__ inline void wait_loads() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ inline void barrier() { asm volatile("s_barrier" ::: "memory"); }
+// descriptor words for `bytes` bytes from p - BIAS on (raw buffer, no swizzle)
+__device__ inline u32x4 dma_rsrc(const void* p, uint32_t bytes) {
+    const uint64_t a = reinterpret_cast<uint64_t>(p) - BIAS;
+    const u32x4 r = {static_cast<uint32_t>(a), static_cast<uint32_t>(a >> 32) & 0xffffu, bytes + BIAS, 0x00020000u};
+    return r;
+}
+
 // XCD-aware workgroup -> tile mapping. The 256 CUs sit in 8 XCDs, each with
 // its own 4 MB L2, and consecutive workgroup ids go round-robin over the XCDs.
 // Every block of a (batch, KV head) unit re-reads that unit's K/V (or Q/dO),
