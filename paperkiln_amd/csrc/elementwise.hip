@@ -7,6 +7,7 @@
 #include <rocblas/rocblas.h>
 
 #include <atomic>
+#include <type_traits>
 #include <cstdlib>
 #include <map>
 #include <cmath>
@@ -456,14 +457,94 @@ __global__ void rms_bwd_dw_part8(const uint16_t* dy, const uint16_t* x, const fl
         part[static_cast<int64_t>(blockIdx.x) * C + j] = t;
     }
 }
+// dx and the dW partial sums in one pass over dY and x (both are wanted in a training step, and each reads both
+// tensors): a wavefront takes ROWS_PB / 4 rows of its block one after another, lane l the columns 8 l .. 8 l + 7 of
+// every 512-column pass (NP passes, C <= 512 NP), keeps its rows' contribution to dW in registers, and the four
+// wavefronts meet in LDS in a fixed order.
+template <int NP>
+__global__ void rms_bwd_dx_dw8(const uint16_t* dy, const uint16_t* x, const float* rinv, const float* w, uint16_t* dx,
+                               float* part, int64_t R, int C) {
+    extern __shared__ float sh_dw[];  // [3][C]: wavefronts 1 .. 3
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int64_t r0 = static_cast<int64_t>(blockIdx.x) * ROWS_PB, r1 = min(r0 + ROWS_PB, R);
+    F8 acc[NP], ww[NP];
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const int j = lane * 8 + p * 512;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) acc[p].v[k] = 0.0f;
+        if (j < C) ww[p] = ld8(w, j);
+    }
+    for (int64_t row = r0 + wv; row < r1; row += 4) {
+        const uint16_t* xr = x + row * C;
+        const uint16_t* gr = dy + row * C;
+        F8 g[NP], v[NP];
+        float term = 0.0f;
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int j = lane * 8 + p * 512;
+            if (j < C) {
+                g[p] = ld8(gr, j);
+                v[p] = ld8(xr, j);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) term = fmaf(g[p].v[k] * ww[p].v[k], v[p].v[k], term);
+            }
+        }
+        term = wave_sum(term);
+        const float ri = rinv[row], kk = ri * ri * term / static_cast<float>(C);
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int j = lane * 8 + p * 512;
+            if (j < C) {
+                F8 o;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    o.v[k] = ri * (g[p].v[k] * ww[p].v[k] - v[p].v[k] * kk);
+                    acc[p].v[k] = fmaf(g[p].v[k] * v[p].v[k], ri, acc[p].v[k]);
+                }
+                st8(dx + row * C, j, o);
+            }
+        }
+    }
+    if (wv > 0) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int j = lane * 8 + p * 512;
+            if (j < C) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) sh_dw[(wv - 1) * C + j + k] = acc[p].v[k];
+            }
+        }
+    }
+    __syncthreads();
+    if (wv == 0) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int j = lane * 8 + p * 512;
+            if (j < C) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    part[static_cast<int64_t>(blockIdx.x) * C + j + k] =
+                        ((acc[p].v[k] + sh_dw[j + k]) + sh_dw[C + j + k]) + sh_dw[2 * C + j + k];
+            }
+        }
+    }
+}
 __global__ void colsum_parts(const float* part, float* dw, int nparts, int C) {
     // 64 columns x 16 groups of parts per block (1024 threads: each walks a sixteenth of the
     // parts, the walk being a chain of dependent loads); the groups meet in a fixed order
     __shared__ float sh[16][64];
     const int col = blockIdx.x * 64 + (threadIdx.x & 63), grp = threadIdx.x >> 6;
     float s = 0.0f;
-    if (col < C)
-        for (int p = grp; p < nparts; p += 16) s += part[static_cast<int64_t>(p) * C + col];
+    if (col < C) {
+        int p = grp;
+        for (; p + 48 < nparts; p += 64) {  // four independent loads in flight, added in index order
+            const float a0 = part[static_cast<int64_t>(p) * C + col], a1 = part[static_cast<int64_t>(p + 16) * C + col];
+            const float a2 = part[static_cast<int64_t>(p + 32) * C + col], a3 = part[static_cast<int64_t>(p + 48) * C + col];
+            s = (((s + a0) + a1) + a2) + a3;
+        }
+        for (; p < nparts; p += 16) s += part[static_cast<int64_t>(p) * C + col];
+    }
     sh[grp][threadIdx.x & 63] = s;
     __syncthreads();
     if (grp == 0 && col < C) {
@@ -915,6 +996,29 @@ void k_rmsnorm_fwd(const Tensor& x, const Tensor& w, float eps, const Tensor& y,
 void k_rmsnorm_bwd(const Tensor& dy, const Tensor& x, const float* rinv, const Tensor& w, const Tensor* dw,
                    const Tensor* dx) {
     const int C = static_cast<int>(x.cols);
+    if (dx && dw && x.dtype == PK_BF16 && C % 8 == 0 && C <= 2048 && aligned16p(x.ptr()) && aligned16p(dy.ptr()) &&
+        aligned16p(dx->ptr()) && aligned16p(w.ptr())) {
+        const int nparts = static_cast<int>((x.rows + ROWS_PB - 1) / ROWS_PB);
+        Buffer part(sizeof(float) * static_cast<size_t>(nparts) * C);
+        const size_t lds = sizeof(float) * 3 * C;
+        auto launch = [&](auto np) {
+            hipLaunchKernelGGL((rms_bwd_dx_dw8<decltype(np)::value>), dim3(nparts), dim3(NT), lds, tape_stream(),
+                               static_cast<const uint16_t*>(dy.ptr()), static_cast<const uint16_t*>(x.ptr()), rinv,
+                               static_cast<const float*>(w.ptr()), static_cast<uint16_t*>(dx->ptr()),
+                               static_cast<float*>(part.p), x.rows, C);
+        };
+        if (C <= 512)
+            launch(std::integral_constant<int, 1>{});
+        else if (C <= 1024)
+            launch(std::integral_constant<int, 2>{});
+        else
+            launch(std::integral_constant<int, 4>{});
+        post();
+        hipLaunchKernelGGL(colsum_parts, dim3((C + 63) / 64), dim3(1024), 0, tape_stream(),
+                           static_cast<const float*>(part.p), static_cast<float*>(dw->ptr()), nparts, C);
+        post();
+        return;
+    }
     if (dx) {
         if (x.dtype == PK_BF16 && C % 8 == 0 && aligned16p(x.ptr()) && aligned16p(dy.ptr()) && aligned16p(dx->ptr()) &&
             aligned16p(w.ptr())) {
