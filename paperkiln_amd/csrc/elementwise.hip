@@ -458,13 +458,14 @@ __global__ void rms_bwd_dw_part8(const uint16_t* dy, const uint16_t* x, const fl
     }
 }
 // dx and the dW partial sums in one pass over dY and x (both are wanted in a training step, and each reads both
-// tensors): a wavefront takes ROWS_PB / 4 rows of its block one after another, lane l the columns 8 l .. 8 l + 7 of
-// every 512-column pass (NP passes, C <= 512 NP), keeps its rows' contribution to dW in registers, and the four
+// tensors): a wavefront takes ROWS_PB / 8 rows of its block, two at a time, lane l the columns 8 l .. 8 l + 7 of
+// every 512-column pass (NP passes, C <= 512 NP), keeps its rows' contribution to dW in registers, and the eight
 // wavefronts meet in LDS in a fixed order.
 template <int NP>
 __global__ void rms_bwd_dx_dw8(const uint16_t* dy, const uint16_t* x, const float* rinv, const float* w, uint16_t* dx,
                                float* part, int64_t R, int C) {
-    extern __shared__ float sh_dw[];  // [3][C]: wavefronts 1 .. 3
+    constexpr int NWV = 8;            // wavefronts per block
+    extern __shared__ float sh_dw[];  // [NWV - 1][C]: wavefronts 1 .. NWV - 1
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int64_t r0 = static_cast<int64_t>(blockIdx.x) * ROWS_PB, r1 = min(r0 + ROWS_PB, R);
     F8 acc[NP], ww[NP];
@@ -475,34 +476,50 @@ __global__ void rms_bwd_dx_dw8(const uint16_t* dy, const uint16_t* x, const floa
         for (int k = 0; k < 8; ++k) acc[p].v[k] = 0.0f;
         if (j < C) ww[p] = ld8(w, j);
     }
-    for (int64_t row = r0 + wv; row < r1; row += 4) {
-        const uint16_t* xr = x + row * C;
-        const uint16_t* gr = dy + row * C;
-        F8 g[NP], v[NP];
-        float term = 0.0f;
+    // two rows of the wavefront at a time: their loads are in flight together, and so are the two row reductions
+    for (int64_t row = r0 + wv; row < r1; row += 2 * NWV) {
+        const bool two = row + NWV < r1;
+        const int64_t rows[2] = {row, two ? row + NWV : row};
+        F8 g[2][NP], v[2][NP];
+        float term[2] = {0.0f, 0.0f};
 #pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            const int j = lane * 8 + p * 512;
-            if (j < C) {
-                g[p] = ld8(gr, j);
-                v[p] = ld8(xr, j);
+        for (int q = 0; q < 2; ++q)
 #pragma unroll
-                for (int k = 0; k < 8; ++k) term = fmaf(g[p].v[k] * ww[p].v[k], v[p].v[k], term);
-            }
-        }
-        term = wave_sum(term);
-        const float ri = rinv[row], kk = ri * ri * term / static_cast<float>(C);
-#pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            const int j = lane * 8 + p * 512;
-            if (j < C) {
-                F8 o;
-#pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    o.v[k] = ri * (g[p].v[k] * ww[p].v[k] - v[p].v[k] * kk);
-                    acc[p].v[k] = fmaf(g[p].v[k] * v[p].v[k], ri, acc[p].v[k]);
+            for (int p = 0; p < NP; ++p) {
+                const int j = lane * 8 + p * 512;
+                if (j < C) {
+                    g[q][p] = ld8(dy + rows[q] * C, j);
+                    v[q][p] = ld8(x + rows[q] * C, j);
                 }
-                st8(dx + row * C, j, o);
+            }
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+#pragma unroll
+            for (int p = 0; p < NP; ++p) {
+                const int j = lane * 8 + p * 512;
+                if (j < C) {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) term[q] = fmaf(g[q][p].v[k] * ww[p].v[k], v[q][p].v[k], term[q]);
+                }
+            }
+        term[0] = wave_sum(term[0]);
+        term[1] = wave_sum(term[1]);
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            if (q == 1 && !two) break;  // wavefront-uniform: an odd row count leaves the second row out
+            const float ri = rinv[rows[q]], kk = ri * ri * term[q] / static_cast<float>(C);
+#pragma unroll
+            for (int p = 0; p < NP; ++p) {
+                const int j = lane * 8 + p * 512;
+                if (j < C) {
+                    F8 o;
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        o.v[k] = ri * (g[q][p].v[k] * ww[p].v[k] - v[q][p].v[k] * kk);
+                        acc[p].v[k] = fmaf(g[q][p].v[k] * v[q][p].v[k], ri, acc[p].v[k]);
+                    }
+                    st8(dx + rows[q] * C, j, o);
+                }
             }
         }
     }
@@ -523,9 +540,12 @@ __global__ void rms_bwd_dx_dw8(const uint16_t* dy, const uint16_t* x, const floa
             const int j = lane * 8 + p * 512;
             if (j < C) {
 #pragma unroll
-                for (int k = 0; k < 8; ++k)
-                    part[static_cast<int64_t>(blockIdx.x) * C + j + k] =
-                        ((acc[p].v[k] + sh_dw[j + k]) + sh_dw[C + j + k]) + sh_dw[2 * C + j + k];
+                for (int k = 0; k < 8; ++k) {
+                    float t = acc[p].v[k];
+#pragma unroll
+                    for (int q = 0; q < NWV - 1; ++q) t += sh_dw[q * C + j + k];
+                    part[static_cast<int64_t>(blockIdx.x) * C + j + k] = t;
+                }
             }
         }
     }
@@ -1000,9 +1020,9 @@ void k_rmsnorm_bwd(const Tensor& dy, const Tensor& x, const float* rinv, const T
         aligned16p(dx->ptr()) && aligned16p(w.ptr())) {
         const int nparts = static_cast<int>((x.rows + ROWS_PB - 1) / ROWS_PB);
         Buffer part(sizeof(float) * static_cast<size_t>(nparts) * C);
-        const size_t lds = sizeof(float) * 3 * C;
+        const size_t lds = sizeof(float) * 7 * C;
         auto launch = [&](auto np) {
-            hipLaunchKernelGGL((rms_bwd_dx_dw8<decltype(np)::value>), dim3(nparts), dim3(NT), lds, tape_stream(),
+            hipLaunchKernelGGL((rms_bwd_dx_dw8<decltype(np)::value>), dim3(nparts), dim3(512), lds, tape_stream(),
                                static_cast<const uint16_t*>(dy.ptr()), static_cast<const uint16_t*>(x.ptr()), rinv,
                                static_cast<const float*>(w.ptr()), static_cast<uint16_t*>(dx->ptr()),
                                static_cast<float*>(part.p), x.rows, C);
