@@ -189,9 +189,9 @@ def clip_grad_norm_(grads, max_norm):
 
 
 def set_gemm_backend(mode: int) -> int:
-    """Choose the kernel for bf16 GEMMs (pk_set_gemm_backend): 1 = per shape class whichever measured faster
-    (default), 0 = rocBLAS only, 2 = the library's own matrix-core kernel wherever it applies, 3 .. 11 = the same
-    with one kernel form forced (measurements; see include/paperkiln_amd.h). Returns the previous setting (0, 1, 2)."""
+    """Choose the kernel for bf16 GEMMs (pk_set_gemm_backend): 1 (default) and 2 = the library's own matrix-core
+    kernel wherever it applies, in the form it picks per shape, 0 = rocBLAS only, 3 .. 11 = the own kernel
+    with one form forced (measurements; see include/paperkiln_amd.h). Returns the previous setting (0, 1, 2)."""
     return int(_lib.lib().pk_set_gemm_backend(int(mode)))
 
 

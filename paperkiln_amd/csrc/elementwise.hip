@@ -1219,13 +1219,9 @@ void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dty
     if (A.dtype != B.dtype) throw std::runtime_error("gemm: operand dtypes differ");
     // Which kernel: measured per shape on the MI355X as GPU time from a kernel trace (timing launches from the host
     // measures the library's longer host path instead), on the Linear shapes of a d = 512 block and of the tied
-    // head. The hand-written kernel is ahead of the library on 12 of the 15 products and level on one; the
-    // library keeps the class it is ahead in by 5 - 15 %: A and B both with the contraction index contiguous
-    // (gradient times weight), an output of at most one 128 x 128 tile per CU and a contraction of 1024 or more.
-    // backend 2 sends everything the hand-written kernel takes to it, backend 0 nothing.
-    const int backend = gemm_backend();
-    const bool theirs = !tA && tB && ((M + 127) / 128) * ((N + 127) / 128) <= 256 && Ka >= 1024;
-    const bool mine = backend == 2 || (backend == 1 && !theirs);
+    // head: the hand-written kernel is ahead of the library or level with it on all 15 products, so bf16 operands
+    // go to it whenever it takes them (backends 1 and 2 alike); backend 0 sends everything to the library.
+    const bool mine = gemm_backend() != 0;
     if (A.dtype == PK_BF16 && mine &&
         gemm_mfma_bf16(A.ptr(), tA, lda, B.ptr(), tB, B.cols, C, c_dtype, M, N, Ka, ldc, beta, tape_stream()))
         return;

@@ -354,7 +354,7 @@ struct TileStore {
 // (virtual block -> (contraction slice, tile) as gemm_bf16 maps (blockIdx.z, blockIdx.x), XCD by XCD), and the ring
 // runs on across tile boundaries: the first slices of the next tile are on their way while the last ones of this tile
 // are multiplied and its result is stored, so a tile's first round trip to memory is paid once per workgroup.
-template <typename G, bool TA, bool TB, bool CF32, int NS>
+template <typename G, bool TA, bool TB, bool CF32, int NS, bool SPREAD>
 __global__ __launch_bounds__(G::NTHR, NS * (RingOp<TA, G::BM, G::NTHR / 64>::BYTES + RingOp<!TB, G::BN, G::NTHR / 64>::BYTES) <= 80 * 1024 ? 2 : 1)
 void gemm_ring(GemmArgs g) {
     constexpr int BM = G::BM, BN = G::BN, NTHR = G::NTHR, FM = G::FM, FN = G::FN, NW = NTHR / 64;
@@ -370,7 +370,7 @@ void gemm_ring(GemmArgs g) {
     constexpr int KS = G::KS, NWQ = G::WGM * G::WGN, KPW = BK / 16 / KS;  // k-chunks of a slice per wavefront
     static_assert(KS == 1 || KS == 2, "one or two wavefront sets");
     static_assert(KS == 1 || (FM % 2 == 0 && NWQ * 64 * (FM / 2) * FN * 64 <= SLOT), "half of the second set's sums per slot");
-    const int ks = w / NWQ, wq = w - ks * NWQ;
+    const int ks = KS == 1 ? 0 : w / NWQ, wq = w - ks * NWQ;
     const int c32 = lane & 31, gh = lane >> 5, wm = wq / G::WGN, wn = wq % G::WGN;
 
     // virtual blocks
@@ -433,24 +433,32 @@ void gemm_ring(GemmArgs g) {
     // One call per slice of the stream, in order, also past the stream's end: a wavefront's count of loads in flight
     // stays the same, and the scalar offset is then outside every buffer, so nothing is fetched (the lanes write zeros
     // into a slot nobody reads).
-    auto fetch = [&](int slot) {
-        const bool none = f_nslices == 0;
-        const uint32_t sa = none ? PAST_END : soff_a, sb = none ? PAST_END : soff_b;
-        const uint32_t la = dst_a + static_cast<uint32_t>(slot) * SLOT, lb = dst_b + static_cast<uint32_t>(slot) * SLOT;
-        const bool last = f_slice == f_nslices - 1;
-        if ((TA || last) && (!TB || last)) {  // wavefront-uniform
-            dma_group<OA::PER>(la, offa_c, da.rsrc, sa);
-            dma_group<OB::PER>(lb, offb_c, db.rsrc, sb);
-        } else if (TA || last) {
-            dma_group<OA::PER>(la, offa_c, da.rsrc, sa);
-            dma_group<OB::PER>(lb, offb, db.rsrc, sb);
-        } else if (!TB || last) {
-            dma_group<OA::PER>(la, offa, da.rsrc, sa);
-            dma_group<OB::PER>(lb, offb_c, db.rsrc, sb);
-        } else {
-            dma_group<OA::PER>(la, offa, da.rsrc, sa);
-            dma_group<OB::PER>(lb, offb, db.rsrc, sb);
+    // A slice's loads are issued one by one between the matrix instructions of the slice in hand (all at once they
+    // hold a wavefront for 500 clocks in which it issues nothing else, and every wavefront of the workgroup does so at
+    // the same time): begin fixes where the slice goes and what it reads, piece<Q> issues its Q-th load, end moves
+    // the stream on.
+    uint32_t f_la = 0, f_lb = 0, f_sa = 0, f_sb = 0;
+    bool f_ca = false, f_cb = false;  // this slice takes the masked lane offsets of A / of B
+    auto fetch_begin = [&](int slot) {
+        const bool none = f_nslices == 0, last = f_slice == f_nslices - 1;
+        f_sa = none ? PAST_END : soff_a;
+        f_sb = none ? PAST_END : soff_b;
+        f_la = dst_a + static_cast<uint32_t>(slot) * SLOT;
+        f_lb = dst_b + static_cast<uint32_t>(slot) * SLOT;
+        f_ca = TA || last;
+        f_cb = !TB || last;
+    };
+    auto fetch_piece = [&](auto qc) {
+        constexpr int Q = decltype(qc)::value;
+        if constexpr (Q < OA::PER) {
+            dma_piece<Q>(f_la, f_ca ? offa_c[Q] : offa[Q], da.rsrc, f_sa);
+        } else if constexpr (Q < PERTOT) {
+            constexpr int J = Q - OA::PER;
+            dma_piece<J>(f_lb, f_cb ? offb_c[J] : offb[J], db.rsrc, f_sb);
         }
+    };
+    auto fetch_end = [&]() {
+        const bool none = f_nslices == 0;
         soff_a += da.step;
         soff_b += db.step;
         if (!none && ++f_slice == f_nslices) {
@@ -458,16 +466,32 @@ void gemm_ring(GemmArgs g) {
             open();
         }
     };
+    auto fetch_pieces = [&](auto first, auto count) {  // pieces first .. first + count - 1
+        constexpr int F = decltype(first)::value, N = decltype(count)::value;
+        if constexpr (N > 0) {
+            fetch_piece(std::integral_constant<int, F>{});
+            if constexpr (N > 1) fetch_piece(std::integral_constant<int, F + 1>{});
+            if constexpr (N > 2) fetch_piece(std::integral_constant<int, F + 2>{});
+            if constexpr (N > 3) fetch_piece(std::integral_constant<int, F + 3>{});
+            static_assert(N <= 4, "at most four pieces per k-chunk");
+        }
+    };
+    auto fetch = [&](int slot) {  // the whole slice at once (before the first slice is multiplied)
+        fetch_begin(slot);
+        fetch_pieces(std::integral_constant<int, 0>{}, std::integral_constant<int, 4>{});
+        if constexpr (PERTOT > 4) fetch_pieces(std::integral_constant<int, 4>{}, std::integral_constant<int, PERTOT - 4>{});
+        fetch_end();
+    };
 
     // ---- lane parts of the fragment reads ----
     // [row][k]: row c32 of a 32-row block, chunk 2 kk + gh, one address per kk (the swizzle is an exclusive-or with a
     // lane value, so kk cannot be an immediate); [k][column]: rows 8 gh + j / 4 (+ 4), columns 16 u + 4 (j % 4) of
     // 32-column block b, one address per block the wavefront reads.
     const int tj = lane & 15, tu = (lane >> 4) & 1;
-    uint32_t r_row[BK / 16], ra_tr[FM], rb_tr[FN];
+    uint32_t r_row[KPW], ra_tr[FM], rb_tr[FN];  // r_row: for this wavefront's own k-chunks ks KPW .. ks KPW + KPW - 1
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk)
-        r_row[kk] = static_cast<uint32_t>(c32 * 128 + (RingOp<false, 128, 4>::swz(c32, 2 * kk + gh)) * 16);
+    for (int kq = 0; kq < KPW; ++kq)
+        r_row[kq] = static_cast<uint32_t>(c32 * 128 + (RingOp<false, 128, 4>::swz(c32, 2 * (ks * KPW + kq) + gh)) * 16);
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
         const int blk = wm * FM + i, r = 8 * gh + (tj >> 2);
@@ -485,12 +509,12 @@ void gemm_ring(GemmArgs g) {
         const s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         return *reinterpret_cast<const bf16x8*>(&v);
     };
-    auto read_a = [&](const uint8_t* As, int i, int kk) -> bf16x8 {
-        if (!TA) return lds_read8(reinterpret_cast<const uint16_t*>(As + r_row[kk] + (wm * FM + i) * 32 * 128));
+    auto read_a = [&](const uint8_t* As, int i, int kq, int kk) -> bf16x8 {
+        if (!TA) return lds_read8(reinterpret_cast<const uint16_t*>(As + r_row[kq] + (wm * FM + i) * 32 * 128));
         return read_tr(As + ra_tr[i] + kk * 16 * OA::ROWB, OA::ROWB);
     };
-    auto read_b = [&](const uint8_t* Bs, int j, int kk) -> bf16x8 {
-        if (TB) return lds_read8(reinterpret_cast<const uint16_t*>(Bs + r_row[kk] + (wn * FN + j) * 32 * 128));
+    auto read_b = [&](const uint8_t* Bs, int j, int kq, int kk) -> bf16x8 {
+        if (TB) return lds_read8(reinterpret_cast<const uint16_t*>(Bs + r_row[kq] + (wn * FN + j) * 32 * 128));
         return read_tr(Bs + rb_tr[j] + kk * 16 * OB::ROWB, OB::ROWB);
     };
 
@@ -631,23 +655,37 @@ void gemm_ring(GemmArgs g) {
             else
                 wait_loads<(NS - 2) * PERTOT>();
             since_store = min(since_store + 1, NS);
-            barrier();                 // ... for every wavefront, and all have read the slice before
-            fetch((u + NS - 1) % NS);  // slice + NS - 1 of the stream into the slot the slice before leaves
+            barrier();                       // ... for every wavefront, and all have read the slice before
+            fetch_begin((u + NS - 1) % NS);  // slice + NS - 1 of the stream goes into the slot the slice before leaves
             const uint8_t* As = lds + u * SLOT;
             const uint8_t* Bs = As + OA::BYTES;
-#pragma unroll
-            for (int kq = 0; kq < KPW; ++kq) {
-                const int kk = ks * KPW + kq;
+            constexpr int SP = SPREAD ? KPW : 0;
+            constexpr int PPK = SP == 0 ? 0 : (PERTOT + SP - 1) / SP;  // loads dropped behind each k-chunk's matrix instructions
+            if constexpr (SP == 0) {
+                fetch_pieces(std::integral_constant<int, 0>{}, std::integral_constant<int, 4>{});
+                if constexpr (PERTOT > 4) fetch_pieces(std::integral_constant<int, 4>{}, std::integral_constant<int, PERTOT - 4>{});
+            }
+            auto chunk = [&](auto kqc) {
+                constexpr int KQ = decltype(kqc)::value;
+                const int kk = ks * KPW + KQ;
                 bf16x8 fa[FM], fbb[FN];
 #pragma unroll
-                for (int i = 0; i < FM; ++i) fa[i] = read_a(As, i, kk);
+                for (int i = 0; i < FM; ++i) fa[i] = read_a(As, i, KQ, kk);
 #pragma unroll
-                for (int j = 0; j < FN; ++j) fbb[j] = read_b(Bs, j, kk);
+                for (int j = 0; j < FN; ++j) fbb[j] = read_b(Bs, j, KQ, kk);
 #pragma unroll
                 for (int i = 0; i < FM; ++i)
 #pragma unroll
                     for (int j = 0; j < FN; ++j) acc[i][j] = mfma32(fbb[j], fa[i], acc[i][j]);
-            }
+                constexpr int F = KQ * PPK, N = SP == 0 || F >= PERTOT ? 0 : (F + PPK <= PERTOT ? PPK : PERTOT - F);
+                fetch_pieces(std::integral_constant<int, F>{}, std::integral_constant<int, (N > 4 ? 4 : N)>{});
+                if constexpr (N > 4) fetch_pieces(std::integral_constant<int, F + 4>{}, std::integral_constant<int, N - 4>{});
+            };
+            chunk(std::integral_constant<int, 0>{});
+            if constexpr (KPW > 1) chunk(std::integral_constant<int, 1>{});
+            if constexpr (KPW > 2) chunk(std::integral_constant<int, 2>{});
+            if constexpr (KPW > 3) chunk(std::integral_constant<int, 3>{});
+            fetch_end();
             if (++c_slice == c_nslices) {  // wavefront-uniform
                 barrier();  // every wavefront has read slot u: it takes the result on its way out
                 store_result(lds + u * SLOT, cb);
@@ -699,12 +737,12 @@ void launch_form(bool tA, bool tB, const GemmArgs& g, dim3 grid, hipStream_t st)
     if (tA && !tB) hipLaunchKernelGGL((gemm_bf16<G, true, false, CF32>), grid, dim3(G::NTHR), 0, st, g);
     if (tA && tB) hipLaunchKernelGGL((gemm_bf16<G, true, true, CF32>), grid, dim3(G::NTHR), 0, st, g);
 }
-template <typename G, bool CF32, int NS>
+template <typename G, bool CF32, int NS, bool SPREAD>
 void launch_ring_form(bool tA, bool tB, const GemmArgs& g, dim3 grid, hipStream_t st) {
-    if (!tA && !tB) hipLaunchKernelGGL((gemm_ring<G, false, false, CF32, NS>), grid, dim3(G::NTHR), 0, st, g);
-    if (!tA && tB) hipLaunchKernelGGL((gemm_ring<G, false, true, CF32, NS>), grid, dim3(G::NTHR), 0, st, g);
-    if (tA && !tB) hipLaunchKernelGGL((gemm_ring<G, true, false, CF32, NS>), grid, dim3(G::NTHR), 0, st, g);
-    if (tA && tB) hipLaunchKernelGGL((gemm_ring<G, true, true, CF32, NS>), grid, dim3(G::NTHR), 0, st, g);
+    if (!tA && !tB) hipLaunchKernelGGL((gemm_ring<G, false, false, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g);
+    if (!tA && tB) hipLaunchKernelGGL((gemm_ring<G, false, true, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g);
+    if (tA && !tB) hipLaunchKernelGGL((gemm_ring<G, true, false, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g);
+    if (tA && tB) hipLaunchKernelGGL((gemm_ring<G, true, true, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g);
 }
 int cu_count() {
     static const int n = [] {
@@ -727,10 +765,22 @@ void launch_ring(bool tA, bool tB, GemmArgs g, int S, bool c_f32, hipStream_t st
     const int64_t vblocks = static_cast<int64_t>((g.tiles_m * g.tiles_n + 7) / 8 * 8) * S;
     const int64_t slots = static_cast<int64_t>(cu_count()) / 8 * 8 * (RING <= 80 * 1024 ? 2 : 1);
     const unsigned gx = static_cast<unsigned>(std::min(vblocks, slots));
-    if (c_f32)
-        launch_ring_form<G, true, NS>(tA, tB, g, dim3(gx), st);
-    else
-        launch_ring_form<G, false, NS>(tA, tB, g, dim3(gx), st);
+    // When a slice's loads are issued. Spread behind the matrix instructions of the slice in hand they cost no issue
+    // time of their own, but the last of them then leaves late: a ring of two slots has only the rest of that slice
+    // to cover its latency, which pays where tiles change often (a short contraction, or the large tile whose slices
+    // take long) and costs 10 % in the steady state of a long one; three and more slots always have the slack.
+    const bool spread = NS > 2 || G::BM > 128 || std::min(g.K, g.k_per_split) <= 768;
+    if constexpr (NS > 2 || (G::BM > 128)) {
+        if (c_f32)
+            launch_ring_form<G, true, NS, true>(tA, tB, g, dim3(gx), st);
+        else
+            launch_ring_form<G, false, NS, true>(tA, tB, g, dim3(gx), st);
+    } else {
+        if (c_f32 && spread) launch_ring_form<G, true, NS, true>(tA, tB, g, dim3(gx), st);
+        if (c_f32 && !spread) launch_ring_form<G, true, NS, false>(tA, tB, g, dim3(gx), st);
+        if (!c_f32 && spread) launch_ring_form<G, false, NS, true>(tA, tB, g, dim3(gx), st);
+        if (!c_f32 && !spread) launch_ring_form<G, false, NS, false>(tA, tB, g, dim3(gx), st);
+    }
     hip_check(hipGetLastError(), "gemm_ring launch");
 }
 template <typename G>
@@ -782,10 +832,11 @@ Plan make_plan(bool tA, bool tB, int64_t M, int64_t N, int64_t K, int64_t lda, i
     // many slices as give every workgroup the chip holds at once one (tile, slice) -- a second round costs more than
     // longer slices -- but none shorter than 1024, since every slice is another partial product to write and add
     // (measured on [512, 1536], [512, 512], [512, 2752] and [1376, 512] outputs over 8192 tokens and on
-    // [2048, 512] over 32000). Split products take the 128 x 128 form with two workgroups per CU.
+    // [2048, 512] over 32000). Split products take 128 x 128 tiles: fewer than 64 of them in the two-set form, one
+    // workgroup of eight wavefronts per CU, otherwise two workgroups of four per CU.
     p.S = 1;
     if (ntiles < 192 && K >= 2048) {
-        if (ring_ok && g_force_geo < 0) p.ring = 6;
+        if (ring_ok && g_force_geo < 0) p.ring = ntiles < 64 ? 11 : 6;
         const bool one_per_cu = p.ring == 5 || p.ring == 7 || p.ring == 8 || p.ring == 10 || p.ring == 11;
         const int64_t s = std::min<int64_t>({(one_per_cu ? cu_count() : 2 * cu_count()) / ntiles, K / 1024, 16});
         p.S = static_cast<int>(std::max<int64_t>(s, 1));

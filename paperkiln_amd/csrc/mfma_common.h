@@ -233,6 +233,17 @@ __device__ inline void dma_group(uint32_t lds_byte, const uint32_t (&off)[PER], 
             "v"(off[0]), "v"(off[1]), "v"(off[2]), "v"(off[3]), "s"(rsrc), "s"(soff)
             : "memory");
 }
+// One piece of such a group on its own: the J-th 1 KB from `lds_byte` on (lane offset already less J KB), for kernels
+// that drop their loads one by one between other instructions. No "memory" clobber: the compiler may move its own LDS
+// reads across the statement (it keeps its place among the other volatile statements, the waits and barriers that
+// guard the slot it fills), which a clobber would forbid -- every piece would then fence the fragment reads of the
+// chunk after it from the matrix instructions of the chunk before.
+template <int J>
+__device__ inline void dma_piece(uint32_t lds_byte, uint32_t off, u32x4 rsrc, uint32_t soff) {
+    static_assert(J >= 0 && J < 4, "immediate offsets below 4096");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen offset:%4 lds" ::"s"(lds_byte), "v"(off),
+                 "s"(rsrc), "s"(soff), "n"(J * 1024));
+}
 template <int N>
 __device__ inline void wait_loads() {
     static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
