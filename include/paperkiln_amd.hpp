@@ -158,6 +158,9 @@ public:
     Tensor grad;  // allocated and zeroed on first accumulate(); fp32 for parameters, data's dtype otherwise
     bool requires_grad = false;
     bool is_param = false;
+    // grad's storage is also another Variable's grad (both parents of an add take the same tensor): it is read-only
+    // until own_grad() has given this Variable a copy of its own. accumulate(), ensure_grad() and zero_grad() do so.
+    bool grad_shared = false;
     std::vector<Var> parents;
     std::function<void()> backward_fn;
 
@@ -170,8 +173,9 @@ public:
     void accumulate(const Tensor& g, float a = 1.0f);  // grad += a * g (autograd.cpp:16-24)
     // The same for a temporary the caller is done with: the first contribution takes the buffer over instead of
     // copying it (the reference's lazily sized grad, autograd.cpp:17-19, makes that first += a copy as well).
-    void accumulate_owned(Tensor&& g);
+    void accumulate_owned(Tensor&& g, bool shared = false);
     Tensor& ensure_grad();                             // zero-filled grad of data's shape
+    Tensor& own_grad();                                // grad, after un-sharing it (call before writing into it in place)
 };
 
 size_t live_variables();  // autograd.hpp:61-64

@@ -461,9 +461,11 @@ __global__ void rms_bwd_dw_part8(const uint16_t* dy, const uint16_t* x, const fl
 // tensors): a wavefront takes ROWS_PB / 8 rows of its block, two at a time, lane l the columns 8 l .. 8 l + 7 of
 // every 512-column pass (NP passes, C <= 512 NP), keeps its rows' contribution to dW in registers, and the eight
 // wavefronts meet in LDS in a fixed order.
-template <int NP>
-__global__ void rms_bwd_dx_dw8(const uint16_t* dy, const uint16_t* x, const float* rinv, const float* w, uint16_t* dx,
-                               float* part, int64_t R, int C) {
+// ADD: dx = addend + (the above), the gradient that reached x along another path (a residual connection), added
+// before the one rounding to bf16.
+template <int NP, bool ADD>
+__global__ void rms_bwd_dx_dw8(const uint16_t* dy, const uint16_t* x, const float* rinv, const float* w,
+                               const uint16_t* addend, uint16_t* dx, float* part, int64_t R, int C) {
     constexpr int NWV = 8;            // wavefronts per block
     extern __shared__ float sh_dw[];  // [NWV - 1][C]: wavefronts 1 .. NWV - 1
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
@@ -480,7 +482,7 @@ __global__ void rms_bwd_dx_dw8(const uint16_t* dy, const uint16_t* x, const floa
     for (int64_t row = r0 + wv; row < r1; row += 2 * NWV) {
         const bool two = row + NWV < r1;
         const int64_t rows[2] = {row, two ? row + NWV : row};
-        F8 g[2][NP], v[2][NP];
+        F8 g[2][NP], v[2][NP], e[2][ADD ? NP : 1];
         float term[2] = {0.0f, 0.0f};
 #pragma unroll
         for (int q = 0; q < 2; ++q)
@@ -490,6 +492,7 @@ __global__ void rms_bwd_dx_dw8(const uint16_t* dy, const uint16_t* x, const floa
                 if (j < C) {
                     g[q][p] = ld8(dy + rows[q] * C, j);
                     v[q][p] = ld8(x + rows[q] * C, j);
+                    if (ADD) e[q][p] = ld8(addend + rows[q] * C, j);
                 }
             }
 #pragma unroll
@@ -516,6 +519,7 @@ __global__ void rms_bwd_dx_dw8(const uint16_t* dy, const uint16_t* x, const floa
 #pragma unroll
                     for (int k = 0; k < 8; ++k) {
                         o.v[k] = ri * (g[q][p].v[k] * ww[p].v[k] - v[q][p].v[k] * kk);
+                        if (ADD) o.v[k] += e[q][p].v[k];
                         acc[p].v[k] = fmaf(g[q][p].v[k] * v[q][p].v[k], ri, acc[p].v[k]);
                     }
                     st8(dx + rows[q] * C, j, o);
@@ -1014,18 +1018,27 @@ void k_rmsnorm_fwd(const Tensor& x, const Tensor& w, float eps, const Tensor& y,
     post();
 }
 void k_rmsnorm_bwd(const Tensor& dy, const Tensor& x, const float* rinv, const Tensor& w, const Tensor* dw,
-                   const Tensor* dx) {
+                   const Tensor* dx, const Tensor* addend) {
     const int C = static_cast<int>(x.cols);
+    if (addend && (!dx || addend->rows != x.rows || addend->cols != x.cols || addend->dtype != dx->dtype))
+        throw std::runtime_error("rmsnorm backward: the addend must have dx's shape and type");
     if (dx && dw && x.dtype == PK_BF16 && C % 8 == 0 && C <= 2048 && aligned16p(x.ptr()) && aligned16p(dy.ptr()) &&
-        aligned16p(dx->ptr()) && aligned16p(w.ptr())) {
+        aligned16p(dx->ptr()) && aligned16p(w.ptr()) && (!addend || aligned16p(addend->ptr()))) {
         const int nparts = static_cast<int>((x.rows + ROWS_PB - 1) / ROWS_PB);
         Buffer part(sizeof(float) * static_cast<size_t>(nparts) * C);
         const size_t lds = sizeof(float) * 7 * C;
         auto launch = [&](auto np) {
-            hipLaunchKernelGGL((rms_bwd_dx_dw8<decltype(np)::value>), dim3(nparts), dim3(512), lds, tape_stream(),
-                               static_cast<const uint16_t*>(dy.ptr()), static_cast<const uint16_t*>(x.ptr()), rinv,
-                               static_cast<const float*>(w.ptr()), static_cast<uint16_t*>(dx->ptr()),
-                               static_cast<float*>(part.p), x.rows, C);
+            constexpr int NP = decltype(np)::value;
+            if (addend)
+                hipLaunchKernelGGL((rms_bwd_dx_dw8<NP, true>), dim3(nparts), dim3(512), lds, tape_stream(),
+                                   static_cast<const uint16_t*>(dy.ptr()), static_cast<const uint16_t*>(x.ptr()), rinv,
+                                   static_cast<const float*>(w.ptr()), static_cast<const uint16_t*>(addend->ptr()),
+                                   static_cast<uint16_t*>(dx->ptr()), static_cast<float*>(part.p), x.rows, C);
+            else
+                hipLaunchKernelGGL((rms_bwd_dx_dw8<NP, false>), dim3(nparts), dim3(512), lds, tape_stream(),
+                                   static_cast<const uint16_t*>(dy.ptr()), static_cast<const uint16_t*>(x.ptr()), rinv,
+                                   static_cast<const float*>(w.ptr()), static_cast<const uint16_t*>(nullptr),
+                                   static_cast<uint16_t*>(dx->ptr()), static_cast<float*>(part.p), x.rows, C);
         };
         if (C <= 512)
             launch(std::integral_constant<int, 1>{});
@@ -1052,6 +1065,7 @@ void k_rmsnorm_bwd(const Tensor& dy, const Tensor& x, const float* rinv, const T
                                                         x.rows, C));
         }
         post();
+        if (addend) k_add(*dx, *addend, *dx);  // elementwise, so in place is fine
     }
     if (dw) {
         const int nparts = static_cast<int>((x.rows + ROWS_PB - 1) / ROWS_PB);

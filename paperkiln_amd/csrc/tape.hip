@@ -163,6 +163,16 @@ Tensor& Variable::ensure_grad() {
         grad = Tensor::make(data.rows, data.cols, is_param ? PK_F32 : data.dtype);
         k_fill(grad, 0.0f);
     }
+    return own_grad();
+}
+
+Tensor& Variable::own_grad() {
+    if (grad_shared && !grad.empty()) {
+        Tensor mine = Tensor::make(grad.rows, grad.cols, grad.dtype);
+        k_scale(grad, 1.0f, mine);
+        grad = std::move(mine);
+    }
+    grad_shared = false;
     return grad;
 }
 
@@ -170,18 +180,27 @@ void Variable::accumulate(const Tensor& g, float a) {
     if (g.rows != data.rows || g.cols != data.cols) shape_fail("accumulate: gradient shape mismatch");
     if (grad.empty()) {
         grad = Tensor::make(data.rows, data.cols, is_param ? PK_F32 : data.dtype);
+        grad_shared = false;
         k_scale(g, a, grad);  // first contribution: grad = a * g, no zero fill
         return;
     }
-    k_axpy(grad, a, g);
+    if (grad_shared && a == 1.0f && g.dtype == grad.dtype) {  // the sum goes into a tensor of this Variable's own
+        Tensor sum = Tensor::make(grad.rows, grad.cols, grad.dtype);
+        k_add(grad, g, sum);
+        grad = std::move(sum);
+        grad_shared = false;
+        return;
+    }
+    k_axpy(own_grad(), a, g);
 }
 
-void Variable::accumulate_owned(Tensor&& g) {
+void Variable::accumulate_owned(Tensor&& g, bool shared) {
     const int want = is_param ? PK_F32 : data.dtype;
-    const bool whole = g.buf && g.off_bytes == 0 && g.buf.use_count() == 1 &&
+    const bool whole = g.buf && g.off_bytes == 0 && (shared || g.buf.use_count() == 1) &&
                        g.buf->bytes == static_cast<size_t>(g.rows) * g.cols * g.esize();
     if (grad.empty() && whole && g.dtype == want && g.rows == data.rows && g.cols == data.cols) {
         grad = std::move(g);
+        grad_shared = shared;
         return;
     }
     accumulate(g);
@@ -214,8 +233,14 @@ void backward(const Var& root) {
 }
 
 void zero_grad(const std::vector<Var>& vars) {
-    for (const auto& v : vars)
-        if (!v->grad.empty()) k_fill(v->grad, 0.0f);
+    for (const auto& v : vars) {
+        if (v->grad.empty()) continue;
+        if (v->grad_shared) {  // a tensor of its own instead of zeroing the other holder's gradient
+            v->grad = Tensor::make(v->grad.rows, v->grad.cols, v->grad.dtype);
+            v->grad_shared = false;
+        }
+        k_fill(v->grad, 0.0f);
+    }
 }
 
 Var checkpoint(const std::function<Var(const Var&)>& fn, const Var& x) {
@@ -238,9 +263,10 @@ Var checkpoint(const std::function<Var(const Var&)>& fn, const Var& x) {
         Var rebuilt = segment(leaf);
         if (rebuilt->data.rows != raw->grad.rows || rebuilt->data.cols != raw->grad.cols)
             shape_fail("checkpoint: recomputed output shape mismatch");
-        rebuilt->accumulate_owned(std::move(raw->grad));
+        rebuilt->accumulate_owned(std::move(raw->grad), raw->grad_shared);
+        raw->grad_shared = false;
         run_backward(rebuilt);
-        if (input->requires_grad && !leaf->grad.empty()) input->accumulate_owned(std::move(leaf->grad));
+        if (input->requires_grad && !leaf->grad.empty()) input->accumulate_owned(std::move(leaf->grad), leaf->grad_shared);
     };
     return node;
 }
@@ -315,9 +341,23 @@ Var add(const Var& a, const Var& b) {
     Tensor y = Tensor::make(a->data.rows, a->data.cols, a->data.dtype);
     k_add(a->data, b->data, y);
     return record(std::move(y), {a, b}, [](Variable* self) {
-        // one parent gets a copy (or an axpy), the other takes the tensor itself
-        if (self->parents[0]->requires_grad) self->parents[0]->accumulate(self->grad);
-        if (self->parents[1]->requires_grad) self->parents[1]->accumulate_owned(std::move(self->grad));
+        // Both parents take the tensor itself where they can: it is the gradient of either, shared and read-only
+        // until one of them has to write (a parameter, or a parent that has a gradient already, gets a copy or
+        // an axpy instead).
+        const Var& a = self->parents[0];
+        const Var& b = self->parents[1];
+        const bool both = a->requires_grad && b->requires_grad && a != b;
+        const bool share = both && !a->is_param && !b->is_param && a->grad.empty() && b->grad.empty() &&
+                           a->data.dtype == self->grad.dtype && b->data.dtype == self->grad.dtype;
+        const bool was_shared = self->grad_shared;
+        self->grad_shared = false;
+        if (share) {
+            a->accumulate_owned(Tensor(self->grad), true);
+            b->accumulate_owned(std::move(self->grad), true);
+            return;
+        }
+        if (a->requires_grad) a->accumulate(self->grad);
+        if (b->requires_grad) b->accumulate_owned(std::move(self->grad), was_shared);
     });
 }
 
@@ -400,9 +440,17 @@ Var rmsnorm(const Var& x, const Var& w) {
         Tensor dx;
         if (x->requires_grad) dx = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
         Tensor* dw = w->requires_grad ? &w->ensure_grad() : nullptr;
+        // x usually has the residual branch's gradient already: the kernel adds it on the way out (one rounding of
+        // the sum instead of two) and the result replaces it, which also leaves a shared tensor untouched
+        const bool onto = x->requires_grad && !x->is_param && !x->grad.empty() && x->grad.dtype == dx.dtype;
         k_rmsnorm_bwd(self->grad, x->data, static_cast<const float*>(rinv->p), w->data, dw,
-                      x->requires_grad ? &dx : nullptr);
-        if (x->requires_grad) x->accumulate_owned(std::move(dx));
+                      x->requires_grad ? &dx : nullptr, onto ? &x->grad : nullptr);
+        if (onto) {
+            x->grad = std::move(dx);
+            x->grad_shared = false;
+        } else if (x->requires_grad) {
+            x->accumulate_owned(std::move(dx));
+        }
     });
 }
 
@@ -417,7 +465,7 @@ Var apply_rope(const Var& qkv, const std::shared_ptr<Buffer>& pos, float theta, 
         return record(Tensor(qkv->data), {qkv}, [pos, theta, head_dim, rot_heads, d](Variable* self) {
             const Var& x = self->parents[0];
             if (!x->requires_grad) return;
-            k_rope_inplace(self->grad, static_cast<const int*>(pos->p), theta, d, head_dim, rot_heads, true);
+            k_rope_inplace(self->own_grad(), static_cast<const int*>(pos->p), theta, d, head_dim, rot_heads, true);
             x->accumulate_owned(std::move(self->grad));
             self->grad = Tensor();
         });
@@ -676,7 +724,7 @@ double clip_grad_norm(const std::vector<Var>& params, float max_norm) {
     if (total > max_norm && total > 0.0) {
         const float s = static_cast<float>(max_norm / total);
         for (const auto& p : params)
-            if (!p->grad.empty()) k_scale(p->grad, s, p->grad);
+            if (!p->grad.empty()) k_scale(p->own_grad(), s, p->grad);
     }
     return total;
 }

@@ -28,8 +28,9 @@ void k_silu_mul_bwd(const Tensor& gate, const Tensor& up, const Tensor& dy, cons
 void k_silu_mul_cat_fwd(const Tensor& gu, const Tensor& y);
 void k_silu_mul_cat_bwd(const Tensor& gu, const Tensor& dy, const Tensor& dgu);
 void k_rmsnorm_fwd(const Tensor& x, const Tensor& w, float eps, const Tensor& y, float* rinv);  // ops.cpp:437-445
+// ops.cpp:447-478; with an addend (dx's shape and type) dx = addend + the gradient through the norm
 void k_rmsnorm_bwd(const Tensor& dy, const Tensor& x, const float* rinv, const Tensor& w, const Tensor* dw_f32,
-                   const Tensor* dx);                                   // ops.cpp:447-478
+                   const Tensor* dx, const Tensor* addend = nullptr);
 // apply_rope on a fused [N, 3d] matrix (ops.cpp:481-537): rotates adjacent pairs of the
 // first `rot_heads` heads of the q third and of the k third; inverse = backward.
 void k_rope(const Tensor& x, const int* pos, float theta, int d, int head_dim, int rot_heads, bool inverse,

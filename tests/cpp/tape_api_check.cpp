@@ -199,6 +199,64 @@ void checkpoint_case() {
     std::printf("  live variables after forward: plain %zu, checkpointed %zu\n", plain.live, ck.live);
 }
 
+// Gradients that reach a Variable along two paths. Both parents of an add take the node's gradient tensor itself
+// (shared, read-only), so writing one parent's gradient afterwards -- a later accumulation, zero_grad -- must not
+// show in the other's; and rmsnorm's backward adds the gradient its input already has inside the kernel.
+void shared_gradient_case(int dtype, const char* name, double tol) {
+    std::printf("gradients along two paths, %s\n", name);
+    const int T = 48, d = 64;
+    const auto hx = draw(static_cast<size_t>(T) * d, 41, 1.0), hu = draw(static_cast<size_t>(T) * d, 42, 1.0),
+               hg = draw(d, 43, 1.0);
+    std::vector<int> target(T);
+    for (int i = 0; i < T; ++i) target[i] = (7 * i + 3) % d;
+    auto tg = device_ints(target);
+    auto diff = [](const std::vector<float>& a, const std::vector<float>& b, double fb) {
+        double w = 0.0;
+        for (size_t i = 0; i < a.size(); ++i) w = std::fmax(w, std::fabs(static_cast<double>(a[i]) - fb * b[i]));
+        return w;
+    };
+    {
+        pk::Var x = pk::make_var(pk::upload(hx.data(), T, d, dtype), true);
+        pk::Var u = pk::make_var(pk::upload(hu.data(), T, d, dtype), true);
+        auto pass = [&] { pk::backward(pk::ops::cross_entropy(pk::ops::add(x, u), tg)); };
+        pass();
+        const auto g1 = host(x->grad);
+        double size = 0.0;
+        for (float v : g1) size = std::fmax(size, std::fabs(v));
+        check(size > 1e-4, "add: the gradient is not zero", size);
+        check(host(u->grad) == g1, "add: both parents hold the node's gradient", 0.0);
+        pass();  // accumulates onto gradients that share storage
+        check(diff(host(x->grad), g1, 2.0) <= tol * size, "second backward doubles the first parent's", diff(host(x->grad), g1, 2.0));
+        check(diff(host(u->grad), g1, 2.0) <= tol * size, "... and the second parent's, once each", diff(host(u->grad), g1, 2.0));
+        pk::Var x2 = pk::make_var(pk::upload(hx.data(), T, d, dtype), true);
+        pk::Var u2 = pk::make_var(pk::upload(hu.data(), T, d, dtype), true);
+        pk::backward(pk::ops::cross_entropy(pk::ops::add(x2, u2), tg));
+        pk::zero_grad({x2});
+        check(diff(host(x2->grad), g1, 0.0) == 0.0, "zero_grad of one parent zeroes it", 0.0);
+        check(host(u2->grad) == g1, "... and leaves the other parent's gradient alone", 0.0);
+    }
+    {
+        // z = x + rmsnorm(x): one Variable on both paths against two leaves with the same values, one per path
+        pk::Var gain = pk::make_var(pk::upload(hg.data(), 1, d), true);
+        gain->is_param = true;
+        pk::Var x = pk::make_var(pk::upload(hx.data(), T, d, dtype), true);
+        pk::backward(pk::ops::cross_entropy(pk::ops::add(x, pk::ops::rmsnorm(x, gain)), tg));
+        const auto both = host(x->grad), gg = host(gain->grad);
+        pk::zero_grad({gain});
+        pk::Var xa = pk::make_var(pk::upload(hx.data(), T, d, dtype), true);
+        pk::Var xb = pk::make_var(pk::upload(hx.data(), T, d, dtype), true);
+        pk::backward(pk::ops::cross_entropy(pk::ops::add(xa, pk::ops::rmsnorm(xb, gain)), tg));
+        const auto ga = host(xa->grad), gb = host(xb->grad);
+        double w = 0.0, size = 0.0;
+        for (size_t i = 0; i < both.size(); ++i) {
+            w = std::fmax(w, std::fabs(static_cast<double>(both[i]) - (static_cast<double>(ga[i]) + gb[i])));
+            size = std::fmax(size, std::fabs(static_cast<double>(ga[i]) + gb[i]));
+        }
+        check(w <= tol * size, "x + rmsnorm(x): gradient = residual path + norm path", w);
+        check(diff(host(gain->grad), gg, 1.0) <= 1e-6, "gain gradient the same either way", diff(host(gain->grad), gg, 1.0));
+    }
+}
+
 void behaviour_case() {
     std::printf("tape behaviour and errors\n");
     const auto h = draw(8 * 4, 31, 1.0);
@@ -252,6 +310,8 @@ int main() {
     attention_case("fused_attention, head_dim 32 (fp32 matrix-core kernels)", 40, 32, 20, true, 0, 0);
     attention_case("swa_attention, window 3 + 2 sinks", 18, 8, 9, true, 3, 2);
     checkpoint_case();
+    shared_gradient_case(PK_F32, "float32", 1e-6);
+    shared_gradient_case(PK_BF16, "bfloat16 (the fused row kernel)", 1.0 / 128);
     behaviour_case();
     if (g_failures == 0) {
         std::printf("tape_api_check PASSED\n");
