@@ -262,6 +262,13 @@ int pk_op_gemm(const void* a, int trans_a, const void* b, int trans_b, void* c, 
  * and 2, 3, 4 slots. Process-wide; returns the previous setting (0, 1 or 2). The environment variable
  * PK_GEMM=library selects 0 at load time. */
 int pk_set_gemm_backend(int mode);
+/* How the chunked tied head (llama.cpp:88 followed by ops::cross_entropy, src/ops.cpp:350-376) forms the loss and
+ * dlogits from bf16 operands. 1 (default): inside the logits product -- the library's own GEMM forms every tile of
+ * logits twice, first for the rows' maxima and sums of exponentials (and the loss), then to emit bf16 dlogits, and the
+ * [rows, vocab] logits never reach memory. 0: one logits product into an fp32 matrix and a row kernel over it (also
+ * what fp32 operands, rocBLAS-only mode and shapes the own GEMM does not take get). Process-wide; returns the previous
+ * setting. */
+int pk_set_head_kernel(int in_product);
 
 #ifdef __cplusplus
 }

@@ -53,7 +53,7 @@ EXPORTS = ["pk_last_error", "pk_init", "pk_attn_fwd", "pk_attn_bwd_workspace_byt
            "pk_llama_set_head_chunk",
            "pk_op_add", "pk_op_mul", "pk_op_scale", "pk_op_axpy", "pk_op_fill", "pk_op_silu_fwd", "pk_op_silu_bwd", "pk_op_silu_mul_fwd", "pk_op_silu_mul_bwd",
            "pk_op_rmsnorm_fwd", "pk_op_rmsnorm_bwd", "pk_op_rope", "pk_op_embedding_fwd", "pk_op_embedding_bwd",
-           "pk_op_cross_entropy", "pk_op_adamw", "pk_op_sumsq", "pk_op_gemm", "pk_set_gemm_backend"]
+           "pk_op_cross_entropy", "pk_op_adamw", "pk_op_sumsq", "pk_op_gemm", "pk_set_gemm_backend", "pk_set_head_kernel"]
 
 
 def lib() -> C.CDLL:
@@ -115,6 +115,7 @@ def lib() -> C.CDLL:
         L.pk_op_sumsq.argtypes = [vp, i64, C.POINTER(C.c_double), vp]
         L.pk_op_gemm.argtypes = [vp, ci, vp, ci, vp, i64, i64, i64, ci, ci, ci, vp]
         L.pk_set_gemm_backend.argtypes = [ci]
+        L.pk_set_head_kernel.argtypes = [ci]
         _lib = L
     return _lib
 

@@ -188,6 +188,13 @@ def clip_grad_norm_(grads, max_norm):
     return total
 
 
+def set_head_kernel(in_product: bool) -> int:
+    """How the chunked tied head forms loss and dlogits from bf16 operands (pk_set_head_kernel): True (default) =
+    inside the logits product, the logits never stored; False = an fp32 logits matrix and a row kernel over it.
+    Returns the previous setting."""
+    return int(_lib.lib().pk_set_head_kernel(1 if in_product else 0))
+
+
 def set_gemm_backend(mode: int) -> int:
     """Choose the kernel for bf16 GEMMs (pk_set_gemm_backend): 1 (default) and 2 = the library's own matrix-core
     kernel wherever it applies, in the form it picks per shape, 0 = rocBLAS only, 3 .. 11 = the own kernel

@@ -1222,6 +1222,11 @@ std::atomic<int> g_gemm_hand_written{[] {
 }
 void set_gemm_backend(int hand_written) { g_gemm_hand_written.store(hand_written, std::memory_order_relaxed); }
 int gemm_backend() { return g_gemm_hand_written.load(std::memory_order_relaxed); }
+namespace {
+std::atomic<int> g_head_in_product{1};
+}
+void set_head_kernel(int in_product) { g_head_in_product.store(in_product != 0, std::memory_order_relaxed); }
+int head_kernel() { return g_head_in_product.load(std::memory_order_relaxed); }
 
 void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dtype, int64_t M, int64_t N, int64_t ldc,
           float beta, int64_t lda) {

@@ -66,6 +66,20 @@ struct GemmArgs {
     int splits;  // slices of the contraction (gemm_ring walks them itself; gemm_bf16 takes them from blockIdx.z)
 };
 
+// What the two passes of the tied head's cross-entropy do with a tile of logits instead of storing it (gemm_ring's
+// EPI parameter). Pass 1: per row and per 64-column span of a wavefront, the span's maximum and its sum of
+// exp(z - maximum), to stats[span][row], and the target column's logit to zt[row]. Pass 2: the same tile formed
+// again, turned into dlogits = (exp(z - row_max) row_inv - [column == target]) gscale and stored as bf16.
+struct HeadArgs {
+    const int* target;     // [M]
+    float2* stats;         // pass 1: [spans][M]
+    float* zt;             // pass 1: [M]
+    const float* row_max;  // pass 2: [M]
+    const float* row_inv;  // pass 2: [M], 1 / sum_j exp(z_j - row_max)
+    float gscale;          // pass 2
+};
+constexpr float LOG2E = 1.4426950408889634f;
+
 // Transposing operand read in natural k order: lane (c32, g) receives rows row0 + 8g .. 8g + 7 of column
 // col0 + c32 of a [k][column] tile.
 __device__ inline bf16x8 read_tr_nat(const uint16_t* tile, int pitch, int row0, int col0, int lane) {
@@ -354,9 +368,10 @@ struct TileStore {
 // (virtual block -> (contraction slice, tile) as gemm_bf16 maps (blockIdx.z, blockIdx.x), XCD by XCD), and the ring
 // runs on across tile boundaries: the first slices of the next tile are on their way while the last ones of this tile
 // are multiplied and its result is stored, so a tile's first round trip to memory is paid once per workgroup.
-template <typename G, bool TA, bool TB, bool CF32, int NS, bool SPREAD>
+template <typename G, bool TA, bool TB, bool CF32, int NS, bool SPREAD, int EPI = 0>
 __global__ __launch_bounds__(G::NTHR, NS * (RingOp<TA, G::BM, G::NTHR / 64>::BYTES + RingOp<!TB, G::BN, G::NTHR / 64>::BYTES) <= 80 * 1024 ? 2 : 1)
-void gemm_ring(GemmArgs g) {
+void gemm_ring(GemmArgs g, HeadArgs hd) {
+    static_assert(EPI == 0 || (G::KS == 1 && !CF32), "the head's epilogues: one wavefront set, bf16 result");
     constexpr int BM = G::BM, BN = G::BN, NTHR = G::NTHR, FM = G::FM, FN = G::FN, NW = NTHR / 64;
     using OA = RingOp<TA, BM, NW>;
     using OB = RingOp<!TB, BN, NW>;
@@ -540,6 +555,63 @@ void gemm_ring(GemmArgs g) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
     };
+    // lane (c32, gh) holds, of row (wm FM + i) 32 + c32 of the tile, columns (wn FN + j) 32 + 8 qd + 4 gh + e
+    auto head_stats = [&](const Block& bl) {  // EPI 1
+        const int span = (bl.n0 / BN) * G::WGN + wn, col0 = bl.n0 + wn * FN * 32 + gh * 4;
+        if (bl.n0 + BN > g.N) {  // wavefront-uniform: columns past the matrix count for nothing
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        if (col0 + j * 32 + (r >> 2) * 8 + (r & 3) >= g.N) acc[i][j][r] = -INFINITY;
+        }
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            const int row = bl.m0 + (wm * FM + i) * 32 + c32;
+            // the target's place among this lane's 16 FN sums of the row, if it is there: 16 j + r
+            const int tt = (row < g.M ? hd.target[row] : -1) - (bl.n0 + wn * FN * 32);
+            const bool has = tt >= 0 && tt < FN * 32 && ((tt >> 2) & 1) == gh && row < g.M;
+            const int at = has ? (tt >> 5) * 16 + ((tt >> 3) & 3) * 4 + (tt & 3) : -1;
+            float mx = -INFINITY, zt = 0.0f;
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    mx = fmaxf(mx, acc[i][j][r]);
+                    zt = at == j * 16 + r ? acc[i][j][r] : zt;
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float ref = mx == -INFINITY ? 0.0f : mx * LOG2E;  // a span wholly past the last column sums to 0
+            float sum = 0.0f;
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sum += __builtin_amdgcn_exp2f(fmaf(acc[i][j][r], LOG2E, -ref));
+            sum += __shfl_xor(sum, 32);
+            if (row < g.M && gh == 0) hd.stats[static_cast<int64_t>(span) * g.M + row] = make_float2(mx, sum);
+            if (has) hd.zt[row] = zt;
+        }
+    };
+    auto head_dlogits = [&](const Block& bl) {  // EPI 2: the sums become dlogits where they lie
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            const int row = bl.m0 + (wm * FM + i) * 32 + c32;
+            const bool in = row < g.M;
+            const int tt = (in ? hd.target[row] : -1) - (bl.n0 + wn * FN * 32);
+            const bool has = tt >= 0 && tt < FN * 32 && ((tt >> 2) & 1) == gh && in;
+            const int at = has ? (tt >> 5) * 16 + ((tt >> 3) & 3) * 4 + (tt & 3) : -1;
+            const float ref = in ? hd.row_max[row] * LOG2E : 0.0f, inv = in ? hd.row_inv[row] : 0.0f;
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float p = __builtin_amdgcn_exp2f(fmaf(acc[i][j][r], LOG2E, -ref)) * inv;
+                    acc[i][j][r] = (p - (at == j * 16 + r ? 1.0f : 0.0f)) * hd.gscale;
+                }
+        }
+    };
     // the tile's result, through the ring slot `strip` (which every wavefront has finished reading)
     auto store_result = [&](uint8_t* strip, const Block& bl) {
         if (KS == 2) {  // set 1 hands its sums to set 0, half of them at a time: [wavefront][16-byte group][lane]
@@ -687,9 +759,14 @@ void gemm_ring(GemmArgs g) {
             if constexpr (KPW > 3) chunk(std::integral_constant<int, 3>{});
             fetch_end();
             if (++c_slice == c_nslices) {  // wavefront-uniform
-                barrier();  // every wavefront has read slot u: it takes the result on its way out
-                store_result(lds + u * SLOT, cb);
-                since_store = 0;
+                if constexpr (EPI == 1) {
+                    head_stats(cb);  // nothing goes through the slot, and no store joins the count of loads in flight
+                } else {
+                    if constexpr (EPI == 2) head_dlogits(cb);
+                    barrier();  // every wavefront has read slot u: it takes the result on its way out
+                    store_result(lds + u * SLOT, cb);
+                    since_store = 0;
+                }
                 cv = next_block(cv + stride, cb);
                 if (cv >= V) {
                     done = true;
@@ -730,6 +807,35 @@ __global__ void sum_slices(const float* part, void* dst, int nparts, int64_t par
     }
 }
 
+// Joins a row's span statistics of the head's first pass, in span order: the row's maximum M, 1 / sum_j exp(z_j - M)
+// and its loss -log(max(P_target, 1e-12)) (src/ops.cpp:360-368). 64 rows x 16 groups of spans per block.
+__global__ __launch_bounds__(1024) void head_rows(const float2* stats, const float* zt, int spans, int M, float* row_max,
+                                                  float* row_inv, float* nll) {
+    __shared__ float sh_m[16][64], sh_s[16][64];
+    const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6, r = blockIdx.x * 64 + lane;
+    auto join = [](float& m, float& s, float m2, float s2) {
+        const float nm = fmaxf(m, m2), ref = nm == -INFINITY ? 0.0f : nm;
+        s = s * __builtin_amdgcn_exp2f((m - ref) * LOG2E) + s2 * __builtin_amdgcn_exp2f((m2 - ref) * LOG2E);
+        m = nm;
+    };
+    float m = -INFINITY, s = 0.0f;
+    if (r < M)
+        for (int p = grp; p < spans; p += 16) {
+            const float2 v = stats[static_cast<int64_t>(p) * M + r];
+            join(m, s, v.x, v.y);
+        }
+    sh_m[grp][lane] = m;
+    sh_s[grp][lane] = s;
+    __syncthreads();
+    if (grp == 0 && r < M) {
+        for (int q = 1; q < 16; ++q) join(m, s, sh_m[q][lane], sh_s[q][lane]);
+        const float inv = 1.0f / s;
+        row_max[r] = m;
+        row_inv[r] = inv;
+        nll[r] = -logf(fmaxf(__builtin_amdgcn_exp2f((zt[r] - m) * LOG2E) * inv, 1e-12f));
+    }
+}
+
 template <typename G, bool CF32>
 void launch_form(bool tA, bool tB, const GemmArgs& g, dim3 grid, hipStream_t st) {
     if (!tA && !tB) hipLaunchKernelGGL((gemm_bf16<G, false, false, CF32>), grid, dim3(G::NTHR), 0, st, g);
@@ -739,10 +845,10 @@ void launch_form(bool tA, bool tB, const GemmArgs& g, dim3 grid, hipStream_t st)
 }
 template <typename G, bool CF32, int NS, bool SPREAD>
 void launch_ring_form(bool tA, bool tB, const GemmArgs& g, dim3 grid, hipStream_t st) {
-    if (!tA && !tB) hipLaunchKernelGGL((gemm_ring<G, false, false, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g);
-    if (!tA && tB) hipLaunchKernelGGL((gemm_ring<G, false, true, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g);
-    if (tA && !tB) hipLaunchKernelGGL((gemm_ring<G, true, false, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g);
-    if (tA && tB) hipLaunchKernelGGL((gemm_ring<G, true, true, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g);
+    if (!tA && !tB) hipLaunchKernelGGL((gemm_ring<G, false, false, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g, HeadArgs{});
+    if (!tA && tB) hipLaunchKernelGGL((gemm_ring<G, false, true, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g, HeadArgs{});
+    if (tA && !tB) hipLaunchKernelGGL((gemm_ring<G, true, false, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g, HeadArgs{});
+    if (tA && tB) hipLaunchKernelGGL((gemm_ring<G, true, true, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g, HeadArgs{});
 }
 int cu_count() {
     static const int n = [] {
@@ -928,6 +1034,64 @@ bool gemm_mfma_bf16_parts(const void* a, bool tA, int64_t lda, const void* b, bo
     g.part_stride = p.S > 1 ? M * N : 0;
     run_plan(p, tA, tB, g, p.S, true, st);
     nparts = p.S;
+    return true;
+}
+
+// ---- the tied head's cross-entropy inside its logits product ----
+namespace {
+bool head_takes(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K) {
+    if (!takes(a, false, lda, b, ldb, M, N, K)) return false;
+    const int64_t ext_max = (int64_t{1} << 30) - 8192;
+    return M * lda * 2 < ext_max && N * ldb * 2 < ext_max && lda < (1 << 21) && ldb < (1 << 21) && N < (1 << 20);
+}
+template <int EPI>
+void launch_head(GemmArgs g, const HeadArgs& hd, hipStream_t st) {
+    using G = GeoLarge;
+    g.tiles_m = (g.M + G::BM - 1) / G::BM;
+    g.tiles_n = (g.N + G::BN - 1) / G::BN;
+    g.splits = 1;
+    const int64_t vblocks = static_cast<int64_t>((g.tiles_m * g.tiles_n + 7) / 8 * 8);
+    const unsigned gx = static_cast<unsigned>(std::min<int64_t>(vblocks, cu_count() / 8 * 8));
+    hipLaunchKernelGGL((gemm_ring<G, false, true, false, 2, true, EPI>), dim3(gx), dim3(G::NTHR), 0, st, g, hd);
+    hip_check(hipGetLastError(), "gemm_ring (head) launch");
+}
+}  // namespace
+
+int64_t gemm_head_spans(int64_t N) { return (N + GeoLarge::BN - 1) / GeoLarge::BN * GeoLarge::WGN; }
+
+// Pass 1 over logits = A B^T (A [M, K] and B [N, K], bf16), which are formed tile by tile and never stored: per row
+// its maximum, 1 / sum exp(z - maximum) and its loss against target[row]. `stats` is scratch of gemm_head_spans(N) * M
+// pairs of floats, `zt` of M floats. False, with nothing done, for operands the kernel does not take.
+bool gemm_head_rows(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K, const int* target,
+                    void* stats, float* zt, float* row_max, float* row_inv, float* nll, hipStream_t st) {
+    if (!head_takes(a, lda, b, ldb, M, N, K)) return false;
+    GemmArgs g = gemm_args(a, lda, b, ldb, M, N, K);
+    HeadArgs hd{};
+    hd.target = target;
+    hd.stats = static_cast<float2*>(stats);
+    hd.zt = zt;
+    launch_head<1>(g, hd, st);
+    hipLaunchKernelGGL(head_rows, dim3(static_cast<unsigned>((M + 63) / 64)), dim3(1024), 0, st, hd.stats, zt,
+                       static_cast<int>(gemm_head_spans(N)), static_cast<int>(M), row_max, row_inv, nll);
+    hip_check(hipGetLastError(), "head_rows launch");
+    return true;
+}
+
+// Pass 2: the same tiles again, stored as dlogits[M, N] (bf16, row pitch ldc) =
+// (exp(z - row_max) row_inv - [column == target]) gscale (src/ops.cpp:371-374).
+bool gemm_head_dlogits(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                       const int* target, const float* row_max, const float* row_inv, float gscale, void* dl, int64_t ldc,
+                       hipStream_t st) {
+    if (!head_takes(a, lda, b, ldb, M, N, K) || !aligned16(dl) || ldc % 8 || ldc >= (1 << 20)) return false;
+    GemmArgs g = gemm_args(a, lda, b, ldb, M, N, K);
+    g.c = dl;
+    g.ldc = ldc;
+    HeadArgs hd{};
+    hd.target = target;
+    hd.row_max = row_max;
+    hd.row_inv = row_inv;
+    hd.gscale = gscale;
+    launch_head<2>(g, hd, st);
     return true;
 }
 

@@ -171,6 +171,11 @@ int pk_set_gemm_backend(int hand_written) {
     gemm_mfma_force_tiles(hand_written == 3 ? 0 : hand_written == 4 ? 1 : hand_written >= 5 ? hand_written : -1);
     return before;
 }
+int pk_set_head_kernel(int in_product) {
+    const int before = head_kernel();
+    set_head_kernel(in_product);
+    return before;
+}
 int pk_op_gemm(const void* a, int trans_a, const void* b, int trans_b, void* c, int64_t m, int64_t n, int64_t k,
                int dtype, int c_dtype, int accumulate, void* stream) {
     return op_guard(stream, [&] {

@@ -659,30 +659,49 @@ Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffe
     const Tensor& Ec = shadow_of(E);
     Buffer nll(sizeof(float) * N);
     const float g1 = 1.0f / static_cast<float>(N);
+    const bool grads = want_dh || want_dE;
+    // bf16 operands the library's own GEMM takes: the cross-entropy runs inside the logits product, which forms
+    // every tile twice (row statistics and loss, then dlogits) instead of storing [rows, V] logits for a row kernel
+    bool in_product = h->data.dtype == PK_BF16 && Ec.dtype == PK_BF16 && head_kernel() != 0 && gemm_backend() != 0;
     for (int64_t r0 = 0; r0 < N; r0 += chunk_rows) {
         const int64_t rows = std::min(chunk_rows, N - r0);
         const Tensor hview = h->data.row_range(r0, rows);
-        Tensor logits = Tensor::make(rows, V, PK_F32);
-        gemm(hview, false, Ec, true, logits.ptr(), PK_F32, rows, V, V, 0.0f);
         float* nll_r = static_cast<float*>(nll.p) + r0;
-        const bool grads = want_dh || want_dE;
-        // dlogits takes the place of the logits it came from: in fp32 the same matrix, in bf16 the first half of
-        // every fp32 row (row pitch 2V bf16 elements), so a chunk holds one [rows, V] fp32 buffer and nothing else.
         Tensor dl;
         int64_t dl_ld = V;
-        if (grads) {
-            dl = logits;
-            if (h->data.dtype != PK_F32) {
-                dl.dtype = h->data.dtype;
-                dl_ld = 2 * V;
+        if (in_product) {
+            Buffer stats(sizeof(float) * 2 * static_cast<size_t>(gemm_head_spans(V)) * rows), rowf(sizeof(float) * 3 * rows);
+            float* zt = static_cast<float*>(rowf.p);
+            float* row_max = zt + rows;
+            float* row_inv = row_max + rows;
+            in_product = gemm_head_rows(hview.ptr(), d, Ec.ptr(), d, rows, V, d, tg + r0, stats.p, zt, row_max, row_inv, nll_r,
+                                        tape_stream());
+            if (in_product && grads) {
+                dl = Tensor::make(rows, V, PK_BF16);
+                if (!gemm_head_dlogits(hview.ptr(), d, Ec.ptr(), d, rows, V, d, tg + r0, row_max, row_inv, g1, dl.ptr(), V,
+                                       tape_stream()))
+                    throw std::runtime_error("linear_cross_entropy: the head's second pass refused what its first took");
             }
         }
-        if (!k_ce_rows_once(logits, tg + r0, g1, nll_r, grads ? &dl : nullptr, dl_ld)) {
-            k_ce_rows(logits, tg + r0, g1, nll_r);  // generic row kernel: dlogits in place as fp32
-            if (grads && h->data.dtype != PK_F32) {
-                dl = Tensor::make(rows, V, h->data.dtype);
-                dl_ld = V;
-                k_cast(logits, dl);
+        if (!in_product) {
+            Tensor logits = Tensor::make(rows, V, PK_F32);
+            gemm(hview, false, Ec, true, logits.ptr(), PK_F32, rows, V, V, 0.0f);
+            // dlogits takes the place of the logits it came from: in fp32 the same matrix, in bf16 the first half of
+            // every fp32 row (row pitch 2V bf16 elements), so a chunk holds one [rows, V] fp32 buffer and nothing else.
+            if (grads) {
+                dl = logits;
+                if (h->data.dtype != PK_F32) {
+                    dl.dtype = h->data.dtype;
+                    dl_ld = 2 * V;
+                }
+            }
+            if (!k_ce_rows_once(logits, tg + r0, g1, nll_r, grads ? &dl : nullptr, dl_ld)) {
+                k_ce_rows(logits, tg + r0, g1, nll_r);  // generic row kernel: dlogits in place as fp32
+                if (grads && h->data.dtype != PK_F32) {
+                    dl = Tensor::make(rows, V, h->data.dtype);
+                    dl_ld = V;
+                    k_cast(logits, dl);
+                }
             }
         }
         if (want_dh)

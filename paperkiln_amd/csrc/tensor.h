@@ -68,12 +68,26 @@ bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB,
 // output alone would leave the chip idle), for a caller that adds them on the way to where the result goes.
 bool gemm_mfma_bf16_parts(const void* a, bool tA, int64_t lda, const void* b, bool tB, int64_t ldb, int64_t M, int64_t N,
                           int64_t K, hipStream_t st, std::unique_ptr<Buffer>& part, int& nparts);
-// Which GEMM serves bf16 operands: 1 (default) = each shape class goes to the kernel that measured faster for it,
-// 0 = the library only, 2 = the hand-written kernel for everything it takes. Set from the environment
+// The tied head's cross-entropy inside its logits product A B^T (bf16 [M, K] and [N, K]): the logits are formed tile
+// by tile, twice, and never stored. gemm_head_rows: per row the maximum, 1 / sum exp(z - maximum) and the loss
+// (stats: scratch of gemm_head_spans(N) * M float pairs, zt: of M floats); gemm_head_dlogits: bf16 dlogits.
+// Both return false, having done nothing, for operands the kernel does not take.
+int64_t gemm_head_spans(int64_t N);
+bool gemm_head_rows(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K, const int* target,
+                    void* stats, float* zt, float* row_max, float* row_inv, float* nll, hipStream_t st);
+bool gemm_head_dlogits(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                       const int* target, const float* row_max, const float* row_inv, float gscale, void* dl, int64_t ldc,
+                       hipStream_t st);
+// Which GEMM serves bf16 operands: 1 (default) and 2 = the hand-written kernel for everything it takes,
+// 0 = the library only. Set from the environment
 // (PK_GEMM=library) or by a caller that wants to compare them.
 void set_gemm_backend(int hand_written);
 void gemm_mfma_force_tiles(int which);  // -1: by shape (default); 0, 1, 5 .. 11: one kernel form always (measurement)
 int gemm_backend();
+// How the chunked tied head forms its cross-entropy from bf16 operands: 1 (default) = inside the logits product
+// (gemm_head_rows / gemm_head_dlogits: no logits in memory), 0 = a logits product into fp32 and a row kernel over it.
+void set_head_kernel(int in_product);
+int head_kernel();
 // dst[k] ([A.cols, B.cols/nsplit] fp32, contiguous) = beta * dst[k] + A^T B[:, k-th column block], k < nsplit <= 4
 void gemm_tn_split(const Tensor& A, const Tensor& B, float* const* dst, int nsplit, float beta);
 

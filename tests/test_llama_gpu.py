@@ -7,7 +7,7 @@ import os
 import numpy as np
 import pytest
 
-from paperkiln_amd import synth
+from paperkiln_amd import blockops, synth
 from paperkiln_amd.llama import Llama
 
 pytestmark = pytest.mark.gpu
@@ -194,51 +194,70 @@ def reldiff(a, b):
     return max(errs) if np.all(np.isfinite(errs)) else float("inf")
 
 
-# (dtype, vocab, tokens, seq_len, rows per head chunk or None = the library's default of 2048)
+# (dtype, vocab, tokens, seq_len, rows per head chunk or None = the library's default of 2048, cross-entropy inside the
+#  logits product (bf16 only; False = fp32 logits and a row kernel over them))
 HEAD_CASES = [
-    ("fp32", 4096, 5000, 1000, None),     # 3 chunks of the default size, the last one ragged (904 rows)
-    ("bf16", 4096, 5000, 1000, None),     # the same through the bf16 dlogits that overlay the fp32 logits
-    ("fp32", 4096, 1500, 500, 256),       # 6 chunks, ragged tail of 220
-    ("bf16", 4096, 1500, 500, 256),
-    ("fp32", 1001, 700, 350, 256),        # vocab % 4 != 0: the generic row kernel (+ cast in bf16)
-    ("bf16", 1001, 700, 350, 256),
-    ("fp32", 50257, 600, 300, 256),       # vocab > 32768: a row no longer fits the one-pass kernel's registers
-    ("bf16", 50257, 600, 300, 256),
+    ("fp32", 4096, 5000, 1000, None, False),     # 3 chunks of the default size, the last one ragged (904 rows)
+    ("bf16", 4096, 5000, 1000, None, False),     # the same through the bf16 dlogits that overlay the fp32 logits
+    ("bf16", 4096, 5000, 1000, None, True),      # ... and with no logits in memory at all
+    ("fp32", 4096, 1500, 500, 256, False),       # 6 chunks, ragged tail of 220
+    ("bf16", 4096, 1500, 500, 256, False),
+    ("bf16", 4096, 1500, 500, 256, True),
+    ("bf16", 4104, 1500, 500, 256, True),        # vocab % 64 != 0: the last 64-column span of a row is partly masked
+    ("bf16", 776, 700, 350, 300, True),          # vocab % 256 != 0 and whole spans past the last column
+    ("fp32", 1001, 700, 350, 256, False),        # vocab % 4 != 0: the generic row kernel (+ cast in bf16)
+    ("bf16", 1001, 700, 350, 256, True),         # ... which the in-product setting falls back to (vocab % 8 != 0)
+    ("fp32", 50257, 600, 300, 256, False),       # vocab > 32768: a row no longer fits the one-pass kernel's registers
+    ("bf16", 50257, 600, 300, 256, False),
 ]
 
 
-@pytest.mark.parametrize("case", HEAD_CASES, ids=lambda c: f"{c[0]}_V{c[1]}_N{c[2]}_chunk{c[4]}")
+@pytest.mark.parametrize("case", HEAD_CASES, ids=lambda c: f"{c[0]}_V{c[1]}_N{c[2]}_chunk{c[4]}_{'inproduct' if c[5] else 'rows'}")
 def test_chunked_tied_head_matches_the_materialised_head(case):
     """ops::cross_entropy over llama.cpp:88's logits (src/ops.cpp:350-376), evaluated chunk by chunk, against the
     same head with the [N, vocab] logits materialised as the reference does: loss and every gradient, with more
-    than two chunks, a ragged last chunk, and both fall-back row kernels. The chunk loop accumulates dE across
-    chunks, offsets the per-row losses, targets and dh rows by the chunk start, and (bf16) writes dlogits over
-    the first half of each fp32 logits row; an error in any of these shows as a difference here."""
-    dtype, vocab, n, sl, chunk = case
+    than two chunks, a ragged last chunk, both fall-back row kernels, and the cross-entropy formed inside the logits
+    product. The chunk loop accumulates dE across chunks, offsets the per-row losses, targets and dh rows by the
+    chunk start, and (bf16, row kernel) writes dlogits over the first half of each fp32 logits row; an error in any
+    of these shows as a difference here."""
+    dtype, vocab, n, sl, chunk, in_product = case
     cfg = dict(vocab=vocab, d=64, n_layers=1, n_heads=2, d_ff=176)
     m = Llama(compute_dtype=dtype, rope_all_heads=True, seed=21, **cfg)
     if chunk:
         m.set_head_chunk(chunk)
     toks = synth.randint(31, n + 1, vocab)
     x, y = toks[:-1], toks[1:]
-    loss_mat, _ = m.loss_backward(x, y, sl, fused_head=False)
-    g_mat = m.grads()
-    loss_chunked, _ = m.loss_backward(x, y, sl, fused_head=True)
-    g_chunked = m.grads()
-    d_abs, d_rel = maxdiff(g_chunked, g_mat), reldiff(g_chunked, g_mat)
-    print(f"\n  {dtype} V={vocab} N={n} chunk={chunk}: loss {loss_chunked:.7f} vs {loss_mat:.7f}, "
-          f"grad diff abs {d_abs:.2e} rel {d_rel:.2e}", flush=True)
-    if dtype == "fp32":
-        assert abs(loss_chunked - loss_mat) < 1e-6 and d_abs < 1e-6 and d_rel < 1e-4
-    else:
-        # both heads round dlogits to bf16 once and accumulate in fp32; what differs is the order of the sums
-        assert abs(loss_chunked - loss_mat) < 1e-5 and d_abs < 1e-4 and d_rel < 2e-2
-    # one chunk that holds every row is the degenerate case and must agree with many chunks
-    m.set_head_chunk(n)
-    loss_one, _ = m.loss_backward(x, y, sl, fused_head=True)
-    assert abs(loss_one - loss_chunked) < 1e-6
-    assert maxdiff(m.grads(), g_chunked) < (1e-6 if dtype == "fp32" else 1e-4)
-    m.close()
+    before = blockops.set_head_kernel(in_product)
+    try:
+        loss_mat, _ = m.loss_backward(x, y, sl, fused_head=False)
+        g_mat = m.grads()
+        loss_chunked, _ = m.loss_backward(x, y, sl, fused_head=True)
+        g_chunked = m.grads()
+        d_abs, d_rel = maxdiff(g_chunked, g_mat), reldiff(g_chunked, g_mat)
+        print(f"\n  {dtype} V={vocab} N={n} chunk={chunk} in_product={in_product}: loss {loss_chunked:.7f} vs {loss_mat:.7f}, "
+              f"grad diff abs {d_abs:.2e} rel {d_rel:.2e}", flush=True)
+        if dtype == "fp32":
+            assert abs(loss_chunked - loss_mat) < 1e-6 and d_abs < 1e-6 and d_rel < 1e-4
+        else:
+            # both heads round dlogits to bf16 once and accumulate in fp32; what differs is the order of the sums
+            assert abs(loss_chunked - loss_mat) < 1e-5 and d_abs < 1e-4 and d_rel < 2e-2
+        # one chunk that holds every row is the degenerate case and must agree with many chunks
+        m.set_head_chunk(n)
+        loss_one, _ = m.loss_backward(x, y, sl, fused_head=True)
+        assert abs(loss_one - loss_chunked) < 1e-6
+        assert maxdiff(m.grads(), g_chunked) < (1e-6 if dtype == "fp32" else 1e-4)
+        if in_product:
+            # the two ways of forming the chunked head's cross-entropy against each other: the same fp32 logits either
+            # way (never rounded in between), so the loss agrees to a few ulp and the gradients to one bf16 rounding
+            m.set_head_chunk(chunk or 2048)
+            blockops.set_head_kernel(False)
+            loss_rows, _ = m.loss_backward(x, y, sl, fused_head=True)
+            g_rows = m.grads()
+            assert abs(loss_rows - loss_chunked) < 2e-6
+            assert maxdiff(g_rows, g_chunked) < 1e-4 and reldiff(g_chunked, g_rows) < 2e-2
+    finally:
+        blockops.set_head_kernel(bool(before))
+        m.close()
 
 
 def test_config5_full_size_checkpointing_bars():
