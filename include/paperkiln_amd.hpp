@@ -211,6 +211,8 @@ namespace ops {
 // y = x W for a parameter W [in, out] kept in fp32 with a compute-dtype shadow
 // (ops::matmul + nn::Linear::forward, ops.cpp:33-58, nn.cpp:106-109).
 Var linear(const Var& x, const Var& W);
+// r + x W: a Linear whose output joins the residual stream (llama.cpp:47, 59), the add done in the product's epilogue
+Var linear_add(const Var& x, const Var& W, const Var& r);
 // Three projections of the same input written side by side into one [N, 3*out]
 // matrix: the concat_cols({q, k, v}) of llama.cpp:30-36 without the copies.
 Var linear3(const Var& x, const Var& Wq, const Var& Wk, const Var& Wv);

@@ -59,7 +59,8 @@ struct GemmArgs {
     void* c;
     int M, N, K;
     int64_t lda, ldb, ldc;
-    int beta;         // 0: C = product, 1: C += product
+    int beta;         // 0: C = product, 1: C = D + product
+    const void* d;    // D of beta 1: C's type and row pitch; null = C itself (C += product)
     int k_per_split;  // contraction elements per blockIdx.z (a multiple of BK); K when not split
     int64_t part_stride;  // elements between the fp32 partial results of two slices (split only)
     int tiles_m, tiles_n;
@@ -601,15 +602,19 @@ void gemm_ring(GemmArgs g, HeadArgs hd) {
             const bool in = row < g.M;
             const int tt = (in ? hd.target[row] : -1) - (bl.n0 + wn * FN * 32);
             const bool has = tt >= 0 && tt < FN * 32 && ((tt >> 2) & 1) == gh && in;
-            const int at = has ? (tt >> 5) * 16 + ((tt >> 3) & 3) * 4 + (tt & 3) : -1;
-            const float ref = in ? hd.row_max[row] * LOG2E : 0.0f, inv = in ? hd.row_inv[row] : 0.0f;
+            // P gscale = exp2(z log2e - (max log2e - log2(gscale / sum))): the scaling rides in the exponent
+            const float ref = in ? fmaf(hd.row_max[row], LOG2E, -__builtin_amdgcn_logf(hd.row_inv[row] * hd.gscale)) : 0.0f;
 #pragma unroll
             for (int j = 0; j < FN; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const float p = __builtin_amdgcn_exp2f(fmaf(acc[i][j][r], LOG2E, -ref)) * inv;
-                    acc[i][j][r] = (p - (at == j * 16 + r ? 1.0f : 0.0f)) * hd.gscale;
-                }
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = __builtin_amdgcn_exp2f(fmaf(acc[i][j][r], LOG2E, -ref));
+            if (__builtin_amdgcn_ballot_w64(has) != 0) {  // few wavefronts hold a target column of one of their rows
+                const int at = has ? (tt >> 5) * 16 + ((tt >> 3) & 3) * 4 + (tt & 3) : -1;
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[i][j][r] -= at == j * 16 + r ? hd.gscale : 0.0f;
+            }
         }
     };
     // the tile's result, through the ring slot `strip` (which every wavefront has finished reading)
@@ -654,7 +659,8 @@ void gemm_ring(GemmArgs g, HeadArgs hd) {
         const uint32_t crec = cleft > 0x7ffffff0 ? 0x7ffffff0u : static_cast<uint32_t>(cleft);
         const uint64_t ca = reinterpret_cast<uint64_t>(ctile);
         const u32x4 crs = {static_cast<uint32_t>(ca), static_cast<uint32_t>(ca >> 32) & 0xffffu, crec, 0x00020000u};
-        const __amdgpu_buffer_rsrc_t crs_b = __builtin_amdgcn_make_buffer_rsrc(ctile, 0, static_cast<int>(crec), 0x00020000);
+        CT* dtile = g.d ? static_cast<CT*>(const_cast<void*>(g.d)) + static_cast<int64_t>(bl.m0) * g.ldc + bl.n0 : ctile;
+        const __amdgpu_buffer_rsrc_t crs_b = __builtin_amdgcn_make_buffer_rsrc(dtile, 0, static_cast<int>(crec), 0x00020000);
         const uint32_t cmask = bl.n0 + st_ch * ST::EPC < g.N ? 0u : OUTSIDE;
         CT* cs = reinterpret_cast<CT*>(strip);
 #pragma unroll
@@ -808,27 +814,36 @@ __global__ void sum_slices(const float* part, void* dst, int nparts, int64_t par
 }
 
 // Joins a row's span statistics of the head's first pass, in span order: the row's maximum M, 1 / sum_j exp(z_j - M)
-// and its loss -log(max(P_target, 1e-12)) (src/ops.cpp:360-368). 64 rows x 16 groups of spans per block.
-__global__ __launch_bounds__(1024) void head_rows(const float2* stats, const float* zt, int spans, int M, float* row_max,
-                                                  float* row_inv, float* nll) {
-    __shared__ float sh_m[16][64], sh_s[16][64];
-    const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6, r = blockIdx.x * 64 + lane;
+// and its loss -log(max(P_target, 1e-12)) (src/ops.cpp:360-368). 16 rows x 16 groups of spans per block.
+__global__ __launch_bounds__(256) void head_rows(const float2* stats, const float* zt, int spans, int M, float* row_max,
+                                                 float* row_inv, float* nll) {
+    __shared__ float sh_m[16][16], sh_s[16][16];
+    const int lr = threadIdx.x & 15, grp = threadIdx.x >> 4, r = blockIdx.x * 16 + lr;
     auto join = [](float& m, float& s, float m2, float s2) {
         const float nm = fmaxf(m, m2), ref = nm == -INFINITY ? 0.0f : nm;
         s = s * __builtin_amdgcn_exp2f((m - ref) * LOG2E) + s2 * __builtin_amdgcn_exp2f((m2 - ref) * LOG2E);
         m = nm;
     };
     float m = -INFINITY, s = 0.0f;
-    if (r < M)
-        for (int p = grp; p < spans; p += 16) {
+    if (r < M) {
+        int p = grp;
+        for (; p + 48 < spans; p += 64) {  // four loads in flight, joined in span order
+            float2 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = stats[static_cast<int64_t>(p + 16 * u) * M + r];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) join(m, s, v[u].x, v[u].y);
+        }
+        for (; p < spans; p += 16) {
             const float2 v = stats[static_cast<int64_t>(p) * M + r];
             join(m, s, v.x, v.y);
         }
-    sh_m[grp][lane] = m;
-    sh_s[grp][lane] = s;
+    }
+    sh_m[grp][lr] = m;
+    sh_s[grp][lr] = s;
     __syncthreads();
     if (grp == 0 && r < M) {
-        for (int q = 1; q < 16; ++q) join(m, s, sh_m[q][lane], sh_s[q][lane]);
+        for (int q = 1; q < 16; ++q) join(m, s, sh_m[q][lr], sh_s[q][lr]);
         const float inv = 1.0f / s;
         row_max[r] = m;
         row_inv[r] = inv;
@@ -982,6 +997,7 @@ GemmArgs gemm_args(const void* a, int64_t lda, const void* b, int64_t ldb, int64
     g.M = static_cast<int>(M), g.N = static_cast<int>(N), g.K = static_cast<int>(K);
     g.lda = lda, g.ldb = ldb, g.ldc = N;
     g.beta = 0;
+    g.d = nullptr;
     g.k_per_split = g.K;
     g.part_stride = 0;
     g.tiles_m = g.tiles_n = 0;
@@ -993,7 +1009,7 @@ GemmArgs gemm_args(const void* a, int64_t lda, const void* b, int64_t ldb, int64
 // Returns false, having done nothing, for what the kernel does not take (fp32 operands, unaligned rows, sizes
 // that are not multiples of 8): the caller then uses the library GEMM.
 bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB, int64_t ldb, void* c, int c_dtype,
-                    int64_t M, int64_t N, int64_t K, int64_t ldc, float beta, hipStream_t st) {
+                    int64_t M, int64_t N, int64_t K, int64_t ldc, float beta, hipStream_t st, const void* addend) {
     if (!takes(a, tA, lda, b, ldb, M, N, K) || !aligned16(c) || ldc % 8) return false;
     if (beta != 0.0f && beta != 1.0f) return false;
     GemmArgs g = gemm_args(a, lda, b, ldb, M, N, K);
@@ -1001,6 +1017,10 @@ bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB,
     g.ldc = ldc;
     g.beta = beta != 0.0f;
     const Plan p = make_plan(tA, tB, M, N, K, lda, ldb, ldc);
+    if (addend) {  // C = addend + product: in the epilogue of the ring kernels, whole contractions only
+        if (beta != 1.0f || !aligned16(addend) || p.ring == 0 || p.S != 1) return false;
+        g.d = addend;
+    }
     if (p.S == 1) {
         run_plan(p, tA, tB, g, 1, c_dtype == PK_F32, st);
         return true;
@@ -1044,19 +1064,20 @@ bool head_takes(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t 
     const int64_t ext_max = (int64_t{1} << 30) - 8192;
     return M * lda * 2 < ext_max && N * ldb * 2 < ext_max && lda < (1 << 21) && ldb < (1 << 21) && N < (1 << 20);
 }
-template <int EPI>
+template <typename G, int EPI>
 void launch_head(GemmArgs g, const HeadArgs& hd, hipStream_t st) {
-    using G = GeoLarge;
     g.tiles_m = (g.M + G::BM - 1) / G::BM;
     g.tiles_n = (g.N + G::BN - 1) / G::BN;
     g.splits = 1;
     const int64_t vblocks = static_cast<int64_t>((g.tiles_m * g.tiles_n + 7) / 8 * 8);
-    const unsigned gx = static_cast<unsigned>(std::min<int64_t>(vblocks, cu_count() / 8 * 8));
+    const unsigned gx = static_cast<unsigned>(std::min<int64_t>(vblocks, cu_count() / 8 * 8 * (G::BM > 128 ? 1 : 2)));
     hipLaunchKernelGGL((gemm_ring<G, false, true, false, 2, true, EPI>), dim3(gx), dim3(G::NTHR), 0, st, g, hd);
     hip_check(hipGetLastError(), "gemm_ring (head) launch");
 }
 }  // namespace
 
+// 256 x 256 tiles, one workgroup of eight wavefronts per CU (128 x 128 tiles with two workgroups per CU, whose
+// epilogues could overlap each other's matrix work, measured 15 % slower on [2048, 32000] x 512)
 int64_t gemm_head_spans(int64_t N) { return (N + GeoLarge::BN - 1) / GeoLarge::BN * GeoLarge::WGN; }
 
 // Pass 1 over logits = A B^T (A [M, K] and B [N, K], bf16), which are formed tile by tile and never stored: per row
@@ -1070,8 +1091,8 @@ bool gemm_head_rows(const void* a, int64_t lda, const void* b, int64_t ldb, int6
     hd.target = target;
     hd.stats = static_cast<float2*>(stats);
     hd.zt = zt;
-    launch_head<1>(g, hd, st);
-    hipLaunchKernelGGL(head_rows, dim3(static_cast<unsigned>((M + 63) / 64)), dim3(1024), 0, st, hd.stats, zt,
+    launch_head<GeoLarge, 1>(g, hd, st);
+    hipLaunchKernelGGL(head_rows, dim3(static_cast<unsigned>((M + 15) / 16)), dim3(256), 0, st, hd.stats, zt,
                        static_cast<int>(gemm_head_spans(N)), static_cast<int>(M), row_max, row_inv, nll);
     hip_check(hipGetLastError(), "head_rows launch");
     return true;
@@ -1091,7 +1112,7 @@ bool gemm_head_dlogits(const void* a, int64_t lda, const void* b, int64_t ldb, i
     hd.row_max = row_max;
     hd.row_inv = row_inv;
     hd.gscale = gscale;
-    launch_head<2>(g, hd, st);
+    launch_head<GeoLarge, 2>(g, hd, st);
     return true;
 }
 

@@ -164,11 +164,9 @@ struct Model {
         Var qkv = ops::linear3(h, b.q, b.k, b.v);
         qkv = ops::apply_rope(qkv, pos, cfg.rope_theta, dk, cfg.rope_all_heads ? cfg.n_heads : 1, /*in_place=*/true);
         const float sc = 1.0f / std::sqrt(static_cast<float>(dk));
-        Var attn = ops::linear(ops::attention_qkv(qkv, cfg.n_heads, sc, seq_len, true, cfg.window, cfg.sinks), b.o);
-        Var x1 = ops::add(x, attn);
+        Var x1 = ops::linear_add(ops::attention_qkv(qkv, cfg.n_heads, sc, seq_len, true, cfg.window, cfg.sinks), b.o, x);
         Var h2 = ops::rmsnorm(x1, b.ln2_w);
-        Var ffn = ops::linear(ops::silu_mul_cat(ops::linear_cat(h2, {b.gate, b.up})), b.down);
-        return ops::add(x1, ffn);
+        return ops::linear_add(ops::silu_mul_cat(ops::linear_cat(h2, {b.gate, b.up})), b.down, x1);
     }
 
     // Llama::forward (llama.cpp:71-89) up to the final norm; positions restart per sequence.

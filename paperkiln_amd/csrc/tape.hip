@@ -293,6 +293,44 @@ Var linear(const Var& x, const Var& W) {
     });
 }
 
+// y = r + x W: a Linear whose output joins a residual stream (o_proj and the MLP's down projection,
+// llama.cpp:47-59), the sum formed in the product's epilogue where the library's own GEMM takes the operands (one
+// rounding of r + x W instead of two, and no pass over y and r afterwards), by an add otherwise. One node with
+// the gradients of both ops: dr is the node's gradient itself.
+Var linear_add(const Var& x, const Var& W, const Var& r) {
+    if (x->data.cols != W->data.rows) shape_fail("matmul: inner dimensions disagree");
+    if (r->data.rows != x->data.rows || r->data.cols != W->data.cols || r->data.dtype != x->data.dtype)
+        shape_fail("add: shape mismatch");
+    const Tensor& Wc = shadow_of(W);
+    Tensor y = Tensor::make(x->data.rows, W->data.cols, x->data.dtype);
+    const bool contiguous = r->data.off_bytes % 16 == 0;
+    if (!(x->data.dtype == PK_BF16 && Wc.dtype == PK_BF16 && gemm_backend() != 0 && contiguous &&
+          gemm_mfma_bf16(x->data.ptr(), false, x->data.cols, Wc.ptr(), false, Wc.cols, y.ptr(), y.dtype, y.rows, y.cols,
+                         x->data.cols, y.cols, 1.0f, tape_stream(), r->data.ptr()))) {
+        gemm(x->data, false, Wc, false, y.ptr(), y.dtype, y.rows, y.cols, y.cols, 0.0f);
+        k_add(r->data, y, y);
+    }
+    return record(std::move(y), {x, W, r}, [](Variable* self) {
+        const Var& x = self->parents[0];
+        const Var& W = self->parents[1];
+        const Var& r = self->parents[2];
+        if (x->requires_grad) {
+            Tensor dx = Tensor::make(x->data.rows, x->data.cols, x->data.dtype);
+            gemm(self->grad, false, shadow_of(W), true, dx.ptr(), dx.dtype, dx.rows, dx.cols, dx.cols, 0.0f);
+            x->accumulate_owned(std::move(dx));
+        }
+        if (W->requires_grad) {
+            Tensor& g = W->ensure_grad();
+            gemm(x->data, true, self->grad, false, g.ptr(), g.dtype, g.rows, g.cols, g.cols, 1.0f);
+        }
+        if (r->requires_grad) {
+            const bool was_shared = self->grad_shared;  // the products above have read it; r takes the tensor itself
+            self->grad_shared = false;
+            r->accumulate_owned(std::move(self->grad), was_shared);
+        }
+    });
+}
+
 // y = x [W_0 | W_1 | ...]: several Linear layers that read the same input (q/k/v projections,
 // gate/up projections) as ONE GEMM against the column-wise concatenation of their weights, which
 // is kept as a compute-dtype copy like any other shadow. Backward is one GEMM for dX and one for

@@ -62,8 +62,9 @@ void k_adamw(const Tensor& p, const Tensor& g, const Tensor& m, const Tensor& v,
 void gemm(const Tensor& A, bool tA, const Tensor& B, bool tB, void* C, int c_dtype, int64_t M, int64_t N, int64_t ldc,
           float beta, int64_t lda = 0);
 // gemm_mfma.hip: the hand-written bf16 matrix-core GEMM. Returns false (nothing done) for operands it does not take.
+// With an addend (C's type and row pitch; beta must be 1) C = addend + op(A) op(B), the sum rounded once.
 bool gemm_mfma_bf16(const void* a, bool tA, int64_t lda, const void* b, bool tB, int64_t ldb, void* c, int c_dtype,
-                    int64_t M, int64_t N, int64_t K, int64_t ldc, float beta, hipStream_t st);
+                    int64_t M, int64_t N, int64_t K, int64_t ldc, float beta, hipStream_t st, const void* addend = nullptr);
 // The same product left as fp32 partial products part[s][M][N], s < nparts (the contraction cut into slices where the
 // output alone would leave the chip idle), for a caller that adds them on the way to where the result goes.
 bool gemm_mfma_bf16_parts(const void* a, bool tA, int64_t lda, const void* b, bool tB, int64_t ldb, int64_t M, int64_t N,

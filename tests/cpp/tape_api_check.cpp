@@ -257,6 +257,50 @@ void shared_gradient_case(int dtype, const char* name, double tol) {
     }
 }
 
+// r + x W with the add inside the product's epilogue (bf16) against the two ops it stands for; edge tiles in both
+// directions, and a contraction long enough for the two-wavefront-set form of the kernel.
+void linear_add_case(int dtype, const char* name, int T, int din, int dout, double tol) {
+    std::printf("linear_add, %s, [%d, %d] x [%d, %d]\n", name, T, din, din, dout);
+    const auto hx = draw(static_cast<size_t>(T) * din, 51, 1.0), hw = draw(static_cast<size_t>(din) * dout, 52, 0.2),
+               hr = draw(static_cast<size_t>(T) * dout, 53, 2.0);
+    std::vector<int> target(T);
+    for (int i = 0; i < T; ++i) target[i] = (3 * i + 1) % dout;
+    auto tg = device_ints(target);
+    pk::set_compute_dtype(dtype);  // the weight's compute-dtype copy follows it
+    struct Run {
+        std::vector<float> y, gx, gw, gr;
+    };
+    auto run = [&](bool fused) {
+        pk::Var x = pk::make_var(pk::upload(hx.data(), T, din, dtype), true);
+        pk::Var r = pk::make_var(pk::upload(hr.data(), T, dout, dtype), true);
+        pk::Var w = pk::make_var(pk::upload(hw.data(), din, dout), true);
+        w->is_param = true;
+        pk::Var y = fused ? pk::ops::linear_add(x, w, r) : pk::ops::add(r, pk::ops::linear(x, w));
+        Run out;
+        out.y = host(y->data);
+        pk::backward(pk::ops::cross_entropy(y, tg));
+        out.gx = host(x->grad);
+        out.gw = host(w->grad);
+        out.gr = host(r->grad);
+        pk::invalidate_shadows();
+        return out;
+    };
+    const Run two = run(false), one = run(true);
+    auto rel = [](const std::vector<float>& a, const std::vector<float>& b) {
+        double w = 0.0, size = 0.0;
+        for (size_t i = 0; i < a.size(); ++i) {
+            w = std::fmax(w, std::fabs(static_cast<double>(a[i]) - b[i]));
+            size = std::fmax(size, std::fabs(static_cast<double>(b[i])));
+        }
+        return w / std::fmax(size, 1e-30);
+    };
+    check(rel(one.y, two.y) <= tol, "r + x W vs add(r, linear(x, W))", rel(one.y, two.y));
+    check(rel(one.gx, two.gx) <= 4 * tol, "dX", rel(one.gx, two.gx));
+    check(rel(one.gw, two.gw) <= 4 * tol, "dW", rel(one.gw, two.gw));
+    check(rel(one.gr, two.gr) <= 4 * tol, "dr", rel(one.gr, two.gr));
+    pk::set_compute_dtype(PK_F32);
+}
+
 void behaviour_case() {
     std::printf("tape behaviour and errors\n");
     const auto h = draw(8 * 4, 31, 1.0);
@@ -312,6 +356,9 @@ int main() {
     checkpoint_case();
     shared_gradient_case(PK_F32, "float32", 1e-6);
     shared_gradient_case(PK_BF16, "bfloat16 (the fused row kernel)", 1.0 / 128);
+    linear_add_case(PK_F32, "float32 (product, then add)", 40, 24, 16, 1e-6);
+    linear_add_case(PK_BF16, "bfloat16, edge tiles", 200, 72, 136, 1.0 / 128);
+    linear_add_case(PK_BF16, "bfloat16, long contraction", 300, 1376, 64, 1.0 / 128);
     behaviour_case();
     if (g_failures == 0) {
         std::printf("tape_api_check PASSED\n");
