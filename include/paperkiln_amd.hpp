@@ -161,6 +161,9 @@ public:
     // grad's storage is also another Variable's grad (both parents of an add take the same tensor): it is read-only
     // until own_grad() has given this Variable a copy of its own. accumulate(), ensure_grad() and zero_grad() do so.
     bool grad_shared = false;
+    // grad is exactly 1: backward() seeded this [1,1] root and nothing has been added since (lets a scalar loss's
+    // backward skip reading its upstream gradient back from the device). Code that writes grad directly clears it.
+    bool grad_is_unit = false;
     std::vector<Var> parents;
     std::function<void()> backward_fn;
 

@@ -836,6 +836,20 @@ __global__ void sum_f32_k(const float* x, int64_t n, double* out) {
     }
     if (threadIdx.x == 0) *out = sh[0];
 }
+// mean of n floats, accumulated in double in the order sum_f32_k uses, rounded to float once: what the host does
+// with k_sum_f32_to_host's result, without the round trip
+__global__ void mean_f32_k(const float* x, int64_t n, float* out) {
+    __shared__ double sh[NT];
+    double s = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += NT) s += static_cast<double>(x[i]);
+    sh[threadIdx.x] = s;
+    __syncthreads();
+    for (int o = NT / 2; o >= 1; o >>= 1) {
+        if (threadIdx.x < o) sh[threadIdx.x] += sh[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *out = static_cast<float>(sh[0] / static_cast<double>(n));
+}
 __global__ void sumsq_part(const float* x, int64_t n, double* part) {
     __shared__ double sh[NT];
     double s = 0.0;
@@ -1159,6 +1173,11 @@ bool k_ce_rows_once(const Tensor& logits, const int* targets, float gscale, floa
     }
     post();
     return true;
+}
+void k_mean_f32(const float* x, int64_t n, const Tensor& out) {
+    if (out.dtype != PK_F32 || out.rows * out.cols != 1) throw std::runtime_error("mean: the result is one float");
+    hipLaunchKernelGGL(mean_f32_k, dim3(1), dim3(NT), 0, tape_stream(), x, n, static_cast<float*>(out.ptr()));
+    post();
 }
 double k_sum_f32_to_host(const float* x, int64_t n) {
     Buffer out(sizeof(double));

@@ -106,6 +106,10 @@ float scalar_to_host(const Tensor& t) {
     return h;
 }
 
+// The gradient of a [1,1] node as a host value: 1 without asking the device where backward() seeded it and nothing
+// has been added since (the usual case: the loss is the root), a copy back and a wait otherwise.
+float upstream_scalar(const Variable* v) { return v->grad_is_unit ? 1.0f : scalar_to_host(v->grad); }
+
 pk_tensor4 view4(const void* base, int64_t elem_off, size_t esize, int64_t sb, int64_t st, int64_t sh) {
     pk_tensor4 t;
     t.ptr = const_cast<char*>(static_cast<const char*>(base)) + elem_off * static_cast<int64_t>(esize);
@@ -173,11 +177,13 @@ Tensor& Variable::own_grad() {
         grad = std::move(mine);
     }
     grad_shared = false;
+    grad_is_unit = false;  // the caller is about to write
     return grad;
 }
 
 void Variable::accumulate(const Tensor& g, float a) {
     if (g.rows != data.rows || g.cols != data.cols) shape_fail("accumulate: gradient shape mismatch");
+    grad_is_unit = false;
     if (grad.empty()) {
         grad = Tensor::make(data.rows, data.cols, is_param ? PK_F32 : data.dtype);
         grad_shared = false;
@@ -201,6 +207,7 @@ void Variable::accumulate_owned(Tensor&& g, bool shared) {
     if (grad.empty() && whole && g.dtype == want && g.rows == data.rows && g.cols == data.cols) {
         grad = std::move(g);
         grad_shared = shared;
+        grad_is_unit = false;
         return;
     }
     accumulate(g);
@@ -228,7 +235,9 @@ void backward(const Var& root) {
         throw std::runtime_error("backward: root must be a [1,1] scalar (compose with mean/sum)");
     Tensor seed = Tensor::make(1, 1, root->data.dtype);
     k_fill(seed, 1.0f);
+    const bool fresh = root->grad.empty();
     root->accumulate(seed);
+    root->grad_is_unit = fresh;
     run_backward(root);
 }
 
@@ -240,6 +249,7 @@ void zero_grad(const std::vector<Var>& vars) {
             v->grad_shared = false;
         }
         k_fill(v->grad, 0.0f);
+        v->grad_is_unit = false;
     }
 }
 
@@ -670,13 +680,12 @@ Var cross_entropy(const Var& logits, const std::shared_ptr<Buffer>& targets) {
     k_cast(logits->data, *P);
     Buffer nll(sizeof(float) * R);
     k_ce_rows(*P, static_cast<const int*>(targets->p), 1.0f / static_cast<float>(R), static_cast<float*>(nll.p));
-    const double total = k_sum_f32_to_host(static_cast<const float*>(nll.p), R);
     Tensor out = Tensor::make(1, 1, PK_F32);
-    k_fill(out, static_cast<float>(total / static_cast<double>(R)));
+    k_mean_f32(static_cast<const float*>(nll.p), R, out);
     return record(std::move(out), {logits}, [P](Variable* self) {
         const Var& l = self->parents[0];
         if (!l->requires_grad) return;
-        l->accumulate(*P, scalar_to_host(self->grad));  // (P - onehot) * g / R, ops.cpp:371-374
+        l->accumulate(*P, upstream_scalar(self));  // (P - onehot) * g / R, ops.cpp:371-374
     });
 }
 
@@ -746,13 +755,12 @@ Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffe
             gemm(dl, false, Ec, false, static_cast<char*>(dh1.ptr()) + r0 * d * hes, dh1.dtype, rows, d, d, 0.0f, dl_ld);
         if (want_dE) gemm(dl, true, hview, false, dE1.ptr(), PK_F32, V, d, d, r0 == 0 ? 0.0f : 1.0f, dl_ld);
     }
-    const double total = k_sum_f32_to_host(static_cast<const float*>(nll.p), N);
     Tensor out = Tensor::make(1, 1, PK_F32);
-    k_fill(out, static_cast<float>(total / static_cast<double>(N)));
+    k_mean_f32(static_cast<const float*>(nll.p), N, out);  // the loss stays on the device: no wait in mid-step
     return record(std::move(out), {h, E}, [dh1, dE1](Variable* self) mutable {
         const Var& h = self->parents[0];
         const Var& E = self->parents[1];
-        const float g = scalar_to_host(self->grad);  // upstream gradient of the scalar loss
+        const float g = upstream_scalar(self);  // upstream gradient of the scalar loss
         if (h->requires_grad && !dh1.empty()) {
             if (g == 1.0f)
                 h->accumulate_owned(std::move(dh1));

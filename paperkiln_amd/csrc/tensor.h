@@ -47,6 +47,7 @@ void k_ce_rows(const Tensor& logits, const int* targets, float gscale, float* nl
 bool k_ce_rows_once(const Tensor& logits, const int* targets, float gscale, float* nll_rows, const Tensor* dl,
                     int64_t dl_ld = 0);  // dl_ld: row pitch of dl in its own elements (0 = cols)
 double k_sum_f32_to_host(const float* x, int64_t n);                   // double accumulation, ops.cpp:360-367
+void k_mean_f32(const float* x, int64_t n, const Tensor& out);         // the same sum / n into a [1,1] float, no host round trip
 double k_sumsq_to_host(const Tensor& g);                               // clip_grad_norm's sum, ops.cpp:1046-1052
 // The same in two halves, so that many gradients cost one host round trip: per-block partial sums (at most
 // SUMSQ_MAX_PARTS doubles) into device memory, then one copy and a host sum over all of them.
