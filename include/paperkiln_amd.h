@@ -196,7 +196,9 @@ int pk_llama_adamw_step(void* handle, float lr, float b1, float b2, float eps, f
                         float* total_norm);
 /* Rows of the tied head (llama.cpp:88 + ops::cross_entropy, src/ops.cpp:350-376) evaluated at a time when
  * fused_head = 1: the [n, vocab] logits the reference materialises exist here one [rows, vocab] chunk at a
- * time. Default 2048; smaller chunks lower the activation peak, larger ones run fewer, larger GEMMs. */
+ * time. Default: 4096 rows where the cross-entropy runs inside the logits product (bf16 operands; the chunk's scratch is
+ * its bf16 dlogits), 2048 where fp32 logits are stored -- 262 MB at a vocabulary of 32000 either way; smaller chunks lower
+ * the activation peak, larger ones run fewer, larger GEMMs. */
 int pk_llama_set_head_chunk(void* handle, int64_t rows);
 
 /* ---- block operators -------------------------------------------------------

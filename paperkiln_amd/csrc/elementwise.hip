@@ -400,6 +400,58 @@ __global__ void rms_fwd8(const uint16_t* x, const float* w, float eps, uint16_t*
         st8(y + row * C, j, v);
     }
 }
+// The same with each row held in registers between the two passes (C <= 512 NP) and two rows of a wavefront in flight:
+// 8 rows per block of four wavefronts.
+template <int NP>
+__global__ void rms_fwd8_reg(const uint16_t* x, const float* w, float eps, uint16_t* y, float* rinv, int64_t R, int C) {
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int64_t row0 = static_cast<int64_t>(blockIdx.x) * 8 + wv;  // and row0 + 4
+    if (row0 >= R) return;
+    const bool two = row0 + 4 < R;
+    const int64_t rows[2] = {row0, two ? row0 + 4 : row0};
+    F8 v[2][NP], g[NP];
+    float ss[2] = {0.0f, 0.0f};
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int j = lane * 8 + p * 512;
+            if (j < C) v[q][p] = ld8(x + rows[q] * C, j);
+        }
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const int j = lane * 8 + p * 512;
+        if (j < C) g[p] = ld8(w, j);
+    }
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int j = lane * 8 + p * 512;
+            if (j < C) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) ss[q] = fmaf(v[q][p].v[k], v[q][p].v[k], ss[q]);
+            }
+        }
+    ss[0] = wave_sum(ss[0]) / static_cast<float>(C);
+    ss[1] = wave_sum(ss[1]) / static_cast<float>(C);
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        if (q == 1 && !two) break;
+        const float ri = 1.0f / sqrtf(ss[q] + eps);
+        if (lane == 0) rinv[rows[q]] = ri;
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int j = lane * 8 + p * 512;
+            if (j < C) {
+                F8 o;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) o.v[k] = v[q][p].v[k] * ri * g[p].v[k];
+                st8(y + rows[q] * C, j, o);
+            }
+        }
+    }
+}
 __global__ void rms_bwd_dx8(const uint16_t* dy, const uint16_t* x, const float* rinv, const float* w, uint16_t* dx, int64_t R,
                             int C) {
     const int lane = threadIdx.x & 63;
@@ -1020,9 +1072,21 @@ void k_silu_mul_cat_bwd(const Tensor& gu, const Tensor& dy, const Tensor& dgu) {
 void k_rmsnorm_fwd(const Tensor& x, const Tensor& w, float eps, const Tensor& y, float* rinv) {
     if (w.rows != 1 || w.cols != x.cols || w.dtype != PK_F32) throw std::runtime_error("rmsnorm: w must be [1, cols(x)]");
     if (x.dtype == PK_BF16 && x.cols % 8 == 0 && aligned16p(x.ptr()) && aligned16p(y.ptr()) && aligned16p(w.ptr())) {
-        hipLaunchKernelGGL(rms_fwd8, dim3((x.rows + 3) / 4), dim3(NT), 0, tape_stream(), static_cast<const uint16_t*>(x.ptr()),
-                           static_cast<const float*>(w.ptr()), eps, static_cast<uint16_t*>(y.ptr()), rinv, x.rows,
-                           static_cast<int>(x.cols));
+        const int C = static_cast<int>(x.cols);
+        auto launch = [&](auto np) {
+            hipLaunchKernelGGL((rms_fwd8_reg<decltype(np)::value>), dim3((x.rows + 7) / 8), dim3(256), 0, tape_stream(),
+                               static_cast<const uint16_t*>(x.ptr()), static_cast<const float*>(w.ptr()), eps,
+                               static_cast<uint16_t*>(y.ptr()), rinv, x.rows, C);
+        };
+        if (C <= 512)
+            launch(std::integral_constant<int, 1>{});
+        else if (C <= 1024)
+            launch(std::integral_constant<int, 2>{});
+        else if (C <= 2048)
+            launch(std::integral_constant<int, 4>{});
+        else
+            hipLaunchKernelGGL(rms_fwd8, dim3((x.rows + 3) / 4), dim3(NT), 0, tape_stream(), static_cast<const uint16_t*>(x.ptr()),
+                               static_cast<const float*>(w.ptr()), eps, static_cast<uint16_t*>(y.ptr()), rinv, x.rows, C);
         post();
         return;
     }

@@ -1078,6 +1078,9 @@ void launch_head(GemmArgs g, const HeadArgs& hd, hipStream_t st) {
 
 // 256 x 256 tiles, one workgroup of eight wavefronts per CU (128 x 128 tiles with two workgroups per CU, whose
 // epilogues could overlap each other's matrix work, measured 15 % slower on [2048, 32000] x 512)
+bool gemm_head_takes(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K) {
+    return head_takes(a, lda, b, ldb, M, N, K);
+}
 int64_t gemm_head_spans(int64_t N) { return (N + GeoLarge::BN - 1) / GeoLarge::BN * GeoLarge::WGN; }
 
 // Pass 1 over logits = A B^T (A [M, K] and B [N, K], bf16), which are formed tile by tile and never stored: per row

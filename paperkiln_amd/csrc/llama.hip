@@ -70,7 +70,7 @@ struct Model {
     // threads from running the same model at once; every C entry holds both for the length of the call.
     TapeContext ctx;
     std::mutex mu;
-    int64_t head_chunk_rows = 2048;  // rows of the tied head evaluated at a time (linear_cross_entropy)
+    int64_t head_chunk_rows = 0;  // rows of the tied head evaluated at a time (linear_cross_entropy); 0 = its default
     Var embed, norm_w;
     std::vector<Block> blocks;
     std::vector<std::pair<std::string, Var>> named;

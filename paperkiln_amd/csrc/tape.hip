@@ -692,7 +692,6 @@ Var cross_entropy(const Var& logits, const std::shared_ptr<Buffer>& targets) {
 Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffer>& targets, int64_t chunk_rows) {
     const int64_t N = h->data.rows, V = E->data.rows, d = h->data.cols;
     if (d != E->data.cols) shape_fail("matmul: inner dimensions disagree");
-    if (chunk_rows <= 0) chunk_rows = 1024;
     const int* tg = static_cast<const int*>(targets->p);
     const size_t hes = h->data.esize();
     // One pass over row chunks. The loss is a scalar, so its gradient with respect to the logits is known up to
@@ -709,7 +708,10 @@ Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffe
     const bool grads = want_dh || want_dE;
     // bf16 operands the library's own GEMM takes: the cross-entropy runs inside the logits product, which forms
     // every tile twice (row statistics and loss, then dlogits) instead of storing [rows, V] logits for a row kernel
-    bool in_product = h->data.dtype == PK_BF16 && Ec.dtype == PK_BF16 && head_kernel() != 0 && gemm_backend() != 0;
+    bool in_product = h->data.dtype == PK_BF16 && Ec.dtype == PK_BF16 && head_kernel() != 0 && gemm_backend() != 0 &&
+                      gemm_head_takes(h->data.ptr(), d, Ec.ptr(), d, std::min<int64_t>(N, chunk_rows > 0 ? chunk_rows : 4096), V, d);
+    // default chunk: the same scratch either way (4096 rows of bf16 dlogits, or 2048 of fp32 logits: 262 MB at 32000 words)
+    if (chunk_rows <= 0) chunk_rows = in_product ? 4096 : 2048;
     for (int64_t r0 = 0; r0 < N; r0 += chunk_rows) {
         const int64_t rows = std::min(chunk_rows, N - r0);
         const Tensor hview = h->data.row_range(r0, rows);

@@ -75,6 +75,7 @@ bool gemm_mfma_bf16_parts(const void* a, bool tA, int64_t lda, const void* b, bo
 // (stats: scratch of gemm_head_spans(N) * M float pairs, zt: of M floats); gemm_head_dlogits: bf16 dlogits.
 // Both return false, having done nothing, for operands the kernel does not take.
 int64_t gemm_head_spans(int64_t N);
+bool gemm_head_takes(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K);
 bool gemm_head_rows(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K, const int* target,
                     void* stats, float* zt, float* row_max, float* row_inv, float* nll, hipStream_t st);
 bool gemm_head_dlogits(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,

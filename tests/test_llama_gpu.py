@@ -194,12 +194,12 @@ def reldiff(a, b):
     return max(errs) if np.all(np.isfinite(errs)) else float("inf")
 
 
-# (dtype, vocab, tokens, seq_len, rows per head chunk or None = the library's default of 2048, cross-entropy inside the
+# (dtype, vocab, tokens, seq_len, rows per head chunk or None = the library's default (2048 rows of fp32 logits or 4096 of bf16 dlogits), cross-entropy inside the
 #  logits product (bf16 only; False = fp32 logits and a row kernel over them))
 HEAD_CASES = [
     ("fp32", 4096, 5000, 1000, None, False),     # 3 chunks of the default size, the last one ragged (904 rows)
     ("bf16", 4096, 5000, 1000, None, False),     # the same through the bf16 dlogits that overlay the fp32 logits
-    ("bf16", 4096, 5000, 1000, None, True),      # ... and with no logits in memory at all
+    ("bf16", 4096, 5000, 1000, None, True),      # ... and with no logits in memory at all (2 chunks, 904 rows ragged)
     ("fp32", 4096, 1500, 500, 256, False),       # 6 chunks, ragged tail of 220
     ("bf16", 4096, 1500, 500, 256, False),
     ("bf16", 4096, 1500, 500, 256, True),
