@@ -915,10 +915,17 @@ __global__ void sumsq_part(const float* x, int64_t n, double* part) {
     }
     if (threadIdx.x == 0) part[blockIdx.x] = sh[0];
 }
-__global__ void adamw_k(float* p, const float* g, float* m, float* v, float lr, float b1, float b2, float eps, float wd,
-                        float c1, float c2, int64_t n) {
+// CLIP: the gradient is scaled by gs first and the scaled value written back, as ops::clip_grad_norm leaves it
+// (src/ops.cpp:1058-1062), in the same pass instead of one of its own.
+template <bool CLIP>
+__global__ void adamw_k(float* p, float* g, float* m, float* v, float lr, float b1, float b2, float eps, float wd, float c1,
+                        float c2, float gs, int64_t n) {
     for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * NT) {
-        const float gi = g[i];
+        float gi = g[i];
+        if (CLIP) {
+            gi *= gs;
+            g[i] = gi;
+        }
         const float mi = b1 * m[i] + (1.0f - b1) * gi;
         const float vi = b2 * v[i] + (1.0f - b2) * gi * gi;
         m[i] = mi;
@@ -1274,10 +1281,15 @@ double k_sumsq_to_host(const Tensor& g) {
     return k_sum_f64_to_host(static_cast<const double*>(part.p), nb);
 }
 void k_adamw(const Tensor& p, const Tensor& g, const Tensor& m, const Tensor& v, float lr, float b1, float b2,
-             float eps, float wd, float c1, float c2) {
-    hipLaunchKernelGGL(adamw_k, ew_grid(p.numel()), dim3(NT), 0, tape_stream(), static_cast<float*>(p.ptr()),
-                       static_cast<const float*>(g.ptr()), static_cast<float*>(m.ptr()), static_cast<float*>(v.ptr()), lr,
-                       b1, b2, eps, wd, c1, c2, p.numel());
+             float eps, float wd, float c1, float c2, float grad_scale) {
+    if (grad_scale != 1.0f)
+        hipLaunchKernelGGL(adamw_k<true>, ew_grid(p.numel()), dim3(NT), 0, tape_stream(), static_cast<float*>(p.ptr()),
+                           static_cast<float*>(g.ptr()), static_cast<float*>(m.ptr()), static_cast<float*>(v.ptr()), lr, b1,
+                           b2, eps, wd, c1, c2, grad_scale, p.numel());
+    else
+        hipLaunchKernelGGL(adamw_k<false>, ew_grid(p.numel()), dim3(NT), 0, tape_stream(), static_cast<float*>(p.ptr()),
+                           static_cast<float*>(g.ptr()), static_cast<float*>(m.ptr()), static_cast<float*>(v.ptr()), lr, b1,
+                           b2, eps, wd, c1, c2, 1.0f, p.numel());
     post();
 }
 

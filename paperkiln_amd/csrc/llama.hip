@@ -377,11 +377,12 @@ int pk_llama_adamw_step(void* h, float lr, float b1, float b2, float eps, float 
         // ops::clip_grad_norm over the slab (the padding between parameters is zero): double
         // accumulation as the reference (ops.cpp:1047-1053), one host round trip.
         double tn = 0.0;
+        float clip = 1.0f;
         if (max_norm > 0.0f) {
             Buffer parts(sizeof(double) * SUMSQ_MAX_PARTS);
             const int nb = k_sumsq_parts(m->gslab, static_cast<double*>(parts.p));
             tn = std::sqrt(k_sum_f64_to_host(static_cast<const double*>(parts.p), nb));
-            if (tn > max_norm && tn > 0.0) k_scale(m->gslab, static_cast<float>(max_norm / tn), m->gslab);
+            if (tn > max_norm && tn > 0.0) clip = static_cast<float>(max_norm / tn);  // applied by the AdamW pass
         }
         if (total_norm) *total_norm = static_cast<float>(tn);
         ++m->t;
@@ -389,7 +390,7 @@ int pk_llama_adamw_step(void* h, float lr, float b1, float b2, float eps, float 
         const float c2 = 1.0f - std::pow(b2, static_cast<float>(m->t));
         // every parameter of this model receives a gradient each step, so the reference's "skip a
         // parameter that never accumulated" (nn.cpp:309) never applies; padding stays at zero
-        k_adamw(m->pslab, m->gslab, m->mslab, m->vslab, lr, b1, b2, eps, wd, c1, c2);
+        k_adamw(m->pslab, m->gslab, m->mslab, m->vslab, lr, b1, b2, eps, wd, c1, c2, clip);
         invalidate_shadows();
         hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
     });

@@ -54,8 +54,9 @@ double k_sumsq_to_host(const Tensor& g);                               // clip_g
 constexpr int SUMSQ_MAX_PARTS = 1024;
 int k_sumsq_parts(const Tensor& g, double* part_dev);
 double k_sum_f64_to_host(const double* part_dev, int64_t n);
+// grad_scale != 1: g is scaled in place first (the clip of ops::clip_grad_norm), in the same pass
 void k_adamw(const Tensor& p, const Tensor& g, const Tensor& m, const Tensor& v, float lr, float b1, float b2,
-             float eps, float wd, float c1, float c2);                 // nn.cpp:301-321
+             float eps, float wd, float c1, float c2, float grad_scale = 1.0f);                 // nn.cpp:301-321
 
 // C[M,N] (+)= op(A) . op(B), row-major, bf16 or fp32 operands, fp32 accumulate
 // (device::gemm, src/device.cpp:91-125). C may be a column slice of a wider
