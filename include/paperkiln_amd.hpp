@@ -243,7 +243,10 @@ Var swa_attention(const Var& q, const Var& k, const Var& v, float scale, int64_t
 // Tied head + loss: mean cross-entropy of logits = h E^T (llama.cpp:88 + ops.cpp:350-376),
 // evaluated in row chunks so that the [N, vocab] logits and their softmax copy never
 // exist as a whole. The chunk's dlogits feed dh and dE immediately; backward scales them.
-Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffer>& targets_dev, int64_t chunk_rows);
+// loss_is_root: the caller promises to call backward() on this loss itself (a unit seed); E's gradient share is then
+// added to E->grad chunk by chunk during the forward instead of being held until the closure runs.
+Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffer>& targets_dev, int64_t chunk_rows,
+                         bool loss_is_root = false);
 // The unfused pair, for parity at sizes where the logits fit: logits = h E^T, then ops::cross_entropy.
 Var matmul_nt(const Var& h, const Var& E);
 Var cross_entropy(const Var& logits, const std::shared_ptr<Buffer>& targets_dev);

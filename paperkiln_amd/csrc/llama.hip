@@ -349,10 +349,10 @@ int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets
         dev_reset_peak();
         const size_t live0 = live_variables();
         Var hid = m->hidden(ids, n, seq_len);
-        Var l = fused_head ? ops::linear_cross_entropy(hid, m->embed, tg, m->head_chunk_rows)
+        Var l = fused_head ? ops::linear_cross_entropy(hid, m->embed, tg, m->head_chunk_rows, do_backward != 0)
                            : ops::cross_entropy(ops::matmul_nt(hid, m->embed), tg);
         hid.reset();
-        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
+        // the allocator's counters move when the host allocates and frees, not when the GPU gets there: no wait here
         if (stats) {
             stats->live_vars_after_forward = static_cast<int64_t>(live_variables() - live0);
             stats->activation_bytes_after_forward = static_cast<int64_t>(dev_live_bytes() - base);

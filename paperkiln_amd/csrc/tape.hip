@@ -689,7 +689,8 @@ Var cross_entropy(const Var& logits, const std::shared_ptr<Buffer>& targets) {
     });
 }
 
-Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffer>& targets, int64_t chunk_rows) {
+Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffer>& targets, int64_t chunk_rows,
+                         bool loss_is_root) {
     const int64_t N = h->data.rows, V = E->data.rows, d = h->data.cols;
     if (d != E->data.cols) shape_fail("matmul: inner dimensions disagree");
     const int* tg = static_cast<const int*>(targets->p);
@@ -699,9 +700,20 @@ Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffe
     // produces dh and dE for an upstream gradient of 1 (dlogits = (P - onehot) / N), and the backward closure only
     // scales them. Nothing of size [N, vocab] outlives its chunk, and no chunk's logits are computed twice.
     const bool want_dh = grad_enabled() && h->requires_grad, want_dE = grad_enabled() && E->requires_grad;
+    // loss_is_root: the caller will seed this loss with 1 and nothing else, so E's share is added to E's gradient as
+    // the chunks go by instead of being kept beside it until the backward closure runs ([V, d] fp32 less at the peak,
+    // one pass over it less); the closure then insists on a unit seed.
+    const bool dE_in_place = want_dE && loss_is_root && E->is_param;
     Tensor dh1, dE1;
     if (want_dh) dh1 = Tensor::make(N, d, h->data.dtype);
-    if (want_dE) dE1 = Tensor::make(V, d, PK_F32);
+    if (want_dE) {
+        if (dE_in_place) {
+            dE1 = E->ensure_grad();
+            if (dE1.dtype != PK_F32) throw std::runtime_error("linear_cross_entropy: the embedding's gradient must be fp32");
+        } else {
+            dE1 = Tensor::make(V, d, PK_F32);
+        }
+    }
     const Tensor& Ec = shadow_of(E);
     Buffer nll(sizeof(float) * N);
     const float g1 = 1.0f / static_cast<float>(N);
@@ -755,14 +767,17 @@ Var linear_cross_entropy(const Var& h, const Var& E, const std::shared_ptr<Buffe
         }
         if (want_dh)
             gemm(dl, false, Ec, false, static_cast<char*>(dh1.ptr()) + r0 * d * hes, dh1.dtype, rows, d, d, 0.0f, dl_ld);
-        if (want_dE) gemm(dl, true, hview, false, dE1.ptr(), PK_F32, V, d, d, r0 == 0 ? 0.0f : 1.0f, dl_ld);
+        if (want_dE) gemm(dl, true, hview, false, dE1.ptr(), PK_F32, V, d, d, r0 == 0 && !dE_in_place ? 0.0f : 1.0f, dl_ld);
     }
     Tensor out = Tensor::make(1, 1, PK_F32);
     k_mean_f32(static_cast<const float*>(nll.p), N, out);  // the loss stays on the device: no wait in mid-step
-    return record(std::move(out), {h, E}, [dh1, dE1](Variable* self) mutable {
+    if (dE_in_place) dE1 = Tensor();
+    return record(std::move(out), {h, E}, [dh1, dE1, dE_in_place](Variable* self) mutable {
         const Var& h = self->parents[0];
         const Var& E = self->parents[1];
         const float g = upstream_scalar(self);  // upstream gradient of the scalar loss
+        if (dE_in_place && g != 1.0f)
+            throw std::runtime_error("linear_cross_entropy: built with loss_is_root, but its gradient is not the unit seed");
         if (h->requires_grad && !dh1.empty()) {
             if (g == 1.0f)
                 h->accumulate_owned(std::move(dh1));
