@@ -949,7 +949,7 @@ Plan make_plan(bool tA, bool tB, int64_t M, int64_t N, int64_t K, int64_t lda, i
     // no second workgroup would come to share the CU.
     const int64_t tiles_large = ((M + 255) / 256) * ((N + 255) / 256);
     p.large = g_force_geo >= 0 ? (g_force_geo == 1 || g_force_geo == 8) : tiles_large >= 240 && (K >= 1024 || tiles_large >= 512);
-    const int64_t ntiles = p.large ? tiles_large : ((M + 127) / 128) * ((N + 127) / 128);
+    int64_t ntiles = p.large ? tiles_large : ((M + 127) / 128) * ((N + 127) / 128);
     // the ring kernels keep offsets and extents in 32 bits
     const int64_t ext_a = (tA ? K : M) * lda * 2, ext_b = (tB ? N : K) * ldb * 2;
     const int64_t ext_max = (int64_t{1} << 30) - 8192;
@@ -966,6 +966,14 @@ Plan make_plan(bool tA, bool tB, int64_t M, int64_t N, int64_t K, int64_t lda, i
     p.S = 1;
     if (ntiles < 192 && K >= 2048) {
         if (ring_ok && g_force_geo < 0) p.ring = ntiles < 64 ? 11 : 6;
+        // ... unless 256 x 256 tiles times slices of 1024 or more fill the chip by themselves (dh of a 4096-row head
+        // chunk, [4096, 512] over 32000: 144 us against 162)
+        const int64_t s_large = std::min<int64_t>({cu_count() / tiles_large, K / 1024, 16});
+        if (ring_ok && g_force_geo < 0 && tiles_large * s_large >= 240) {
+            p.large = true;
+            p.ring = 8;
+            ntiles = tiles_large;
+        }
         const bool one_per_cu = p.ring == 5 || p.ring == 7 || p.ring == 8 || p.ring == 10 || p.ring == 11;
         const int64_t s = std::min<int64_t>({(one_per_cu ? cu_count() : 2 * cu_count()) / ntiles, K / 1024, 16});
         p.S = static_cast<int>(std::max<int64_t>(s, 1));
