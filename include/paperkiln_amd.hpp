@@ -260,5 +260,9 @@ double clip_grad_norm(const std::vector<Var>& params, float max_norm);  // ops.c
 void set_compute_dtype(int dtype);
 int compute_dtype();
 void invalidate_shadows();
+// Builds the compute-dtype copy of a parameter (or of the side-by-side concatenation linear_cat multiplies by) now
+// instead of at its first use, so that a caller measuring activation memory can have them allocated beforehand.
+void prepare_shadow(const Var& W);
+void prepare_shadow_cat(const std::vector<Var>& Ws);
 
 }  // namespace pk

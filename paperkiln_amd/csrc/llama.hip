@@ -330,19 +330,13 @@ int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets
         auto tg = ints_to_dev(host_targets, n);
         // Everything allocated from here on, until backward returns, is activation memory.
         if (compute_dtype() != PK_F32) {  // build the bf16 parameter shadows first: they are not activations
-            NoGrad ng;
-            Tensor probe = Tensor::make(1, m->cfg.d, compute_dtype());
-            k_fill(probe, 0.0f);
             for (const auto& b : m->blocks) {
-                Var x = make_var(probe);
-                (void)ops::linear3(x, b.q, b.k, b.v);
-                (void)ops::linear(x, b.o);
-                (void)ops::linear_cat(x, {b.gate, b.up});
-                Tensor pf = Tensor::make(1, m->cfg.d_ff, compute_dtype());
-                k_fill(pf, 0.0f);
-                (void)ops::linear(make_var(pf), b.down);
+                prepare_shadow_cat({b.q, b.k, b.v});
+                prepare_shadow(b.o);
+                prepare_shadow_cat({b.gate, b.up});
+                prepare_shadow(b.down);
             }
-            (void)ops::matmul_nt(make_var(probe), m->embed);
+            prepare_shadow(m->embed);
         }
         hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
         const size_t base = dev_live_bytes();

@@ -161,6 +161,8 @@ void set_compute_dtype(int dtype) {
 }
 int compute_dtype() { return tape_context().compute; }
 void invalidate_shadows() { tape_context().shadows.reset(); }
+void prepare_shadow(const Var& W) { (void)shadow_of(W); }
+void prepare_shadow_cat(const std::vector<Var>& Ws) { (void)shadow_cat(Ws); }
 
 Tensor& Variable::ensure_grad() {
     if (grad.empty()) {
