@@ -53,13 +53,6 @@ Var make_param(int64_t r, int64_t c, const std::vector<float>& host) {
     return v;
 }
 
-std::shared_ptr<Buffer> ints_to_dev(const int* h, size_t n) {
-    auto b = std::make_shared<Buffer>(sizeof(int) * n);
-    hip_check(hipMemcpyAsync(b->p, h, sizeof(int) * n, hipMemcpyHostToDevice, tape_stream()), "hipMemcpyAsync");
-    hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
-    return b;
-}
-
 struct Block {
     Var ln1_w, ln2_w, q, k, v, o, gate, up, down;
 };
@@ -80,6 +73,26 @@ struct Model {
     // zero_grad, the clip norm and the optimiser step are then one launch each, not one per parameter.
     Tensor pslab, gslab, mslab, vslab;
     long t = 0;
+    // Pinned staging for what a pass sends up (ids, targets, positions): one host copy and asynchronous transfers
+    // instead of three transfers from pageable memory with a wait each. Written only between passes (a pass ends
+    // with a wait for its stream).
+    int* stage = nullptr;
+    size_t stage_cap = 0;
+    ~Model() {
+        if (stage) (void)hipHostFree(stage);
+    }
+    int* staging(size_t n_ints) {
+        if (n_ints > stage_cap) {
+            if (stage) hip_check(hipHostFree(stage), "hipHostFree");
+            stage = nullptr;
+            stage_cap = 0;
+            void* p = nullptr;
+            hip_check(hipHostMalloc(&p, sizeof(int) * n_ints, hipHostMallocDefault), "hipHostMalloc");
+            stage = static_cast<int*>(p);
+            stage_cap = n_ints;
+        }
+        return stage;
+    }
 
     void reg(const std::string& name, const Var& p) { named.emplace_back(name, p); }
 
@@ -170,12 +183,7 @@ struct Model {
     }
 
     // Llama::forward (llama.cpp:71-89) up to the final norm; positions restart per sequence.
-    Var hidden(const std::shared_ptr<Buffer>& ids, int64_t n, int64_t seq_len) const {
-        const int64_t sl = seq_len == 0 ? n : seq_len;
-        if (n % sl != 0) shape_fail("ids not a multiple of seq_len");
-        std::vector<int> pos(n);
-        for (int64_t i = 0; i < n; ++i) pos[i] = static_cast<int>(i % sl);
-        auto pos_dev = ints_to_dev(pos.data(), pos.size());
+    Var hidden(const std::shared_ptr<Buffer>& ids, const std::shared_ptr<Buffer>& pos_dev, int64_t n, int64_t seq_len) const {
         Var h = ops::embedding(embed, ids, n);
         for (const Block& blk : blocks) {
             if (checkpoint_blocks && grad_enabled()) {
@@ -325,9 +333,23 @@ int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets
             if (host_targets[i] < 0 || host_targets[i] >= m->cfg.vocab)
                 throw std::runtime_error("cross_entropy: target out of range");
         m->checkpoint_blocks = checkpoint_blocks != 0;
+        const int64_t sl = seq_len == 0 ? n : seq_len;
+        if (n % sl != 0) shape_fail("ids not a multiple of seq_len");
         k_fill(m->gslab, 0.0f);  // zero_grad: every parameter's gradient is a view of this slab
-        auto ids = ints_to_dev(host_ids, n);
-        auto tg = ints_to_dev(host_targets, n);
+        // ids, targets and positions (which restart per sequence, llama.cpp:73-76) go up from pinned memory behind
+        // the fill, without a wait
+        int* st = m->staging(static_cast<size_t>(3 * n));
+        std::memcpy(st, host_ids, sizeof(int) * n);
+        std::memcpy(st + n, host_targets, sizeof(int) * n);
+        for (int64_t i = 0; i < n; ++i) st[2 * n + i] = static_cast<int>(i % sl);
+        auto up = [&](const int* src) {
+            auto b = std::make_shared<Buffer>(sizeof(int) * n);
+            hip_check(hipMemcpyAsync(b->p, src, sizeof(int) * n, hipMemcpyHostToDevice, tape_stream()), "hipMemcpyAsync");
+            return b;
+        };
+        auto ids = up(st);
+        auto tg = up(st + n);
+        auto pos_dev = up(st + 2 * n);
         // Everything allocated from here on, until backward returns, is activation memory.
         if (compute_dtype() != PK_F32) {  // build the bf16 parameter shadows first: they are not activations
             for (const auto& b : m->blocks) {
@@ -338,11 +360,10 @@ int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets
             }
             prepare_shadow(m->embed);
         }
-        hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
-        const size_t base = dev_live_bytes();
+        const size_t base = dev_live_bytes();  // the allocator's host-side counters: nothing to wait for
         dev_reset_peak();
         const size_t live0 = live_variables();
-        Var hid = m->hidden(ids, n, seq_len);
+        Var hid = m->hidden(ids, pos_dev, n, seq_len);
         Var l = fused_head ? ops::linear_cross_entropy(hid, m->embed, tg, m->head_chunk_rows, do_backward != 0)
                            : ops::cross_entropy(ops::matmul_nt(hid, m->embed), tg);
         hid.reset();
