@@ -338,7 +338,7 @@ int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets
         k_fill(m->gslab, 0.0f);  // zero_grad: every parameter's gradient is a view of this slab
         // ids, targets and positions (which restart per sequence, llama.cpp:73-76) go up from pinned memory behind
         // the fill, without a wait
-        int* st = m->staging(static_cast<size_t>(3 * n));
+        int* st = m->staging(static_cast<size_t>(3 * n + 1));
         std::memcpy(st, host_ids, sizeof(int) * n);
         std::memcpy(st + n, host_targets, sizeof(int) * n);
         for (int64_t i = 0; i < n; ++i) st[2 * n + i] = static_cast<int>(i % sl);
@@ -373,11 +373,12 @@ int pk_llama_loss_backward(void* h, const int* host_ids, const int* host_targets
             stats->activation_bytes_after_forward = static_cast<int64_t>(dev_live_bytes() - base);
         }
         if (do_backward) backward(l);
+        // the loss comes back into the pinned staging's spare word behind the last kernel: one wait ends the pass
+        float* hl = reinterpret_cast<float*>(st + 3 * n);
+        hip_check(hipMemcpyAsync(hl, l->data.ptr(), 4, hipMemcpyDeviceToHost, tape_stream()), "hipMemcpyAsync");
         hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
         if (stats) stats->peak_activation_bytes = static_cast<int64_t>(dev_peak_bytes() - base);
-        float hl = 0.0f;
-        hip_check(hipMemcpy(&hl, l->data.ptr(), 4, hipMemcpyDeviceToHost), "hipMemcpy");
-        *loss = hl;
+        *loss = *hl;
     });
 }
 
