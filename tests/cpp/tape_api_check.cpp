@@ -301,6 +301,50 @@ void linear_add_case(int dtype, const char* name, int T, int din, int dout, doub
     pk::set_compute_dtype(PK_F32);
 }
 
+// The chunked tied head with the cross-entropy inside the logits product against the same head through fp32 logits
+// and the row kernel, on logits of a few tens in size (far from the ~0.01 of a freshly initialised model): the
+// in-product path carries the row maximum and the scaling in the exponent of exp2, which is where a large logit
+// would show.
+void head_case() {
+    std::printf("linear_cross_entropy, logits of size ~50: inside the product vs fp32 logits + row kernel\n");
+    const int T = 300, d = 64, V = 1000;
+    const auto hh = draw(static_cast<size_t>(T) * d, 61, 3.0), he = draw(static_cast<size_t>(V) * d, 62, 3.0);
+    std::vector<int> target(T);
+    for (int i = 0; i < T; ++i) target[i] = (37 * i + 11) % V;
+    auto tg = device_ints(target);
+    pk::set_compute_dtype(PK_BF16);
+    struct Run {
+        float loss;
+        std::vector<float> gh, ge;
+    };
+    auto run = [&](int in_product) {
+        const int before = pk_set_head_kernel(in_product);
+        pk::Var h = pk::make_var(pk::upload(hh.data(), T, d, PK_BF16), true);
+        pk::Var E = pk::make_var(pk::upload(he.data(), V, d), true);
+        E->is_param = true;
+        pk::Var loss = pk::ops::linear_cross_entropy(h, E, tg, 128);  // 3 chunks, the last of 44 rows
+        pk::backward(loss);
+        Run r{host(loss->data)[0], host(h->grad), host(E->grad)};
+        pk::invalidate_shadows();
+        pk_set_head_kernel(before);
+        return r;
+    };
+    const Run rows = run(0), prod = run(1);
+    auto rel = [](const std::vector<float>& a, const std::vector<float>& b) {
+        double w = 0.0, size = 0.0;
+        for (size_t i = 0; i < a.size(); ++i) {
+            w = std::fmax(w, std::fabs(static_cast<double>(a[i]) - b[i]));
+            size = std::fmax(size, std::fabs(static_cast<double>(b[i])));
+        }
+        return w / std::fmax(size, 1e-30);
+    };
+    check(std::isfinite(prod.loss) && prod.loss > 10.0f, "loss is finite and large (the logits are)", prod.loss);
+    check(std::fabs(prod.loss - rows.loss) <= 2e-5 * rows.loss, "loss", std::fabs(prod.loss - rows.loss));
+    check(rel(prod.gh, rows.gh) <= 1.0 / 64, "dh", rel(prod.gh, rows.gh));
+    check(rel(prod.ge, rows.ge) <= 1.0 / 64, "dE", rel(prod.ge, rows.ge));
+    pk::set_compute_dtype(PK_F32);
+}
+
 void behaviour_case() {
     std::printf("tape behaviour and errors\n");
     const auto h = draw(8 * 4, 31, 1.0);
@@ -359,6 +403,7 @@ int main() {
     linear_add_case(PK_F32, "float32 (product, then add)", 40, 24, 16, 1e-6);
     linear_add_case(PK_BF16, "bfloat16, edge tiles", 200, 72, 136, 1.0 / 128);
     linear_add_case(PK_BF16, "bfloat16, long contraction", 300, 1376, 64, 1.0 / 128);
+    head_case();
     behaviour_case();
     if (g_failures == 0) {
         std::printf("tape_api_check PASSED\n");
