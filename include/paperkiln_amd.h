@@ -253,12 +253,13 @@ int pk_op_sumsq(const float* g, int64_t n, double* host_out, void* stream);
  * op = transpose when the flag is set (A is [k,m] then, B is [n,k]); operands dtype, output c_dtype, fp32 accumulate. */
 int pk_op_gemm(const void* a, int trans_a, const void* b, int trans_b, void* c, int64_t m, int64_t n, int64_t k,
                int dtype, int c_dtype, int accumulate, void* stream);
-/* Which kernel multiplies bf16 operands. 1 (default) and 2: this library's own matrix-core GEMM (the counterpart of
- * the reference's tiled kernel, src/cuda_resident.cu:141-171) for everything it takes (16-byte aligned rows, sizes
- * that are multiples of 8) -- measured on the MI355X it is ahead of rocBLAS or level with it on every Linear
- * product of a d = 512 block and of a 32000-word tied head -- in
- * the form it picks per shape; rocBLAS for the rest. 0: rocBLAS for everything, as for fp32 operands. Measurement
- * settings, all like 2 but with one form forced: 3 / 4 the register-staged
+/* Which kernel multiplies bf16 operands. 1 (default): this library's own matrix-core GEMM (the counterpart of the
+ * reference's tiled kernel, src/cuda_resident.cu:141-171) for everything it takes (16-byte aligned rows, sizes that
+ * are multiples of 8) -- measured on the MI355X it is ahead of rocBLAS or level with it on every Linear product of a
+ * d = 512 block and of a 32000-word tied head -- in the form it picks per shape, rocBLAS for the rest; and the
+ * weight-gradient products X^T dY of a backward pass over 2048 tokens or more are held back and multiplied several
+ * at a time as one grouped launch. 2: the same kernel, every product on its own. 0: rocBLAS for everything, as for
+ * fp32 operands. Measurement settings, all like 2 but with one form forced: 3 / 4 the register-staged
  * kernel with 128 x 128 / 256 x 256 tiles; 5, 6, 7 the LDS-ring kernel with 128 x 128 tiles and 4, 2, 3 ring slots;
  * 8 the ring kernel with 256 x 256 tiles; 9, 10, 11 the ring kernel with 128 x 128 tiles shared by two wavefront sets
  * and 2, 3, 4 slots. Process-wide; returns the previous setting (0, 1 or 2). The environment variable

@@ -123,6 +123,8 @@ struct TapeContext {
     int compute = PK_F32;
     struct Shadows;  // compute-dtype copies of fp32 parameters (tape.hip)
     std::shared_ptr<Shadows> shadows;
+    struct Pending;  // weight-gradient products a backward pass has held back to run several as one launch (tape.hip)
+    std::shared_ptr<Pending> pending;
 };
 TapeContext& tape_context();
 class ContextScope {

@@ -196,9 +196,11 @@ def set_head_kernel(in_product: bool) -> int:
 
 
 def set_gemm_backend(mode: int) -> int:
-    """Choose the kernel for bf16 GEMMs (pk_set_gemm_backend): 1 (default) and 2 = the library's own matrix-core
-    kernel wherever it applies, in the form it picks per shape, 0 = rocBLAS only, 3 .. 11 = the own kernel
-    with one form forced (measurements; see include/paperkiln_amd.h). Returns the previous setting (0, 1, 2)."""
+    """Choose the kernel for bf16 GEMMs (pk_set_gemm_backend): 1 (default) = the library's own matrix-core kernel
+    wherever it applies, in the form it picks per shape, with a backward pass's weight-gradient products multiplied
+    several at a time as one grouped launch; 2 = the same with every product on its own; 0 = rocBLAS only; 3 .. 11 =
+    the own kernel with one form forced (measurements; see include/paperkiln_amd.h). Returns the previous setting
+    (0, 1, 2)."""
     return int(_lib.lib().pk_set_gemm_backend(int(mode)))
 
 

@@ -81,6 +81,21 @@ struct HeadArgs {
 };
 constexpr float LOG2E = 1.4426950408889634f;
 
+// Several products of one launch (gemm_ring's EPI 3): C_p (+)= op(A_p) op(B_p), p < count, all with the contraction
+// length, transposition flags and result type of the launch; the workgroups walk the tiles of all of them as one
+// sequence (problem after problem, each row by row). For products that are each too small to fill the chip and would
+// otherwise each cut their contraction into slices and add partial results afterwards.
+constexpr int GROUP_MAX = 8;
+struct GroupArgs {
+    int count;
+    int tile_end[GROUP_MAX];  // tiles of problems 0 .. p
+    const uint16_t* a[GROUP_MAX];
+    const uint16_t* b[GROUP_MAX];
+    void* c[GROUP_MAX];
+    int M[GROUP_MAX], N[GROUP_MAX], tiles_n[GROUP_MAX];
+    int lda[GROUP_MAX], ldb[GROUP_MAX], ldc[GROUP_MAX];
+};
+
 // Transposing operand read in natural k order: lane (c32, g) receives rows row0 + 8g .. 8g + 7 of column
 // col0 + c32 of a [k][column] tile.
 __device__ inline bf16x8 read_tr_nat(const uint16_t* tile, int pitch, int row0, int col0, int lane) {
@@ -371,8 +386,9 @@ struct TileStore {
 // are multiplied and its result is stored, so a tile's first round trip to memory is paid once per workgroup.
 template <typename G, bool TA, bool TB, bool CF32, int NS, bool SPREAD, int EPI = 0>
 __global__ __launch_bounds__(G::NTHR, NS * (RingOp<TA, G::BM, G::NTHR / 64>::BYTES + RingOp<!TB, G::BN, G::NTHR / 64>::BYTES) <= 80 * 1024 ? 2 : 1)
-void gemm_ring(GemmArgs g, HeadArgs hd) {
-    static_assert(EPI == 0 || (G::KS == 1 && !CF32), "the head's epilogues: one wavefront set, bf16 result");
+void gemm_ring(GemmArgs g, HeadArgs hd, GroupArgs gr) {
+    static_assert(EPI == 0 || EPI == 3 || (G::KS == 1 && !CF32), "the head's epilogues: one wavefront set, bf16 result");
+    constexpr bool GROUPED = EPI == 3;
     constexpr int BM = G::BM, BN = G::BN, NTHR = G::NTHR, FM = G::FM, FN = G::FN, NW = NTHR / 64;
     using OA = RingOp<TA, BM, NW>;
     using OB = RingOp<!TB, BN, NW>;
@@ -396,31 +412,53 @@ void gemm_ring(GemmArgs g, HeadArgs hd) {
     // -- and on whole rows of tiles. (Walking tiles in blocks of 4 or 8 rows instead halves what the L2s fetch for
     // [4096, 32000] x 512, 543 -> ~270 MB, and changes its time by nothing -- the last-level cache serves those misses
     // at 7 TB/s -- while [8192, 2752] x 512, whose weight matrix fits an L2 whole, loses 20 %.)
-    const int ntiles = g.tiles_m * g.tiles_n, total = ntiles * g.splits, per_xcd = (total + 7) / 8, V = per_xcd * 8;
+    const int ntiles = GROUPED ? gr.tile_end[gr.count - 1] : g.tiles_m * g.tiles_n;
+    const int total = ntiles * g.splits, per_xcd = (total + 7) / 8, V = per_xcd * 8;
     const int stride = static_cast<int>(gridDim.x);
     struct Block {
-        int m0, n0, k_begin, k_end, z;
+        int m0, n0, k_begin, k_end, z, p;  // p: which problem of a grouped launch
     };
     auto next_block = [&](int v, Block& bl) {  // first virtual block at or after v (in steps of the grid) that is a tile
         for (; v < V; v += stride) {
             const int u = (v & 7) * per_xcd + (v >> 3);
             if (u >= total) continue;
-            const int z = u / ntiles, t = u - z * ntiles;
-            const int tm = t / g.tiles_n;
+            const int z = u / ntiles;
+            int t = u - z * ntiles, p = 0, tiles_n = g.tiles_n;
+            if (GROUPED) {
+                while (t >= gr.tile_end[p]) ++p;
+                if (p > 0) t -= gr.tile_end[p - 1];
+                tiles_n = gr.tiles_n[p];
+            }
+            const int tm = t / tiles_n;
             bl.m0 = tm * BM;
-            bl.n0 = (t - tm * g.tiles_n) * BN;
+            bl.n0 = (t - tm * tiles_n) * BN;
             bl.z = z;
+            bl.p = p;
             bl.k_begin = z * g.k_per_split;
             bl.k_end = min(g.K, bl.k_begin + g.k_per_split);
             return v;
         }
         return V;
     };
+    // the operands and sizes of the problem a block belongs to
+    struct Prob {
+        const uint16_t* a;
+        const uint16_t* b;
+        void* c;
+        int M, N;
+        int64_t lda, ldb, ldc;
+    };
+    auto prob = [&](const Block& bl) -> Prob {
+        if (GROUPED) return Prob{gr.a[bl.p], gr.b[bl.p], gr.c[bl.p], gr.M[bl.p], gr.N[bl.p], gr.lda[bl.p], gr.ldb[bl.p], gr.ldc[bl.p]};
+        return Prob{g.a, g.b, g.c, g.M, g.N, g.lda, g.ldb, g.ldc};
+    };
 
     // ---- fetch side: a stream of slices, tile after tile ----
     uint32_t offa[OA::PER], offb[OB::PER], offa_c[OA::PER], offb_c[OB::PER];
-    lane_offsets<OA>(offa, w, lane, g.lda);
-    lane_offsets<OB>(offb, w, lane, g.ldb);
+    if (!GROUPED) {  // a grouped launch forms them per tile: the row pitches are the problem's
+        lane_offsets<OA>(offa, w, lane, g.lda);
+        lane_offsets<OB>(offb, w, lane, g.ldb);
+    }
     const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
     const uint32_t dst_a = lds0 + w * OA::PER * 1024u, dst_b = lds0 + OA::BYTES + w * OB::PER * 1024u;
     Block fb;
@@ -438,17 +476,22 @@ void gemm_ring(GemmArgs g, HeadArgs hd) {
         }
         f_nslices = (fb.k_end - fb.k_begin + BK - 1) / BK;
         f_ktail = (fb.k_end - fb.k_begin) % BK;
-        da = tile_desc<TA>(g.a, g.lda, fb.m0, g.M, fb.k_begin, fb.k_end);
-        db = tile_desc<!TB>(g.b, g.ldb, fb.n0, g.N, fb.k_begin, fb.k_end);
+        const Prob fp = prob(fb);
+        if (GROUPED) {
+            lane_offsets<OA>(offa, w, lane, fp.lda);
+            lane_offsets<OB>(offb, w, lane, fp.ldb);
+        }
+        da = tile_desc<TA>(fp.a, fp.lda, fb.m0, fp.M, fb.k_begin, fb.k_end);
+        db = tile_desc<!TB>(fp.b, fp.ldb, fb.n0, fp.N, fb.k_begin, fb.k_end);
         // the masked lane offsets: used by every slice of a [k][column] operand, by the last slice of a [row][k] one
-        if (TA ? fb.m0 + BM > g.M : f_ktail != 0)
-            lane_offsets_masked<OA, TA>(offa_c, offa, w, lane, fb.m0, g.M, f_ktail);
+        if (TA ? fb.m0 + BM > fp.M : f_ktail != 0)
+            lane_offsets_masked<OA, TA>(offa_c, offa, w, lane, fb.m0, fp.M, f_ktail);
         else {
 #pragma unroll
             for (int j = 0; j < OA::PER; ++j) offa_c[j] = offa[j];
         }
-        if (!TB ? fb.n0 + BN > g.N : f_ktail != 0)
-            lane_offsets_masked<OB, !TB>(offb_c, offb, w, lane, fb.n0, g.N, f_ktail);
+        if (!TB ? fb.n0 + BN > fp.N : f_ktail != 0)
+            lane_offsets_masked<OB, !TB>(offb_c, offb, w, lane, fb.n0, fp.N, f_ktail);
         else {
 #pragma unroll
             for (int j = 0; j < OB::PER; ++j) offb_c[j] = offb[j];
@@ -552,7 +595,7 @@ void gemm_ring(GemmArgs g, HeadArgs hd) {
         const int srow = (static_cast<int>(threadIdx.x) + k * NTHR) / ST::CPR;
         // bf16 strips hold the i-th 32-row block of every wavefront row: strip row -> tile row (srow / 32) FM 32 + srow % 32
         const int trow = CF32 ? srow : (srow >> 5) * FM * 32 + (srow & 31);
-        coff[k] = (static_cast<uint32_t>(trow) * static_cast<uint32_t>(g.ldc) + st_ch * ST::EPC) * ES;
+        coff[k] = (static_cast<uint32_t>(trow) * static_cast<uint32_t>(g.ldc) + st_ch * ST::EPC) * ES;  // (not grouped)
     }
 
     f32x16 acc[FM][FN];
@@ -661,15 +704,16 @@ void gemm_ring(GemmArgs g, HeadArgs hd) {
         }
         // descriptor of C from the tile's first element on (rows past the matrix are dropped by the range check,
         // columns past it by the lane's offset)
-        CT* ctile = static_cast<CT*>(g.c) + (g.part_stride ? static_cast<int64_t>(bl.z) * g.part_stride : 0) +
-                    static_cast<int64_t>(bl.m0) * g.ldc + bl.n0;
-        const int64_t cleft = (static_cast<int64_t>(g.M - bl.m0 - 1) * g.ldc + (g.N - bl.n0)) * ES;
+        const Prob cp = prob(bl);
+        CT* ctile = static_cast<CT*>(cp.c) + (g.part_stride ? static_cast<int64_t>(bl.z) * g.part_stride : 0) +
+                    static_cast<int64_t>(bl.m0) * cp.ldc + bl.n0;
+        const int64_t cleft = (static_cast<int64_t>(cp.M - bl.m0 - 1) * cp.ldc + (cp.N - bl.n0)) * ES;
         const uint32_t crec = cleft > 0x7ffffff0 ? 0x7ffffff0u : static_cast<uint32_t>(cleft);
         const uint64_t ca = reinterpret_cast<uint64_t>(ctile);
         const u32x4 crs = {static_cast<uint32_t>(ca), static_cast<uint32_t>(ca >> 32) & 0xffffu, crec, 0x00020000u};
-        CT* dtile = g.d ? static_cast<CT*>(const_cast<void*>(g.d)) + static_cast<int64_t>(bl.m0) * g.ldc + bl.n0 : ctile;
+        CT* dtile = g.d ? static_cast<CT*>(const_cast<void*>(g.d)) + static_cast<int64_t>(bl.m0) * cp.ldc + bl.n0 : ctile;
         const __amdgpu_buffer_rsrc_t crs_b = __builtin_amdgcn_make_buffer_rsrc(dtile, 0, static_cast<int>(crec), 0x00020000);
-        const uint32_t cmask = bl.n0 + st_ch * ST::EPC < g.N ? 0u : OUTSIDE;
+        const uint32_t cmask = bl.n0 + st_ch * ST::EPC < cp.N ? 0u : OUTSIDE;
         CT* cs = reinterpret_cast<CT*>(strip);
 #pragma unroll
         for (int ph = 0; ph < ST::PHASES; ++ph) {
@@ -692,12 +736,17 @@ void gemm_ring(GemmArgs g, HeadArgs hd) {
             }
             __syncthreads();
             // rows of C this strip holds start at tile row (ws FM + i) 32 (fp32) or i 32 (bf16, plus the lane's part)
-            const uint32_t soff = static_cast<uint32_t>((CF32 ? ws * FM + i : i) * 32) * static_cast<uint32_t>(g.ldc) * ES;
+            const uint32_t soff = static_cast<uint32_t>((CF32 ? ws * FM + i : i) * 32) * static_cast<uint32_t>(cp.ldc) * ES;
 #pragma unroll
             for (int k = 0; k < ST::PER_PHASE; ++k) {
                 const int srow = (static_cast<int>(threadIdx.x) + k * NTHR) / ST::CPR;
                 u32x4 v = *reinterpret_cast<const u32x4*>(cs + srow * ST::CP + st_ch * ST::EPC);
-                const uint32_t off = coff[k] | cmask;
+                uint32_t off = coff[k];
+                if (GROUPED) {  // the row pitch is the problem's
+                    const int trow = CF32 ? srow : (srow >> 5) * FM * 32 + (srow & 31);
+                    off = (static_cast<uint32_t>(trow) * static_cast<uint32_t>(cp.ldc) + st_ch * ST::EPC) * ES;
+                }
+                off |= cmask;
                 if (g.beta) {
                     const u32x4 old = __builtin_amdgcn_raw_buffer_load_b128(crs_b, static_cast<int>(off), static_cast<int>(soff), 0);
                     if (CF32) {
@@ -868,10 +917,10 @@ void launch_form(bool tA, bool tB, const GemmArgs& g, dim3 grid, hipStream_t st)
 }
 template <typename G, bool CF32, int NS, bool SPREAD>
 void launch_ring_form(bool tA, bool tB, const GemmArgs& g, dim3 grid, hipStream_t st) {
-    if (!tA && !tB) hipLaunchKernelGGL((gemm_ring<G, false, false, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g, HeadArgs{});
-    if (!tA && tB) hipLaunchKernelGGL((gemm_ring<G, false, true, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g, HeadArgs{});
-    if (tA && !tB) hipLaunchKernelGGL((gemm_ring<G, true, false, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g, HeadArgs{});
-    if (tA && tB) hipLaunchKernelGGL((gemm_ring<G, true, true, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g, HeadArgs{});
+    if (!tA && !tB) hipLaunchKernelGGL((gemm_ring<G, false, false, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g, HeadArgs{}, GroupArgs{});
+    if (!tA && tB) hipLaunchKernelGGL((gemm_ring<G, false, true, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g, HeadArgs{}, GroupArgs{});
+    if (tA && !tB) hipLaunchKernelGGL((gemm_ring<G, true, false, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g, HeadArgs{}, GroupArgs{});
+    if (tA && tB) hipLaunchKernelGGL((gemm_ring<G, true, true, CF32, NS, SPREAD>), grid, dim3(G::NTHR), 0, st, g, HeadArgs{}, GroupArgs{});
 }
 int cu_count() {
     static const int n = [] {
@@ -1088,7 +1137,7 @@ void launch_head(GemmArgs g, const HeadArgs& hd, hipStream_t st) {
     const int64_t vblocks = static_cast<int64_t>((g.tiles_m * g.tiles_n + 7) / 8 * 8);
     const int64_t slots = cu_count() / 8 * 8 * (G::BM > 128 ? 1 : 2);
     const unsigned gx = static_cast<unsigned>(std::min<int64_t>(vblocks, slots));
-    hipLaunchKernelGGL((gemm_ring<G, false, true, false, 2, true, EPI>), dim3(gx), dim3(G::NTHR), 0, st, g, hd);
+    hipLaunchKernelGGL((gemm_ring<G, false, true, false, 2, true, EPI>), dim3(gx), dim3(G::NTHR), 0, st, g, hd, GroupArgs{});
     hip_check(hipGetLastError(), "gemm_ring (head) launch");
 }
 }  // namespace
@@ -1133,6 +1182,58 @@ bool gemm_head_dlogits(const void* a, int64_t lda, const void* b, int64_t ldb, i
     hd.row_inv = row_inv;
     hd.gscale = gscale;
     launch_head<GeoLarge, 2>(g, hd, st);
+    return true;
+}
+
+// ---- several small weight-gradient products as one launch ----
+// C_p += A_p^T B_p, p < count <= GROUP_MAX: A_p [K, M_p] and B_p [K, N_p] bf16 with row pitches lda / ldb, C_p
+// [M_p, N_p] fp32 with row pitch ldc, one contraction length K for all. The products of a layer's backward pass
+// (X^T dY per weight, K = every token) are each a few dozen 128 x 128 tiles: alone each would cut its contraction into
+// slices to fill the chip and add the partial products afterwards; together their tiles fill it with whole
+// contractions. False, with nothing done, when an operand is not what the ring kernel takes or the tiles are too few
+// to be worth it (the caller then multiplies them one by one).
+bool gemm_mfma_grouped_tn(const GroupedProduct* ps, int count, int64_t K, hipStream_t st) {
+    if (count < 2 || count > GROUP_MAX || K < 2048) return false;
+    GroupArgs gr{};
+    gr.count = count;
+    int tiles = 0;
+    const int64_t ext_max = (int64_t{1} << 30) - 8192;
+    for (int p = 0; p < count; ++p) {
+        const GroupedProduct& q = ps[p];
+        if (!takes(q.a, true, q.lda, q.b, q.ldb, q.M, q.N, K) || !aligned16(q.c) || q.ldc % 4) return false;
+        if (K * q.lda * 2 >= ext_max || K * q.ldb * 2 >= ext_max || q.lda >= (1 << 21) || q.ldb >= (1 << 21) || q.ldc >= (1 << 20))
+            return false;
+        gr.a[p] = static_cast<const uint16_t*>(q.a);
+        gr.b[p] = static_cast<const uint16_t*>(q.b);
+        gr.c[p] = q.c;
+        gr.M[p] = static_cast<int>(q.M);
+        gr.N[p] = static_cast<int>(q.N);
+        gr.lda[p] = static_cast<int>(q.lda);
+        gr.ldb[p] = static_cast<int>(q.ldb);
+        gr.ldc[p] = static_cast<int>(q.ldc);
+        gr.tiles_n[p] = static_cast<int>((q.N + 127) / 128);
+        tiles += static_cast<int>((q.M + 127) / 128) * gr.tiles_n[p];
+        gr.tile_end[p] = tiles;
+    }
+    for (int p = count; p < GROUP_MAX; ++p) gr.tile_end[p] = tiles;
+    // worth it from about 3/8 of the CUs busy with whole contractions (measured: 196 tiles x 8192 in 69 us against 132
+    // for the same four products one by one); with more tiles than CUs the 4-wavefront form, two workgroups per CU
+    if (tiles < cu_count() * 3 / 8) return false;
+    GemmArgs g = gemm_args(ps[0].a, ps[0].lda, ps[0].b, ps[0].ldb, ps[0].M, ps[0].N, K);
+    g.beta = 1;
+    g.splits = 1;
+    g.tiles_m = g.tiles_n = 0;
+    const int64_t vblocks = (static_cast<int64_t>(tiles) + 7) / 8 * 8;
+    if (tiles <= cu_count()) {
+        const unsigned gx = static_cast<unsigned>(std::min<int64_t>(vblocks, cu_count() / 8 * 8));
+        hipLaunchKernelGGL((gemm_ring<GeoSmallK2, true, false, true, 4, true, 3>), dim3(gx), dim3(GeoSmallK2::NTHR), 0, st, g,
+                           HeadArgs{}, gr);
+    } else {
+        const unsigned gx = static_cast<unsigned>(std::min<int64_t>(vblocks, cu_count() / 8 * 8 * 2));
+        hipLaunchKernelGGL((gemm_ring<GeoSmall, true, false, true, 2, false, 3>), dim3(gx), dim3(GeoSmall::NTHR), 0, st, g,
+                           HeadArgs{}, gr);
+    }
+    hip_check(hipGetLastError(), "gemm_ring (grouped) launch");
     return true;
 }
 

@@ -20,6 +20,21 @@ struct TapeContext::Shadows {
     std::unordered_map<const Variable*, Tensor> cat;     // [W_0 | W_1 | ...], keyed by the first weight
 };
 
+// Weight-gradient products dW += X^T dY that the Linear closures of a running backward pass have handed in instead
+// of multiplying at once. Each is a few dozen output tiles over a contraction as long as the token count; several
+// of them fill the chip as one launch where each alone would have to cut its contraction into slices and add partial
+// products afterwards. They are multiplied when eight have gathered and whenever a backward pass (a checkpointed
+// segment's included) ends, so every parameter's gradient is complete when backward() returns.
+struct TapeContext::Pending {
+    struct Job {
+        Tensor x, dy;           // [tokens, in], [tokens, columns of all the weights multiplied together]
+        int64_t col0, ncols;    // this weight's columns of dy
+        Var W;
+    };
+    std::vector<Job> jobs;
+    int depth = 0;  // run_backward calls in progress
+};
+
 namespace {
 thread_local bool g_grad_enabled = true;
 thread_local TapeContext g_own_context;            // what a thread works on outside any ContextScope
@@ -86,9 +101,71 @@ std::vector<Variable*> backward_order(const Var& root) {
     return order;
 }
 
+TapeContext::Pending& pending() {
+    TapeContext& c = tape_context();
+    if (!c.pending) c.pending = std::make_shared<TapeContext::Pending>();
+    return *c.pending;
+}
+
+void flush_weight_gradients() {
+    auto& jobs = pending().jobs;
+    size_t i = 0;
+    while (i < jobs.size()) {
+        // a run of jobs with one token count
+        size_t j = i;
+        GroupedProduct gp[8];
+        while (j < jobs.size() && j - i < 8 && jobs[j].x.rows == jobs[i].x.rows) {
+            const auto& job = jobs[j];
+            Tensor& g = job.W->ensure_grad();
+            gp[j - i] = GroupedProduct{job.x.ptr(), job.x.cols,
+                                       static_cast<const char*>(job.dy.ptr()) + job.col0 * static_cast<int64_t>(job.dy.esize()),
+                                       job.dy.cols, static_cast<float*>(g.ptr()), g.cols, job.x.cols, job.ncols};
+            ++j;
+        }
+        const int64_t K = jobs[i].x.rows;
+        if (!gemm_mfma_grouped_tn(gp, static_cast<int>(j - i), K, tape_stream())) {
+            for (size_t k = 0; k < j - i; ++k)
+                if (!gemm_mfma_bf16(gp[k].a, true, gp[k].lda, gp[k].b, false, gp[k].ldb, gp[k].c, PK_F32, gp[k].M, gp[k].N, K,
+                                    gp[k].ldc, 1.0f, tape_stream()))
+                    throw std::runtime_error("a deferred weight-gradient product was refused by the kernel it was queued for");
+        }
+        i = j;
+    }
+    jobs.clear();
+}
+
+// Whether dW += x^T dy[:, col0 : col0 + ncols] can wait in the queue: a backward pass is running and the product is one
+// the hand-written kernel takes (bf16 operands, fp32 parameter gradient, aligned, a contraction worth grouping).
+bool weight_gradient_can_wait(const Tensor& x, const Tensor& dy, int64_t col0, int64_t ncols, const Var& W) {
+    if (pending().depth == 0 || gemm_backend() != 1) return false;
+    if (x.dtype != PK_BF16 || dy.dtype != PK_BF16 || !W->is_param || x.rows != dy.rows || x.rows < 2048) return false;
+    if (x.cols % 8 || dy.cols % 8 || col0 % 8 || ncols % 8 || W->data.rows != x.cols || W->data.cols != ncols) return false;
+    return W->grad.empty() || W->grad.dtype == PK_F32;
+}
+void hold_weight_gradient(const Tensor& x, const Tensor& dy, int64_t col0, int64_t ncols, const Var& W) {
+    auto& pd = pending();
+    if (pd.jobs.size() == 8) flush_weight_gradients();
+    pd.jobs.push_back(TapeContext::Pending::Job{x, dy, col0, ncols, W});
+}
+bool defer_weight_gradient(const Tensor& x, const Tensor& dy, int64_t col0, int64_t ncols, const Var& W) {
+    if (!weight_gradient_can_wait(x, dy, col0, ncols, W)) return false;
+    hold_weight_gradient(x, dy, col0, ncols, W);
+    return true;
+}
+
 void run_backward(const Var& root) {
-    for (Variable* n : backward_order(root))
-        if (n->backward_fn && !n->grad.empty()) n->backward_fn();
+    auto& pd = pending();
+    ++pd.depth;
+    try {
+        for (Variable* n : backward_order(root))
+            if (n->backward_fn && !n->grad.empty()) n->backward_fn();
+        flush_weight_gradients();
+    } catch (...) {
+        pd.jobs.clear();
+        --pd.depth;
+        throw;
+    }
+    --pd.depth;
 }
 
 float scalar_to_host(const Tensor& t) {
@@ -298,8 +375,8 @@ Var linear(const Var& x, const Var& W) {
             gemm(self->grad, false, shadow_of(W), true, dx.ptr(), dx.dtype, dx.rows, dx.cols, dx.cols, 0.0f);
             x->accumulate_owned(std::move(dx));
         }
-        if (W->requires_grad) {  // dW += X^T dY (ops.cpp:52-55), straight into the fp32 grad
-            Tensor& g = W->ensure_grad();
+        if (W->requires_grad && !defer_weight_gradient(x->data, self->grad, 0, W->data.cols, W)) {
+            Tensor& g = W->ensure_grad();  // dW += X^T dY (ops.cpp:52-55), straight into the fp32 grad
             gemm(x->data, true, self->grad, false, g.ptr(), g.dtype, g.rows, g.cols, g.cols, 1.0f);
         }
     });
@@ -331,14 +408,18 @@ Var linear_add(const Var& x, const Var& W, const Var& r) {
             gemm(self->grad, false, shadow_of(W), true, dx.ptr(), dx.dtype, dx.rows, dx.cols, dx.cols, 0.0f);
             x->accumulate_owned(std::move(dx));
         }
+        bool held = false;  // a held-back product still reads this node's gradient
         if (W->requires_grad) {
-            Tensor& g = W->ensure_grad();
-            gemm(x->data, true, self->grad, false, g.ptr(), g.dtype, g.rows, g.cols, g.cols, 1.0f);
+            held = defer_weight_gradient(x->data, self->grad, 0, W->data.cols, W);
+            if (!held) {
+                Tensor& g = W->ensure_grad();
+                gemm(x->data, true, self->grad, false, g.ptr(), g.dtype, g.rows, g.cols, g.cols, 1.0f);
+            }
         }
         if (r->requires_grad) {
             const bool was_shared = self->grad_shared;  // the products above have read it; r takes the tensor itself
             self->grad_shared = false;
-            r->accumulate_owned(std::move(self->grad), was_shared);
+            r->accumulate_owned(std::move(self->grad), was_shared || held);
         }
     });
 }
@@ -367,6 +448,17 @@ Var linear_cat(const Var& x, const std::vector<Var>& Ws) {
         }
         bool any = false;
         for (const Var& W : Ws) any = any || W->requires_grad;
+        if (any) {  // held back, one product per weight, if every one of them can wait
+            bool all = true;
+            const int64_t d = Ws[0]->data.cols;
+            for (int k = 0; k < n; ++k)
+                all = all && (!Ws[k]->requires_grad || weight_gradient_can_wait(x->data, self->grad, k * d, d, Ws[k]));
+            if (all) {
+                for (int k = 0; k < n; ++k)
+                    if (Ws[k]->requires_grad) hold_weight_gradient(x->data, self->grad, k * d, d, Ws[k]);
+                any = false;
+            }
+        }
         if (any) {  // dW_k += X^T dY[:, block k]
             float* dst[4] = {nullptr, nullptr, nullptr, nullptr};
             std::vector<Tensor> unused;

@@ -75,6 +75,19 @@ bool gemm_mfma_bf16_parts(const void* a, bool tA, int64_t lda, const void* b, bo
 // by tile, twice, and never stored. gemm_head_rows: per row the maximum, 1 / sum exp(z - maximum) and the loss
 // (stats: scratch of gemm_head_spans(N) * M float pairs, zt: of M floats); gemm_head_dlogits: bf16 dlogits.
 // Both return false, having done nothing, for operands the kernel does not take.
+// Several weight-gradient products C_p += A_p^T B_p (A_p [K, M_p], B_p [K, N_p] bf16; C_p [M_p, N_p] fp32) that share
+// the contraction length, as one launch of the hand-written kernel. False, with nothing done, where that does not
+// apply (operands it does not take, too few tiles): the caller multiplies them one by one.
+struct GroupedProduct {
+    const void* a;
+    int64_t lda;
+    const void* b;
+    int64_t ldb;
+    float* c;
+    int64_t ldc;
+    int64_t M, N;
+};
+bool gemm_mfma_grouped_tn(const GroupedProduct* ps, int count, int64_t K, hipStream_t st);
 int64_t gemm_head_spans(int64_t N);
 bool gemm_head_takes(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K);
 bool gemm_head_rows(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K, const int* target,
@@ -82,8 +95,8 @@ bool gemm_head_rows(const void* a, int64_t lda, const void* b, int64_t ldb, int6
 bool gemm_head_dlogits(const void* a, int64_t lda, const void* b, int64_t ldb, int64_t M, int64_t N, int64_t K,
                        const int* target, const float* row_max, const float* row_inv, float gscale, void* dl, int64_t ldc,
                        hipStream_t st);
-// Which GEMM serves bf16 operands: 1 (default) and 2 = the hand-written kernel for everything it takes,
-// 0 = the library only. Set from the environment
+// Which GEMM serves bf16 operands: 1 (default) and 2 = the hand-written kernel for everything it takes (1 also
+// groups a backward pass's weight-gradient products into shared launches), 0 = the library only. Set from the environment
 // (PK_GEMM=library) or by a caller that wants to compare them.
 void set_gemm_backend(int hand_written);
 void gemm_mfma_force_tiles(int which);  // -1: by shape (default); 0, 1, 5 .. 11: one kernel form always (measurement)

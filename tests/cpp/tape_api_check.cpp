@@ -345,6 +345,57 @@ void head_case() {
     pk::set_compute_dtype(PK_F32);
 }
 
+// Weight gradients of several Linears over 2048 tokens: in the default setting the backward pass holds the X^T dY
+// products back and multiplies them as one grouped launch; pk_set_gemm_backend(2) multiplies them one by one. Output
+// widths that are not multiples of the 128-wide tile, two different inputs (row pitches 512 and 136, the second
+// with a ragged last row tile), one pair sharing a concatenated product.
+void grouped_weight_gradient_case() {
+    std::printf("weight gradients held back and multiplied as one grouped launch vs one by one\n");
+    const int T = 2048, d = 512;
+    const int widths[6] = {1376, 520, 520, 136, 512, 512};  // Wa, {Wb | Wc}, W0 (feeds Wf), We, Wf [136, 512]
+    const auto hx = draw(static_cast<size_t>(T) * d, 71, 1.0);
+    std::vector<std::vector<float>> hw;
+    for (int k = 0; k < 5; ++k) hw.push_back(draw(static_cast<size_t>(d) * widths[k], 72 + k, 0.05));
+    hw.push_back(draw(static_cast<size_t>(136) * 512, 78, 0.05));
+    std::vector<int> target(T);
+    for (int i = 0; i < T; ++i) target[i] = (5 * i + 2) % 136;
+    auto tg = device_ints(target);
+    pk::set_compute_dtype(PK_BF16);
+    auto run = [&](int backend) {
+        const int before = pk_set_gemm_backend(backend);
+        pk::Var x = pk::make_var(pk::upload(hx.data(), T, d, PK_BF16), true);
+        std::vector<pk::Var> W;
+        for (int k = 0; k < 5; ++k) W.push_back(pk::make_var(pk::upload(hw[k].data(), d, widths[k]), true));
+        W.push_back(pk::make_var(pk::upload(hw[5].data(), 136, 512), true));
+        for (auto& w : W) w->is_param = true;
+        pk::Var ya = pk::ops::linear(x, W[0]);
+        pk::Var ybc = pk::ops::linear_cat(x, {W[1], W[2]});
+        pk::Var y0 = pk::ops::linear(x, W[3]);
+        pk::Var ye = pk::ops::linear(x, W[4]);
+        pk::Var yf = pk::ops::linear_add(y0, W[5], ye);
+        pk::Var loss = pk::ops::add(pk::ops::add(pk::ops::cross_entropy(ya, tg), pk::ops::cross_entropy(ybc, tg)),
+                                    pk::ops::cross_entropy(yf, tg));
+        pk::backward(loss);
+        std::vector<std::vector<float>> g;
+        for (auto& w : W) g.push_back(host(w->grad));
+        pk::invalidate_shadows();
+        pk_set_gemm_backend(before);
+        return g;
+    };
+    const auto one = run(2), grouped = run(1);
+    const char* names[6] = {"dW [512, 1376]", "dW [512, 520] (first of a pair)", "dW [512, 520] (second of a pair)", "dW [512, 136]",
+                            "dW [512, 512]", "dW [136, 512]"};
+    for (int k = 0; k < 6; ++k) {
+        double w = 0.0, size = 0.0;
+        for (size_t i = 0; i < one[k].size(); ++i) {
+            w = std::fmax(w, std::fabs(static_cast<double>(one[k][i]) - grouped[k][i]));
+            size = std::fmax(size, std::fabs(static_cast<double>(one[k][i])));
+        }
+        check(size > 0.0 && w <= 1e-4 * size, names[k], w / std::fmax(size, 1e-30));
+    }
+    pk::set_compute_dtype(PK_F32);
+}
+
 void behaviour_case() {
     std::printf("tape behaviour and errors\n");
     const auto h = draw(8 * 4, 31, 1.0);
@@ -404,6 +455,7 @@ int main() {
     linear_add_case(PK_BF16, "bfloat16, edge tiles", 200, 72, 136, 1.0 / 128);
     linear_add_case(PK_BF16, "bfloat16, long contraction", 300, 1376, 64, 1.0 / 128);
     head_case();
+    grouped_weight_gradient_case();
     behaviour_case();
     if (g_failures == 0) {
         std::printf("tape_api_check PASSED\n");
