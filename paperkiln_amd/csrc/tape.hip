@@ -144,7 +144,11 @@ bool weight_gradient_can_wait(const Tensor& x, const Tensor& dy, int64_t col0, i
 }
 void hold_weight_gradient(const Tensor& x, const Tensor& dy, int64_t col0, int64_t ncols, const Var& W) {
     auto& pd = pending();
-    if (pd.jobs.size() == 8) flush_weight_gradients();
+    // a weight that is used twice must not meet itself in one launch: its two products would add into the same
+    // gradient tiles at the same time
+    bool again = false;
+    for (const auto& job : pd.jobs) again = again || job.W.get() == W.get();
+    if (again || pd.jobs.size() == 8) flush_weight_gradients();
     pd.jobs.push_back(TapeContext::Pending::Job{x, dy, col0, ncols, W});
 }
 bool defer_weight_gradient(const Tensor& x, const Tensor& dy, int64_t col0, int64_t ncols, const Var& W) {

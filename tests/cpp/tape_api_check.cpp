@@ -348,7 +348,8 @@ void head_case() {
 // Weight gradients of several Linears over 2048 tokens: in the default setting the backward pass holds the X^T dY
 // products back and multiplies them as one grouped launch; pk_set_gemm_backend(2) multiplies them one by one. Output
 // widths that are not multiples of the 128-wide tile, two different inputs (row pitches 512 and 136, the second
-// with a ragged last row tile), one pair sharing a concatenated product.
+// with a ragged last row tile), one pair sharing a concatenated product, one weight used by two Linears (whose two
+// products must not run in one launch: they add into the same gradient).
 void grouped_weight_gradient_case() {
     std::printf("weight gradients held back and multiplied as one grouped launch vs one by one\n");
     const int T = 2048, d = 512;
@@ -371,7 +372,7 @@ void grouped_weight_gradient_case() {
         pk::Var ya = pk::ops::linear(x, W[0]);
         pk::Var ybc = pk::ops::linear_cat(x, {W[1], W[2]});
         pk::Var y0 = pk::ops::linear(x, W[3]);
-        pk::Var ye = pk::ops::linear(x, W[4]);
+        pk::Var ye = pk::ops::linear(pk::ops::linear(x, W[4]), W[4]);  // one weight used twice
         pk::Var yf = pk::ops::linear_add(y0, W[5], ye);
         pk::Var loss = pk::ops::add(pk::ops::add(pk::ops::cross_entropy(ya, tg), pk::ops::cross_entropy(ybc, tg)),
                                     pk::ops::cross_entropy(yf, tg));
