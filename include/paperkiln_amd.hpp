@@ -195,6 +195,8 @@ void zero_grad(const std::vector<Var>& vars);   // autograd.cpp:104-108
 // copy of x and pushes the output gradient through the fresh subgraph
 // (autograd.cpp:68-102). fn must be recomputation-deterministic.
 Var checkpoint(const std::function<Var(const Var&)>& fn, const Var& x);
+// True while checkpoint() re-runs a segment at backward time: the segment's own result is not needed then, only its tape.
+bool recomputing();
 
 bool grad_enabled();
 class NoGrad {
@@ -217,7 +219,9 @@ namespace ops {
 // (ops::matmul + nn::Linear::forward, ops.cpp:33-58, nn.cpp:106-109).
 Var linear(const Var& x, const Var& W);
 // r + x W: a Linear whose output joins the residual stream (llama.cpp:47, 59), the add done in the product's epilogue
-Var linear_add(const Var& x, const Var& W, const Var& r);
+// result_needed = false (only under grad): the node is recorded but its value is not computed -- for the last op of a
+// checkpointed segment while it is re-run at backward time (recomputing()), whose value nobody reads.
+Var linear_add(const Var& x, const Var& W, const Var& r, bool result_needed = true);
 // Three projections of the same input written side by side into one [N, 3*out]
 // matrix: the concat_cols({q, k, v}) of llama.cpp:30-36 without the copies.
 Var linear3(const Var& x, const Var& Wq, const Var& Wk, const Var& Wv);

@@ -179,7 +179,9 @@ struct Model {
         const float sc = 1.0f / std::sqrt(static_cast<float>(dk));
         Var x1 = ops::linear_add(ops::attention_qkv(qkv, cfg.n_heads, sc, seq_len, true, cfg.window, cfg.sinks), b.o, x);
         Var h2 = ops::rmsnorm(x1, b.ln2_w);
-        return ops::linear_add(ops::silu_mul_cat(ops::linear_cat(h2, {b.gate, b.up})), b.down, x1);
+        // re-run at backward time, the block's own output is not needed again (the gradient arrives from outside): the
+        // down projection is recorded but not multiplied
+        return ops::linear_add(ops::silu_mul_cat(ops::linear_cat(h2, {b.gate, b.up})), b.down, x1, !recomputing());
     }
 
     // Llama::forward (llama.cpp:71-89) up to the final norm; positions restart per sequence.

@@ -36,6 +36,7 @@ struct TapeContext::Pending {
 };
 
 namespace {
+thread_local bool g_recomputing = false;  // inside a checkpointed segment's re-run at backward time
 thread_local bool g_grad_enabled = true;
 thread_local TapeContext g_own_context;            // what a thread works on outside any ContextScope
 thread_local TapeContext* g_context = nullptr;
@@ -297,6 +298,7 @@ void Variable::accumulate_owned(Tensor&& g, bool shared) {
 }
 
 bool grad_enabled() { return g_grad_enabled; }
+bool recomputing() { return g_recomputing; }
 NoGrad::NoGrad() : prev_(g_grad_enabled) { g_grad_enabled = false; }
 NoGrad::~NoGrad() { g_grad_enabled = prev_; }
 
@@ -353,7 +355,16 @@ Var checkpoint(const std::function<Var(const Var&)>& fn, const Var& x) {
         // node's gradient -- nobody else reads it -- and run the rebuilt tape. Parameters used inside the
         // segment are the model's own Variables, so their gradients land where they belong.
         Var leaf = make_var(input->data, /*requires_grad=*/true);
-        Var rebuilt = segment(leaf);
+        const bool outer = g_recomputing;
+        g_recomputing = true;  // the segment may skip what only its own result needs (recomputing())
+        Var rebuilt;
+        try {
+            rebuilt = segment(leaf);
+        } catch (...) {
+            g_recomputing = outer;
+            throw;
+        }
+        g_recomputing = outer;
         if (rebuilt->data.rows != raw->grad.rows || rebuilt->data.cols != raw->grad.cols)
             shape_fail("checkpoint: recomputed output shape mismatch");
         rebuilt->accumulate_owned(std::move(raw->grad), raw->grad_shared);
@@ -390,14 +401,18 @@ Var linear(const Var& x, const Var& W) {
 // llama.cpp:47-59), the sum formed in the product's epilogue where the library's own GEMM takes the operands (one
 // rounding of r + x W instead of two, and no pass over y and r afterwards), by an add otherwise. One node with
 // the gradients of both ops: dr is the node's gradient itself.
-Var linear_add(const Var& x, const Var& W, const Var& r) {
+Var linear_add(const Var& x, const Var& W, const Var& r, bool result_needed) {
     if (x->data.cols != W->data.rows) shape_fail("matmul: inner dimensions disagree");
     if (r->data.rows != x->data.rows || r->data.cols != W->data.cols || r->data.dtype != x->data.dtype)
         shape_fail("add: shape mismatch");
     const Tensor& Wc = shadow_of(W);
     Tensor y = Tensor::make(x->data.rows, W->data.cols, x->data.dtype);
     const bool contiguous = r->data.off_bytes % 16 == 0;
-    if (!(x->data.dtype == PK_BF16 && Wc.dtype == PK_BF16 && gemm_backend() != 0 && contiguous &&
+    // result_needed = false: the caller only wants the node (the last op of a segment that is being re-run for its
+    // tape: the backward closure reads x, W and the node's gradient, never the node's value), so nothing is multiplied
+    if (!result_needed && grad_enabled()) {
+        // y stays as allocated: its shape is what the tape needs
+    } else if (!(x->data.dtype == PK_BF16 && Wc.dtype == PK_BF16 && gemm_backend() != 0 && contiguous &&
           gemm_mfma_bf16(x->data.ptr(), false, x->data.cols, Wc.ptr(), false, Wc.cols, y.ptr(), y.dtype, y.rows, y.cols,
                          x->data.cols, y.cols, 1.0f, tape_stream(), r->data.ptr()))) {
         gemm(x->data, false, Wc, false, y.ptr(), y.dtype, y.rows, y.cols, y.cols, 0.0f);
