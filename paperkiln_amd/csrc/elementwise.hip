@@ -888,13 +888,18 @@ __global__ void sum_f32_k(const float* x, int64_t n, double* out) {
     }
     if (threadIdx.x == 0) *out = sh[0];
 }
-// mean of n floats, accumulated in double in the order sum_f32_k uses, rounded to float once: what the host does
-// with k_sum_f32_to_host's result, without the round trip
-__global__ void mean_f32_k(const float* x, int64_t n, float* out) {
-    __shared__ double sh[NT];
+// mean of n floats, accumulated in double and rounded to float once: what the host does with
+// k_sum_f32_to_host's result, without the round trip
+__global__ __launch_bounds__(1024) void mean_f32_k(const float* x, int64_t n, float* out) {
+    // thread t takes the elements sum_f32_k's thread t % NT takes, a quarter of them: the NT partial sums are formed
+    // from four pieces each and then added in sum_f32_k's tree
+    __shared__ double sh[1024];
     double s = 0.0;
-    for (int64_t i = threadIdx.x; i < n; i += NT) s += static_cast<double>(x[i]);
+    const int t = threadIdx.x % NT, q = threadIdx.x / NT;
+    for (int64_t i = t + static_cast<int64_t>(q) * NT; i < n; i += 4 * NT) s += static_cast<double>(x[i]);
     sh[threadIdx.x] = s;
+    __syncthreads();
+    if (threadIdx.x < NT) sh[threadIdx.x] = (sh[threadIdx.x] + sh[threadIdx.x + NT]) + (sh[threadIdx.x + 2 * NT] + sh[threadIdx.x + 3 * NT]);
     __syncthreads();
     for (int o = NT / 2; o >= 1; o >>= 1) {
         if (threadIdx.x < o) sh[threadIdx.x] += sh[threadIdx.x + o];
@@ -1262,7 +1267,7 @@ bool k_ce_rows_once(const Tensor& logits, const int* targets, float gscale, floa
 }
 void k_mean_f32(const float* x, int64_t n, const Tensor& out) {
     if (out.dtype != PK_F32 || out.rows * out.cols != 1) throw std::runtime_error("mean: the result is one float");
-    hipLaunchKernelGGL(mean_f32_k, dim3(1), dim3(NT), 0, tape_stream(), x, n, static_cast<float*>(out.ptr()));
+    hipLaunchKernelGGL(mean_f32_k, dim3(1), dim3(1024), 0, tape_stream(), x, n, static_cast<float*>(out.ptr()));
     post();
 }
 double k_sum_f32_to_host(const float* x, int64_t n) {
