@@ -260,6 +260,30 @@ def test_chunked_tied_head_matches_the_materialised_head(case):
         m.close()
 
 
+def test_grouped_weight_gradients_match_one_by_one():
+    """A block's seven weight-gradient products X^T dY (nn.cpp / ops.cpp:52-55 per Linear) run as one grouped launch
+    in the default setting and one by one with set_gemm_backend(2): same bf16 operands, fp32 sums in another order,
+    so every gradient agrees to fp32 rounding -- plain and checkpointed (where the queue is emptied at the end of
+    each block's re-run)."""
+    cfg = dict(vocab=1000, d=512, n_layers=2, n_heads=8, d_ff=1376)
+    m = Llama(compute_dtype="bf16", seed=5, **cfg)
+    toks = synth.randint(17, 2048 + 1, cfg["vocab"])
+    x, y = toks[:-1], toks[1:]
+    before = blockops.set_gemm_backend(2)
+    try:
+        loss_one, _ = m.loss_backward(x, y, 1024, checkpoint=False)
+        g_one = m.grads()
+        for ck in (False, True):
+            blockops.set_gemm_backend(1)
+            loss_grouped, _ = m.loss_backward(x, y, 1024, checkpoint=ck)
+            g_grouped = m.grads()
+            assert loss_grouped == loss_one
+            assert reldiff(g_grouped, g_one) < 1e-5, (ck, reldiff(g_grouped, g_one))
+    finally:
+        blockops.set_gemm_backend(before)
+        m.close()
+
+
 def test_config5_full_size_checkpointing_bars():
     """BASELINE config 5 at full size (6 layers, d 512, 8 heads of 64, d_ff 1376, vocab 32000 tied, B=8 x T=1024,
     bf16 compute over fp32 master weights): the checkpointed step's loss equals the plain step's within 1e-4 and
