@@ -345,14 +345,14 @@ void head_case() {
     pk::set_compute_dtype(PK_F32);
 }
 
-// Weight gradients of several Linears over 2048 tokens: in the default setting the backward pass holds the X^T dY
+// Weight gradients of several Linears over 2056 tokens: in the default setting the backward pass holds the X^T dY
 // products back and multiplies them as one grouped launch; pk_set_gemm_backend(2) multiplies them one by one. Output
 // widths that are not multiples of the 128-wide tile, two different inputs (row pitches 512 and 136, the second
 // with a ragged last row tile), one pair sharing a concatenated product, one weight used by two Linears (whose two
 // products must not run in one launch: they add into the same gradient).
 void grouped_weight_gradient_case() {
     std::printf("weight gradients held back and multiplied as one grouped launch vs one by one\n");
-    const int T = 2048, d = 512;
+    const int T = 2056, d = 512;  // not a multiple of the kernel's 64-deep slices: the last slice is 8 tokens
     const int widths[6] = {1376, 520, 520, 136, 512, 512};  // Wa, {Wb | Wc}, W0 (feeds Wf), We, Wf [136, 512]
     const auto hx = draw(static_cast<size_t>(T) * d, 71, 1.0);
     std::vector<std::vector<float>> hw;
