@@ -266,6 +266,9 @@ double clip_grad_norm(const std::vector<Var>& params, float max_norm);  // ops.c
 void set_compute_dtype(int dtype);
 int compute_dtype();
 void invalidate_shadows();
+// The same effect for a caller whose parameters outlive the copies (a model that owns both): every copy is
+// re-cast from its parameter where it lies, all of them in one launch.
+void refresh_shadows();
 // Builds the compute-dtype copy of a parameter (or of the side-by-side concatenation linear_cat multiplies by) now
 // instead of at its first use, so that a caller measuring activation memory can have them allocated beforehand.
 void prepare_shadow(const Var& W);

@@ -683,6 +683,27 @@ __global__ void cast_cols_k(const TA* src, TY* dst, int64_t rows, int64_t cols, 
         stf(dst, (i / cols) * ld + off + i % cols, ldf(src, i));
 }
 
+// Many casts of fp32 matrices into column blocks of bf16 matrices as one launch (the refresh of every compute-dtype
+// weight copy after an optimizer step): job j covers blocks [block_begin[j], block_begin[j + 1]), eight elements a thread.
+struct CastJobs {
+    static constexpr int MAX = 64;
+    int count;
+    int block_begin[MAX + 1];
+    const float* src[MAX];
+    uint16_t* dst[MAX];
+    int rows[MAX], cols[MAX], ld[MAX], off[MAX];
+};
+__global__ void cast_jobs_k(CastJobs jobs) {
+    int j = 0;
+    while (static_cast<int>(blockIdx.x) >= jobs.block_begin[j + 1]) ++j;
+    const int cols = jobs.cols[j];
+    const int64_t n8 = static_cast<int64_t>(jobs.rows[j]) * cols / 8;  // cols, ld and off are multiples of 8
+    const int64_t i = (static_cast<int64_t>(blockIdx.x) - jobs.block_begin[j]) * NT + threadIdx.x;
+    if (i >= n8) return;
+    const int64_t e = i * 8, r = e / cols, c = e - r * cols;
+    st8(jobs.dst[j], r * jobs.ld[j] + jobs.off[j] + c, ld8(jobs.src[j], e));
+}
+
 // apply_rope (ops.cpp:497-509 forward, :519-533 backward = rotation by -theta).
 // The inverse frequencies come from the host, computed with the reference's own expression
 // 1 / pow(theta, dim / head_dim): the angle pos * inv_freq is then the same fp32 number the
@@ -981,6 +1002,38 @@ void k_cast_cols(const Tensor& src, const Tensor& dst, int64_t col_off) {
                                     static_cast<const TA*>(src.ptr()), static_cast<TY*>(dst.ptr()), src.rows, src.cols,
                                     dst.cols, col_off)));
     post();
+}
+// dst_k[:, off_k : off_k + cols_k] = bf16(src_k) for every job, one launch per 64 jobs. False, with nothing done,
+// if a job is not an fp32 -> bf16 cast with column counts and offsets that are multiples of 8 (the caller casts one by one).
+bool k_cast_many(const std::vector<CastJob>& list) {
+    for (const CastJob& c : list)
+        if (c.src.dtype != PK_F32 || c.dst.dtype != PK_BF16 || c.src.cols % 8 || c.dst.cols % 8 || c.col_off % 8 ||
+            c.src.rows != c.dst.rows || c.col_off < 0 || c.col_off + c.src.cols > c.dst.cols ||
+            c.src.numel() / 8 > (int64_t{1} << 30) || !aligned16p(c.src.ptr()) || !aligned16p(c.dst.ptr()))
+            return false;
+    size_t done = 0;
+    while (done < list.size()) {
+        CastJobs jobs{};
+        int blocks = 0;
+        while (done < list.size() && jobs.count < CastJobs::MAX) {
+            const CastJob& c = list[done++];
+            const int k = jobs.count++;
+            jobs.block_begin[k] = blocks;
+            jobs.src[k] = static_cast<const float*>(c.src.ptr());
+            jobs.dst[k] = static_cast<uint16_t*>(c.dst.ptr());
+            jobs.rows[k] = static_cast<int>(c.src.rows);
+            jobs.cols[k] = static_cast<int>(c.src.cols);
+            jobs.ld[k] = static_cast<int>(c.dst.cols);
+            jobs.off[k] = static_cast<int>(c.col_off);
+            blocks += static_cast<int>((c.src.numel() / 8 + NT - 1) / NT);
+        }
+        for (int k = jobs.count; k <= CastJobs::MAX; ++k) jobs.block_begin[k] = blocks;
+        if (blocks > 0) {
+            hipLaunchKernelGGL(cast_jobs_k, dim3(static_cast<unsigned>(blocks)), dim3(NT), 0, tape_stream(), jobs);
+            post();
+        }
+    }
+    return true;
 }
 template <int OP>
 static void binary(const Tensor& a, const Tensor& b, const Tensor& y, const char* who) {

@@ -409,7 +409,7 @@ int pk_llama_adamw_step(void* h, float lr, float b1, float b2, float eps, float 
         // every parameter of this model receives a gradient each step, so the reference's "skip a
         // parameter that never accumulated" (nn.cpp:309) never applies; padding stays at zero
         k_adamw(m->pslab, m->gslab, m->mslab, m->vslab, lr, b1, b2, eps, wd, c1, c2, clip);
-        invalidate_shadows();
+        refresh_shadows();  // the bf16 copies of the weights follow them, in one launch
         hip_check(hipStreamSynchronize(tape_stream()), "hipStreamSynchronize");
     });
 }

@@ -16,8 +16,12 @@ size_t live_variables() { return detail::g_live_vars.load(); }
 
 // compute-dtype copies of a context's fp32 parameters, valid until the next optimizer step
 struct TapeContext::Shadows {
+    struct Cat {
+        Tensor t;
+        std::vector<const Variable*> ws;
+    };
     std::unordered_map<const Variable*, Tensor> single;  // one weight
-    std::unordered_map<const Variable*, Tensor> cat;     // [W_0 | W_1 | ...], keyed by the first weight
+    std::unordered_map<const Variable*, Cat> cat;        // [W_0 | W_1 | ...], keyed by the first weight
 };
 
 // Weight-gradient products dW += X^T dY that the Linear closures of a running backward pass have handed in instead
@@ -66,10 +70,14 @@ const Tensor& shadow_cat(const std::vector<Var>& Ws) {
     if (it == map.end()) {
         const int64_t d = Ws[0]->data.cols;
         Tensor t = Tensor::make(Ws[0]->data.rows, d * static_cast<int64_t>(Ws.size()), tape_context().compute);
-        for (size_t k = 0; k < Ws.size(); ++k) k_cast_cols(Ws[k]->data, t, static_cast<int64_t>(k) * d);
-        it = map.emplace(Ws[0].get(), std::move(t)).first;
+        std::vector<const Variable*> ws;
+        for (size_t k = 0; k < Ws.size(); ++k) {
+            k_cast_cols(Ws[k]->data, t, static_cast<int64_t>(k) * d);
+            ws.push_back(Ws[k].get());
+        }
+        it = map.emplace(Ws[0].get(), TapeContext::Shadows::Cat{std::move(t), std::move(ws)}).first;
     }
-    return it->second;
+    return it->second.t;
 }
 
 // The order the backward closures run in: the root first, every other node once all the nodes that consume it
@@ -243,6 +251,24 @@ void set_compute_dtype(int dtype) {
 }
 int compute_dtype() { return tape_context().compute; }
 void invalidate_shadows() { tape_context().shadows.reset(); }
+// The copies are brought up to date where they lie instead of being dropped and rebuilt at their next use: one
+// launch for all of them (a model's dozens of weights would otherwise each be a cast kernel of a few microseconds
+// after every optimizer step). The parameters they were made from must still be alive.
+void refresh_shadows() {
+    TapeContext& c = tape_context();
+    if (!c.shadows) return;
+    std::vector<CastJob> jobs;
+    for (auto& kv : c.shadows->single) jobs.push_back(CastJob{kv.first->data, kv.second, 0});
+    for (auto& kv : c.shadows->cat) {
+        int64_t off = 0;
+        for (const Variable* w : kv.second.ws) {
+            jobs.push_back(CastJob{w->data, kv.second.t, off});
+            off += w->data.cols;
+        }
+    }
+    if (jobs.empty()) return;
+    if (!k_cast_many(jobs)) c.shadows.reset();  // not casts the batched kernel takes: rebuilt at their next use
+}
 void prepare_shadow(const Var& W) { (void)shadow_of(W); }
 void prepare_shadow_cat(const std::vector<Var>& Ws) { (void)shadow_cat(Ws); }
 

@@ -3,6 +3,7 @@
 // tape context) are public and live in include/paperkiln_amd.hpp.
 #pragma once
 #include <memory>
+#include <vector>
 #include <hip/hip_runtime.h>
 
 #include "paperkiln_amd.hpp"
@@ -15,7 +16,13 @@ void hip_check(hipError_t e, const char* what);  // throws Error(PK_ERR_HIP), as
 // All take row-major contiguous tensors; T = fp32 or bf16 storage, fp32 math.
 void k_fill(const Tensor& y, float v);
 void k_cast(const Tensor& src, const Tensor& dst);                      // dtype conversion / copy
-void k_cast_cols(const Tensor& src, const Tensor& dst, int64_t col_off);  // dst[:, off:off+src.cols] = src
+void k_cast_cols(const Tensor& src, const Tensor& dst, int64_t col_off);
+// many such casts (fp32 -> a column block of a bf16 matrix) as one launch; false = not applicable, nothing done
+struct CastJob {
+    Tensor src, dst;
+    int64_t col_off;
+};
+bool k_cast_many(const std::vector<CastJob>& list);  // dst[:, off:off+src.cols] = src
 void k_add(const Tensor& a, const Tensor& b, const Tensor& y);          // y = a + b      (ops.cpp:60-65)
 void k_mul(const Tensor& a, const Tensor& b, const Tensor& y);          // y = a .* b     (ops.cpp:76-83)
 void k_scale(const Tensor& a, float s, const Tensor& y);                // y = a * s
