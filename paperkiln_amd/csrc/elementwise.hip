@@ -757,6 +757,15 @@ __global__ void emb_fwd(const float* table, const int* ids, T* y, int64_t n, int
     for (int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x; i < n * d; i += static_cast<int64_t>(gridDim.x) * NT)
         stf(y, i, table[static_cast<int64_t>(ids[i / d]) * d + i % d]);
 }
+// the same gather, eight columns a thread (d a multiple of 8, bf16 rows 16-byte aligned)
+__global__ void emb_fwd8(const float* table, const int* ids, uint16_t* y, int64_t n, int d) {
+    const int d8 = d / 8;
+    const int64_t i = blockIdx.x * static_cast<int64_t>(NT) + threadIdx.x;
+    if (i >= n * d8) return;
+    const int64_t r = i / d8;
+    const int c = static_cast<int>(i - r * d8) * 8;
+    st8(y, r * d + c, ld8(table, static_cast<int64_t>(ids[r]) * d + c));
+}
 // Scatter-add without atomics. The rows are visited in the order of a stable sort by id (sorted_id, row_of), so
 // the rows that share an id are neighbours, in ascending row order. The block at the head of such a run adds the
 // run's rows one after another and is the only writer of that table row; every other block leaves at once. The
@@ -1271,6 +1280,14 @@ void k_rope_inplace(const Tensor& x, const int* pos, float theta, int d, int hea
     post();
 }
 void k_embedding_fwd(const Tensor& table, const int* ids, const Tensor& y) {
+    if (y.dtype == PK_BF16 && y.cols % 8 == 0 && aligned16p(y.ptr()) && aligned16p(table.ptr())) {
+        const int64_t n8 = y.numel() / 8;
+        hipLaunchKernelGGL(emb_fwd8, dim3(static_cast<unsigned>((n8 + NT - 1) / NT)), dim3(NT), 0, tape_stream(),
+                           static_cast<const float*>(table.ptr()), ids, static_cast<uint16_t*>(y.ptr()), y.rows,
+                           static_cast<int>(y.cols));
+        post();
+        return;
+    }
     PK_DISPATCH1(T, y.dtype, hipLaunchKernelGGL((emb_fwd<T>), ew_grid(y.numel()), dim3(NT), 0, tape_stream(),
                                                 static_cast<const float*>(table.ptr()), ids, static_cast<T*>(y.ptr()),
                                                 y.rows, static_cast<int>(y.cols)));
